@@ -1,0 +1,149 @@
+// Shared device helpers for the gfx950 kernels of libbitween_hip.so.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/bitween_hip.h"
+
+typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+typedef float f4 __attribute__((ext_vector_type(4)));
+typedef unsigned int u4 __attribute__((ext_vector_type(4)));
+typedef unsigned int u2 __attribute__((ext_vector_type(2)));
+
+#define BW_DEV __device__ __forceinline__
+
+BW_DEV h2 as_h2(uint32_t u) { return __builtin_bit_cast(h2, u); }
+BW_DEV uint32_t as_u32(h2 v) { return __builtin_bit_cast(uint32_t, v); }
+BW_DEV h2 splat(_Float16 v) { return h2{v, v}; }
+
+// ---- bfloat16 <-> float32 (round to nearest even; NaN kept quiet) -----------
+BW_DEV float bf16_to_f32(uint16_t b) { return __builtin_bit_cast(float, (uint32_t)b << 16); }
+BW_DEV uint16_t f32_to_bf16(float f) {
+    uint32_t u = __builtin_bit_cast(uint32_t, f);
+    if ((u & 0x7FFFFFFFu) > 0x7F800000u) return (uint16_t)((u >> 16) | 0x40u);
+    return (uint16_t)((u + 0x7FFFu + ((u >> 16) & 1u)) >> 16);
+}
+
+// ---- in-register dequantisation to float16 pairs -----------------------------
+// All routines produce W16 = fp16(s * (q - z)) with ONE rounding, which is
+// bit-for-bit what the reference's dequantize kernel stores
+// (bitween/modules.py:55-58): q - z is formed exactly in float16 from the
+// magic-number encoding 0x6400 | q = 1024 + q, then multiplied by s.
+// Requires z to be an integer in [0, 2^bits).
+//
+// Per-group constants a lane keeps while it walks the words of that group.
+template <int BITS> struct GroupConst;
+
+template <> struct GroupConst<4> {
+    h2 s, z0, z1;   // s, -(1024+z), -(64+z)
+    BW_DEV void set(_Float16 sv, _Float16 zv) {
+        s = splat(sv);
+        z0 = splat((_Float16)(-1024.0f) - zv);
+        z1 = splat((_Float16)(-64.0f) - zv);
+    }
+};
+template <> struct GroupConst<8> {
+    h2 s, z0;
+    BW_DEV void set(_Float16 sv, _Float16 zv) {
+        s = splat(sv);
+        z0 = splat((_Float16)(-1024.0f) - zv);
+    }
+};
+template <> struct GroupConst<2> {
+    h2 s, z0, z1, z2, z3, z4;   // -(1024+z), -(256+z), -(64+z), -(16+z), -(4+z)
+    BW_DEV void set(_Float16 sv, _Float16 zv) {
+        s = splat(sv);
+        z0 = splat((_Float16)(-1024.0f) - zv);
+        z1 = splat((_Float16)(-256.0f) - zv);
+        z2 = splat((_Float16)(-64.0f) - zv);
+        z3 = splat((_Float16)(-16.0f) - zv);
+        z4 = splat((_Float16)(-4.0f) - zv);
+    }
+};
+
+constexpr uint32_t kMagic = 0x64006400u;   // two float16 1024.0
+
+// One 4-bit word (nibbles n0..n7) -> 4 pairs in slot order (n0,n4)(n1,n5)(n2,n6)(n3,n7).
+BW_DEV void dequant_word4(uint32_t w, const GroupConst<4>& c, h2 out[4]) {
+    const h2 k16 = splat((_Float16)0.0625f);
+    const uint32_t w8 = w >> 8;
+    h2 a = as_h2((w & 0x000F000Fu) | kMagic);     // 1024 + n
+    h2 b = as_h2((w & 0x00F000F0u) | kMagic);     // 1024 + 16 n
+    h2 d = as_h2((w8 & 0x000F000Fu) | kMagic);
+    h2 e = as_h2((w8 & 0x00F000F0u) | kMagic);
+    out[0] = (a + c.z0) * c.s;
+    out[1] = __builtin_elementwise_fma(b, k16, c.z1) * c.s;
+    out[2] = (d + c.z0) * c.s;
+    out[3] = __builtin_elementwise_fma(e, k16, c.z1) * c.s;
+}
+
+// One 8-bit word (bytes b0..b3) -> 2 pairs in natural order (b0,b1)(b2,b3).
+BW_DEV void dequant_word8(uint32_t w, const GroupConst<8>& c, h2 out[2]) {
+    h2 a = as_h2(__builtin_amdgcn_perm(0x64646464u, w, 0x04010400u));
+    h2 b = as_h2(__builtin_amdgcn_perm(0x64646464u, w, 0x04030402u));
+    out[0] = (a + c.z0) * c.s;
+    out[1] = (b + c.z0) * c.s;
+}
+
+// One 2-bit word (crumbs c0..c15) -> 8 pairs (c_i, c_{i+8}), i = 0..7.
+BW_DEV void dequant_word2(uint32_t w, const GroupConst<2>& c, h2 out[8]) {
+    const uint32_t w10 = w >> 10;
+    h2 t0 = as_h2((w & 0x00030003u) | kMagic);     // 1024 + c
+    h2 t1 = as_h2((w & 0x000C000Cu) | kMagic);     // 1024 + 4c
+    h2 t2 = as_h2((w & 0x00300030u) | kMagic);     // 1024 + 16c
+    h2 t3 = as_h2((w & 0x00C000C0u) | kMagic);     // 1024 + 64c
+    h2 t4 = as_h2((w & 0x03000300u) | kMagic);     // 1024 + 256c
+    h2 t5 = as_h2((w10 & 0x00030003u) | kMagic);
+    h2 t6 = as_h2((w10 & 0x000C000Cu) | kMagic);
+    h2 t7 = as_h2((w10 & 0x00300030u) | kMagic);
+    const h2 k4 = splat((_Float16)0.25f), k16 = splat((_Float16)0.0625f), k64 = splat((_Float16)0.015625f),
+             k256 = splat((_Float16)0.00390625f);
+    out[0] = (t0 + c.z0) * c.s;
+    out[1] = __builtin_elementwise_fma(t1, k4, c.z1) * c.s;
+    out[2] = __builtin_elementwise_fma(t2, k16, c.z2) * c.s;
+    out[3] = __builtin_elementwise_fma(t3, k64, c.z3) * c.s;
+    out[4] = __builtin_elementwise_fma(t4, k256, c.z4) * c.s;
+    out[5] = (t5 + c.z0) * c.s;
+    out[6] = __builtin_elementwise_fma(t6, k4, c.z1) * c.s;
+    out[7] = __builtin_elementwise_fma(t7, k16, c.z2) * c.s;
+}
+
+// Position p of a block of VPI consecutive k holds original element perm(p):
+// the order in which the routines above emit the values of one word.
+template <int BITS> BW_DEV constexpr int slot_to_k(int p);
+template <> BW_DEV constexpr int slot_to_k<8>(int p) { return p; }
+template <> BW_DEV constexpr int slot_to_k<4>(int p) { return (p >> 1) + ((p & 1) << 2); }
+template <> BW_DEV constexpr int slot_to_k<2>(int p) { return (p >> 1) + ((p & 1) << 3); }
+
+// Dequantise the 16 bytes a lane loaded (4 words = 128/BITS values) into
+// 128/BITS/2 float16 pairs, MFMA-operand ready: pairs [4t, 4t+4) feed MFMA t.
+// NG = number of quantisation groups those 16 bytes span (1 or 2).
+template <int BITS, int NG>
+BW_DEV void dequant_lane16(const u4& w, const GroupConst<BITS>* gc, h2* out) {
+    if constexpr (BITS == 4) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) dequant_word4(w[i], gc[NG == 1 ? 0 : i / (4 / NG)], out + 4 * i);
+    } else if constexpr (BITS == 8) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) dequant_word8(w[i], gc[NG == 1 ? 0 : i / (4 / NG)], out + 2 * i);
+    } else {
+#pragma unroll
+        for (int i = 0; i < 4; i++) dequant_word2(w[i], gc[NG == 1 ? 0 : i / (4 / NG)], out + 8 * i);
+    }
+}
+
+BW_DEV h8 pack_h8(const h2* p) {
+    h8 r;
+    r[0] = p[0][0]; r[1] = p[0][1]; r[2] = p[1][0]; r[3] = p[1][1];
+    r[4] = p[2][0]; r[5] = p[2][1]; r[6] = p[3][0]; r[7] = p[3][1];
+    return r;
+}
+
+// Host-side argument checks shared by the entry points.
+static inline bool bw_bits_ok(int bits) { return bits == 2 || bits == 4 || bits == 8; }
+static inline bool bw_shape_ok(int64_t N, int64_t K, int bits, int group) {
+    return N > 0 && K > 0 && group > 0 && bw_bits_ok(bits) && K % group == 0 && K % (32 / bits) == 0 &&
+           N < (int64_t)1 << 31 && K < (int64_t)1 << 31;
+}
+static inline bool bw_aligned(const void* p, size_t a) { return ((uintptr_t)p & (a - 1)) == 0; }

@@ -1,0 +1,63 @@
+"""quantize_rtn / dequantize_rtn with the reference's signatures
+(bitween/functional.py:4,48), executed by the HIP kernels of
+libbitween_hip.so.  Tensors that live on the CPU are staged through the GPU
+and the results returned on the input's device; without a GPU these
+functions raise (there is no CPU implementation in this package).
+"""
+import torch
+
+from .kernels import hip_loader as _hip
+
+
+def _gpu_for(t):
+    if t.is_cuda:
+        return t.device
+    if not torch.cuda.is_available():
+        raise _hip.BitweenHipError("bitween_amd needs a ROCm GPU: there is no CPU implementation of this operator")
+    return torch.device("cuda", torch.cuda.current_device())
+
+
+@torch.no_grad()
+def quantize_rtn(weight: torch.Tensor, bits: int = 8, group_size: int = 32):
+    """Round-to-nearest asymmetric per-group quantisation and packing.
+
+    Returns (q_packed int32 [N, K*bits/32], scale [N, K/group_size] in
+    weight.dtype, zero_point int32 [N, K/group_size], group_size) - the tuple
+    of bitween/functional.py:45.  Arithmetic is carried out in weight.dtype,
+    as the reference's eager ops do.
+    """
+    assert bits in [2, 4, 8], "Only 2, 4, or 8-bit quantization supported."
+    if weight.dim() != 2:
+        raise ValueError("weight must be [out_features, in_features]")
+    out_features, in_features = weight.shape
+    pad = (group_size - in_features % group_size) % group_size
+    if pad > 0:
+        raise ValueError(f"Padding {pad} columns to {in_features} to make it a multiple of {group_size}")
+    if in_features % (32 // bits):
+        raise ValueError(f"in_features={in_features} does not fill whole int32 words at {bits} bits")
+    if weight.dtype not in (torch.float32, torch.float16, torch.bfloat16):
+        raise NotImplementedError(f"quantize_rtn: weight dtype {weight.dtype} is not supported")
+    dev = _gpu_for(weight)
+    w = weight.to(dev)
+    qweight, scale, zp = _hip.quantize_pack(w, bits, group_size, math_dtype=weight.dtype, scale_dtype=weight.dtype,
+                                            zp_dtype=torch.int32)
+    if not weight.is_cuda:
+        qweight, scale, zp = qweight.to(weight.device), scale.to(weight.device), zp.to(weight.device)
+    return qweight, scale, zp, group_size
+
+
+@torch.no_grad()
+def dequantize_rtn(q_packed: torch.Tensor, scale: torch.Tensor, zero_point: torch.Tensor, group_size: int,
+                   bits: int = 8):
+    """scale * (q - zero_point) as float32 [N, K] (bitween/functional.py:47-71)."""
+    assert bits in [2, 4, 8], "Only 2, 4, or 8-bit quantization supported."
+    dev = _gpu_for(q_packed)
+    s = scale.to(dev)
+    z = zero_point.to(dev)
+    if s.dtype == torch.bfloat16:
+        s = s.float()                       # exact widening; the product is float32 either way
+    if z.dtype not in (torch.int32, torch.float16):
+        z = z.to(torch.int32) if not z.is_floating_point() else z.float().to(torch.int32)
+    n = q_packed.shape[0]
+    out = _hip.dequantize(q_packed.to(dev), s.reshape(n, -1), z.reshape(n, -1), group_size, bits, torch.float32)
+    return out if q_packed.is_cuda else out.to(q_packed.device)

@@ -1,0 +1,153 @@
+"""ctypes binding of libbitween_hip.so (the C ABI in include/bitween_hip.h).
+
+This module takes the place of the reference's absent
+`bitween.kernels.cuda_loader` (main.py:401): `quantized_matmul_hip` has the
+signature and meaning of `quantized_matmul_cuda(x, qweight, scale, zero_point,
+bias, bits, group_size)` (main.py:433).
+
+There is no CPU path: a missing library or a missing GPU raises.
+"""
+import ctypes
+import os
+
+import torch
+
+_LIB_PATH = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "csrc", "libbitween_hip.so")
+_lib = None
+
+BW_F16, BW_BF16, BW_F32, BW_I32 = 0, 1, 2, 3
+_DTYPE_CODE = {torch.float16: BW_F16, torch.bfloat16: BW_BF16, torch.float32: BW_F32, torch.int32: BW_I32}
+
+ENTRY_POINTS = ("bw_abi_version", "bw_strerror", "bw_quantize_pack", "bw_dequantize", "bw_qgemv", "bw_qgemm",
+                "bw_qlinear")
+
+
+class BitweenHipError(RuntimeError):
+    pass
+
+
+def library_path():
+    return _LIB_PATH
+
+
+def load():
+    """Load the shared library once; raise if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(_LIB_PATH):
+        raise BitweenHipError(
+            f"{_LIB_PATH} is missing: build it with `python -m bitween_amd.csrc.build` "
+            "(bitween_amd has no CPU or eager fallback)")
+    lib = ctypes.CDLL(_LIB_PATH)
+    vp, i64, i32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int
+    lib.bw_abi_version.restype = i32
+    lib.bw_strerror.restype = ctypes.c_char_p
+    lib.bw_strerror.argtypes = [i32]
+    lib.bw_quantize_pack.argtypes = [vp, i32, i32, i64, i64, i64, i32, i32, vp, vp, i32, vp, i32, vp]
+    lib.bw_dequantize.argtypes = [vp, vp, i32, vp, i32, i64, i64, i32, i32, vp, i32, i64, vp]
+    mm = [vp, i32, i64, i64, i64, vp, vp, vp, vp, i64, i32, i32, vp, i64, vp]
+    for name in ("bw_qgemv", "bw_qgemm", "bw_qlinear"):
+        getattr(lib, name).argtypes = mm
+    for name in ("bw_quantize_pack", "bw_dequantize", "bw_qgemv", "bw_qgemm", "bw_qlinear"):
+        getattr(lib, name).restype = i32
+    _lib = lib
+    return lib
+
+
+def _check(status, what):
+    if status == 0:
+        return
+    msg = load().bw_strerror(status).decode()
+    if status == -2:
+        raise NotImplementedError(f"{what}: {msg}")
+    raise BitweenHipError(f"{what}: {msg} (status {status})")
+
+
+def require_gpu(t, what):
+    if not t.is_cuda:
+        raise BitweenHipError(f"{what}: expected a tensor on the ROCm GPU, got device {t.device} "
+                              "(bitween_amd has no CPU path)")
+
+
+def _stream(device):
+    return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+
+
+def quantize_pack(weight, bits, group_size, math_dtype, scale_dtype, zp_dtype):
+    """weight [N,K] on GPU (f16/bf16/f32) -> (qweight int32, scale, zero_point) per bw_quantize_pack."""
+    require_gpu(weight, "quantize_pack")
+    if weight.stride(-1) != 1:
+        weight = weight.contiguous()
+    n, k = weight.shape
+    vpi = 32 // bits
+    dev = weight.device
+    qweight = torch.empty((n, k // vpi), dtype=torch.int32, device=dev)
+    scale = torch.empty((n, k // group_size), dtype=scale_dtype, device=dev)
+    zp = torch.empty((n, k // group_size), dtype=zp_dtype, device=dev)
+    with torch.cuda.device(dev):
+        st = load().bw_quantize_pack(weight.data_ptr(), _DTYPE_CODE[weight.dtype], _DTYPE_CODE[math_dtype], n, k,
+                                     weight.stride(0), bits, group_size, qweight.data_ptr(), scale.data_ptr(),
+                                     _DTYPE_CODE[scale_dtype], zp.data_ptr(), _DTYPE_CODE[zp_dtype], _stream(dev))
+    _check(st, "bw_quantize_pack")
+    return qweight, scale, zp
+
+
+def dequantize(qweight, scale, zero_point, group_size, bits, out_dtype):
+    """(qweight, scale f32|f16, zero_point i32|f16) on GPU -> weight [N,K] of out_dtype per bw_dequantize."""
+    require_gpu(qweight, "dequantize")
+    qweight, scale, zero_point = qweight.contiguous(), scale.contiguous(), zero_point.contiguous()
+    n, words = qweight.shape
+    k = words * (32 // bits)
+    out = torch.empty((n, k), dtype=out_dtype, device=qweight.device)
+    with torch.cuda.device(qweight.device):
+        st = load().bw_dequantize(qweight.data_ptr(), scale.data_ptr(), _DTYPE_CODE[scale.dtype], zero_point.data_ptr(),
+                                  _DTYPE_CODE[zero_point.dtype], n, k, bits, group_size, out.data_ptr(),
+                                  _DTYPE_CODE[out_dtype], k, _stream(qweight.device))
+    _check(st, "bw_dequantize")
+    return out
+
+
+def _matmul(entry, x, qweight, scale, zero_point, bias, bits, group_size):
+    require_gpu(x, entry)
+    if x.dim() != 2:
+        raise ValueError("x must be [M, K]")
+    if qweight.dtype != torch.int32 or scale.dtype != torch.float16 or zero_point.dtype != torch.float16:
+        raise TypeError("qweight must be int32 and scale / zero_point float16 (the QuantizedLinear buffers)")
+    if x.dtype != torch.float16:
+        raise TypeError("x must be float16")
+    if bias is not None and bias.dtype != x.dtype:
+        raise TypeError("bias must have the dtype of x")
+    x = x if x.stride(-1) == 1 and (x.stride(0) * 2) % 16 == 0 and x.data_ptr() % 16 == 0 else x.contiguous().clone()
+    qweight, scale, zero_point = qweight.contiguous(), scale.contiguous(), zero_point.contiguous()
+    m, k = x.shape
+    n, words = qweight.shape
+    if words * (32 // bits) != k:
+        raise ValueError(f"x has K={k} but qweight packs K={words * (32 // bits)}")
+    if scale.shape != (n, k // group_size) or zero_point.shape != scale.shape:
+        raise ValueError("scale / zero_point must be [N, K // group_size]")
+    y = torch.empty((m, n), dtype=x.dtype, device=x.device)
+    if m == 0:
+        return y
+    with torch.cuda.device(x.device):
+        st = getattr(load(), entry)(x.data_ptr(), _DTYPE_CODE[x.dtype], m, k, x.stride(0), qweight.data_ptr(),
+                                    scale.data_ptr(), zero_point.data_ptr(),
+                                    None if bias is None else bias.contiguous().data_ptr(), n, bits, group_size,
+                                    y.data_ptr(), n, _stream(x.device))
+    _check(st, entry)
+    return y
+
+
+def quantized_matmul_hip(x, qweight, scale, zero_point, bias, bits, group_size):
+    """y[M,N] = x[M,K] @ dequant(qweight, scale, zero_point)^T + bias, float16 (main.py:433's operator)."""
+    return _matmul("bw_qlinear", x, qweight, scale, zero_point, bias, bits, group_size)
+
+
+def quantized_gemv_hip(x, qweight, scale, zero_point, bias, bits, group_size):
+    """Decode kernel only (M <= 16)."""
+    return _matmul("bw_qgemv", x, qweight, scale, zero_point, bias, bits, group_size)
+
+
+def quantized_gemm_hip(x, qweight, scale, zero_point, bias, bits, group_size):
+    """Prefill kernel only (any M)."""
+    return _matmul("bw_qgemm", x, qweight, scale, zero_point, bias, bits, group_size)

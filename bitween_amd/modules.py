@@ -1,0 +1,103 @@
+"""QuantizedLinear and its autograd function with the reference's interface
+(bitween/modules.py:60-217): same constructor, buffers (qweight int32,
+scale / zero_point / bias float16), from_float, forward and repr.  The
+forward is one fused dequantise+matmul HIP kernel instead of the reference's
+dequantise-to-HBM, BLAS matmul and bias add.
+"""
+import torch
+import torch.nn as nn
+
+from .kernels import hip_loader as _hip
+
+
+class QuantizedLinearFunction(torch.autograd.Function):
+    """apply(x, qweight, scale, zero_point, bias, bits, group_size) -> float16 [..., N]
+    (bitween/modules.py:62-106).  backward returns grad_input only
+    (bitween/modules.py:108-141)."""
+
+    @staticmethod
+    def forward(ctx, x, qweight, scale, zero_point, bias, bits, group_size):
+        ctx.save_for_backward(x, qweight, scale, zero_point, bias)
+        ctx.bits = bits
+        ctx.group_size = group_size
+        original_shape = x.shape
+        x2 = x.reshape(-1, original_shape[-1]).to(torch.float16)
+        n = qweight.shape[0]
+        y = _hip.quantized_matmul_hip(x2, qweight, scale, zero_point, bias, bits, group_size)
+        return y.reshape(*original_shape[:-1], n)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        x, qweight, scale, zero_point, bias = ctx.saved_tensors
+        grad_input = None
+        if ctx.needs_input_grad[0]:
+            # W = scale * (q - zp) in float32, cast to grad_output.dtype: the float32 product is exact,
+            # so dequantising straight to that dtype gives the same bits.
+            gdt = grad_output.dtype if grad_output.dtype in (torch.float16, torch.bfloat16, torch.float32) else torch.float32
+            weight = _hip.dequantize(qweight, scale, zero_point, ctx.group_size, ctx.bits, gdt)
+            grad_input = grad_output @ weight.to(grad_output.dtype)
+        return grad_input, None, None, None, None, None, None
+
+
+class QuantizedLinear(nn.Module):
+    """Linear layer holding 2/4/8-bit group-quantised weights."""
+
+    def __init__(self, in_features, out_features, bits=8, group_size=32, bias=True, dtype=torch.float16):
+        super().__init__()
+        self.in_features = in_features
+        self.out_features = out_features
+        self.bits = bits
+        self.group_size = group_size
+        self.requires_grad = False
+        if self.bits not in [2, 4, 8]:
+            raise ValueError("Only 2, 4, or 8 bits are supported.")
+        if group_size < 1:
+            raise ValueError("Group size must be at least 1.")
+        self.dtype = torch.float16          # the reference forces float16 whatever is asked (modules.py:167)
+        values_per_int32 = 32 // self.bits
+        self.register_buffer("qweight", torch.zeros((out_features, in_features // values_per_int32), dtype=torch.int32))
+        meta_shape = (out_features, in_features // group_size)
+        self.register_buffer("scale", torch.zeros(meta_shape, dtype=self.dtype))
+        self.register_buffer("zero_point", torch.zeros(meta_shape, dtype=self.dtype))
+        if bias:
+            self.register_buffer("bias", torch.zeros(out_features, dtype=self.dtype))
+        else:
+            self.bias = None
+
+    def forward(self, x):
+        return QuantizedLinearFunction.apply(x, self.qweight, self.scale, self.zero_point, self.bias, self.bits,
+                                             self.group_size)
+
+    @classmethod
+    def from_float(cls, float_layer: nn.Linear, bits=8, group_size=32):
+        """RTN-quantise an nn.Linear.  The reference upcasts the layer to float32, quantises, and stores
+        scale / zero_point as float16 (modules.py:189-213); here the upcast, the quantiser and the stores
+        are one kernel reading the layer's own dtype."""
+        if bits not in [2, 4, 8]:
+            raise AssertionError("Only 2, 4, or 8-bit quantization supported.")
+        weight = float_layer.weight.data
+        if weight.shape[1] % group_size:
+            pad = group_size - weight.shape[1] % group_size
+            raise ValueError(f"Padding {pad} columns to {weight.shape[1]} to make it a multiple of {group_size}")
+        device = weight.device
+        if weight.dtype not in (torch.float16, torch.bfloat16, torch.float32):
+            weight = weight.to(torch.float32)
+        if not weight.is_cuda:
+            if not torch.cuda.is_available():
+                raise _hip.BitweenHipError("QuantizedLinear.from_float needs a ROCm GPU (no CPU implementation)")
+            weight = weight.to("cuda")
+        qweight, scale, zero_point = _hip.quantize_pack(weight, bits, group_size, math_dtype=torch.float32,
+                                                        scale_dtype=torch.float16, zp_dtype=torch.float16)
+        q_layer = cls(float_layer.in_features, float_layer.out_features, bits, group_size,
+                      bias=float_layer.bias is not None, dtype=torch.float16)
+        q_layer = q_layer.to(device)
+        q_layer.qweight.copy_(qweight)
+        q_layer.scale.copy_(scale)
+        q_layer.zero_point.copy_(zero_point)
+        if float_layer.bias is not None:
+            q_layer.bias.data.copy_(float_layer.bias.data)
+        return q_layer
+
+    def __repr__(self):
+        return (f"QuantizedLinear(in_features={self.in_features}, out_features={self.out_features}, "
+                f"bias={self.bias is not None}, bits={self.bits}, group_size={self.group_size})")

@@ -1,0 +1,63 @@
+"""Bitween: the model-level quantiser (bitween/quantizer/quantizer.py:11-118).
+
+Only the RTN branch is on this package's path: every nn.Linear not listed in
+ignore_layers is replaced by QuantizedLinear.from_float.  Trainable
+quantisation and perplexity / KL evaluation belong to other subsystems of the
+reference (calibration data, training loop, downloaded datasets) and raise
+NotImplementedError here.
+"""
+import copy
+
+import torch.nn as nn
+
+from ..modules import QuantizedLinear
+from .func import _set_module
+
+
+class Bitween:
+    def __init__(self, model, tokenizer=None, bits=8, group_size=32, iters=1, lr=0.005, enable_minmax_tuning=True,
+                 seqlen=2048, cache_to_disk=False, max_memory_mb=512, ignore_layers=None, batch_size=32):
+        self.model = model
+        self.tokenizer = tokenizer
+        self.bits = bits
+        self.group_size = group_size
+        self.iters = iters
+        self.lr = lr
+        self.enable_minmax_tuning = enable_minmax_tuning
+        self.seqlen = seqlen
+        self.cache_to_disk = cache_to_disk
+        self.max_memory_mb = max_memory_mb
+        self.ignore_layers = set(ignore_layers) if ignore_layers else set()
+        self.batch_size = batch_size
+        assert group_size > 0, "Group size must be greater than 0."
+
+    def quantize(self, evaluate_perplexity=False, eval_samples=100, rtn=False, trainable=False, calib_dataset="pile-10k",
+                 nsamples=None, cache_to_disk=None, max_memory_mb=None, ignore_layers=None, batch_size=None,
+                 verbose=True, **eval_kwargs):
+        """Returns a deep copy of the model with its linear layers RTN-quantised.  As in the reference,
+        trainable=False selects RTN whatever `rtn` says (quantizer.py:67)."""
+        if trainable:
+            raise NotImplementedError("trainable quantisation is outside this package (RTN only)")
+        if evaluate_perplexity and self.tokenizer is not None and eval_samples > 0:
+            raise NotImplementedError("perplexity / KL evaluation needs the reference's dataset pipeline")
+        saved_ignore = self.ignore_layers
+        if ignore_layers is not None:
+            self.ignore_layers = set(ignore_layers)
+        if batch_size is not None:
+            self.batch_size = batch_size
+        try:
+            quantized_model = copy.deepcopy(self.model)
+            targets = [(name, module) for name, module in quantized_model.named_modules() if isinstance(module, nn.Linear)]
+            for name, module in targets:
+                if name in self.ignore_layers:
+                    if verbose:
+                        print(f"  - Skipping ignored layer: {name}")
+                    continue
+                if verbose:
+                    print(f"  - Quantizing layer: {name}")
+                _set_module(quantized_model, name, QuantizedLinear.from_float(module, self.bits, self.group_size))
+            if verbose:
+                print("--- Quantization complete ---")
+        finally:
+            self.ignore_layers = saved_ignore
+        return quantized_model

@@ -1,0 +1,104 @@
+/* bitween_hip.h - C ABI of libbitween_hip.so, the MI355X (gfx950) implementation
+ * of Bitween's quantized-linear hot path.
+ *
+ * The reference (Andriykkk/Bitween) is pure Python; its operator boundary for
+ * this path is the set of Python callables cited at each entry point below
+ * (paths relative to the reference checkout).  The host package bitween_amd
+ * keeps those callables' names and signatures and forwards to this ABI.
+ *
+ * Conventions for every entry point:
+ *   - plain C: pointers, sizes, ints.  All data pointers are DEVICE pointers
+ *     owned by the caller; nothing is allocated, freed or retained.
+ *   - `stream` is a hipStream_t passed as void* (NULL = the null stream).
+ *     Work is enqueued on it; no entry point synchronises.
+ *   - returns BW_OK (0) or a negative bw_status; never throws.  A non-zero
+ *     status means nothing was launched.
+ *   - weight layout is the reference's: W is [N][K] (N = out_features,
+ *     K = in_features); qweight is int32 [N][K*bits/32], value k of a row in
+ *     word k / (32/bits) at bit offset (k % (32/bits)) * bits
+ *     (bitween/functional.py:31-43); scale and zero_point are [N][K/group].
+ *   - bits is 2, 4 or 8; K % group == 0 and K % (32/bits) == 0.
+ */
+#ifndef BITWEEN_HIP_H
+#define BITWEEN_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum bw_dtype { BW_F16 = 0, BW_BF16 = 1, BW_F32 = 2, BW_I32 = 3 } bw_dtype;
+
+typedef enum bw_status {
+    BW_OK = 0,
+    BW_EINVAL = -1,       /* bad bits / group / shape / null pointer            */
+    BW_EUNSUPPORTED = -2, /* valid for the reference, not built here (see msg)  */
+    BW_EALIGN = -3,       /* pointer or pitch not aligned as the kernel needs   */
+    BW_ELAUNCH = -4,      /* the HIP runtime refused the launch                 */
+    BW_EWORKSPACE = -5    /* workspace missing or too small                     */
+} bw_status;
+
+/* Library ABI version (bumped on any signature change). */
+int bw_abi_version(void);
+
+/* Static text for a bw_status. */
+const char* bw_strerror(int status);
+
+/* quantize_rtn(weight, bits, group_size) -> (q_packed, scale, zero_point)
+ * replaces bitween/functional.py:3-45 and, through the output dtypes, the
+ * buffer stores of QuantizedLinear.from_float (bitween/modules.py:189-213).
+ *   w          [N][ldw] of w_dtype (BW_F16 | BW_BF16 | BW_F32), row pitch ldw elements
+ *   math_dtype dtype the arithmetic is rounded to after every operation:
+ *              BW_F32 = what from_float does (upcast first, modules.py:191);
+ *              BW_F16 / BW_BF16 = eager torch ops on a half tensor.
+ *   qweight    int32 [N][K*bits/32]
+ *   scale      [N][K/group] of scale_dtype (BW_F32 | BW_F16 | BW_BF16); a 16-bit
+ *              type applies the module's round-to-nearest-even store
+ *   zp         [N][K/group] of zp_dtype (BW_I32 | BW_F16 | BW_BF16)
+ * Bit-exact against the reference arithmetic for finite inputs. */
+int bw_quantize_pack(const void* w, int w_dtype, int math_dtype, int64_t N, int64_t K, int64_t ldw,
+                     int bits, int group, int32_t* qweight, void* scale, int scale_dtype,
+                     void* zp, int zp_dtype, void* stream);
+
+/* dequantize_rtn(q_packed, scale, zero_point, group_size, bits) -> weight
+ * replaces bitween/functional.py:47-71 (out_dtype BW_F32) and the per-forward
+ * dequantize kernel bitween/modules.py:10-58 (out_dtype BW_F16: one rounding
+ * of the float32 product).  BW_BF16 output is an extension.
+ *   scale [N][K/group] of scale_dtype (BW_F32 | BW_F16), zp of zp_dtype
+ *   (BW_I32 | BW_F16); w_out [N][ldo] of out_dtype.  Bit-exact. */
+int bw_dequantize(const int32_t* qweight, const void* scale, int scale_dtype, const void* zp, int zp_dtype,
+                  int64_t N, int64_t K, int bits, int group, void* w_out, int out_dtype, int64_t ldo,
+                  void* stream);
+
+/* Fused dequantize + matmul (+ bias):  y[M][N] = x[M][K] @ W16[N][K]^T + bias
+ * replaces QuantizedLinearFunction.forward (bitween/modules.py:62-106) and
+ * fills the slot of the absent bitween.kernels.cuda_loader.quantized_matmul_cuda
+ * (main.py:401,433).  W16 = fp16(scale16 * (q - zp16)) exactly as the
+ * reference dequantizes; products accumulate in float32; y is rounded once
+ * (the reference rounds before and after the bias add; within its 1e-2
+ * tolerance, main.py:471-477).
+ *   x      [M][ldx] of act_dtype (BW_F16; BW_BF16 where noted), y [M][ldy] same dtype
+ *   scale16, zp16  float16 [N][K/group] (the module buffers); zp16 must hold
+ *                  integers in [0, 2^bits), as every quantizer here produces
+ *   bias   [N] of act_dtype or NULL
+ * bw_qgemv: decode path, 1 <= M <= 16, HBM-bound, no workspace.
+ * bw_qgemm: prefill path, any M >= 1, MFMA-bound.
+ * bw_qlinear: picks between them by M (what the Python forward calls). */
+int bw_qgemv(const void* x, int act_dtype, int64_t M, int64_t K, int64_t ldx,
+             const int32_t* qweight, const void* scale16, const void* zp16, const void* bias,
+             int64_t N, int bits, int group, void* y, int64_t ldy, void* stream);
+
+int bw_qgemm(const void* x, int act_dtype, int64_t M, int64_t K, int64_t ldx,
+             const int32_t* qweight, const void* scale16, const void* zp16, const void* bias,
+             int64_t N, int bits, int group, void* y, int64_t ldy, void* stream);
+
+int bw_qlinear(const void* x, int act_dtype, int64_t M, int64_t K, int64_t ldx,
+               const int32_t* qweight, const void* scale16, const void* zp16, const void* bias,
+               int64_t N, int bits, int group, void* y, int64_t ldy, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* BITWEEN_HIP_H */

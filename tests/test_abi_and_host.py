@@ -1,0 +1,91 @@
+"""CPU-side checks: the C-ABI library loads and exports every symbol the
+header declares; the host layer validates arguments the way the reference
+does and refuses to run without a GPU instead of falling back."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "bitween_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(bw_[a-z_0-9]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    from bitween_amd.kernels import hip_loader
+    if not os.path.exists(hip_loader.library_path()):
+        from bitween_amd.csrc import build
+        build.build()
+    lib = ctypes.CDLL(hip_loader.library_path())
+    declared = _declared_symbols()
+    assert set(declared) == set(hip_loader.ENTRY_POINTS)
+    for name in declared:
+        assert hasattr(lib, name), name
+    lib.bw_abi_version.restype = ctypes.c_int
+    assert lib.bw_abi_version() == 1
+    lib.bw_strerror.restype = ctypes.c_char_p
+    assert lib.bw_strerror(0) == b"ok" and b"invalid" in lib.bw_strerror(-1)
+
+
+def test_entry_points_reject_bad_arguments_before_touching_the_gpu():
+    from bitween_amd.kernels import hip_loader
+    lib = hip_loader.load()
+    one = ctypes.c_void_p(16)
+    # bits = 3
+    assert lib.bw_quantize_pack(one, 2, 2, 4, 128, 128, 3, 32, one, one, 2, one, 3, None) == -1
+    # K % group != 0
+    assert lib.bw_quantize_pack(one, 2, 2, 4, 100, 100, 4, 32, one, one, 2, one, 3, None) == -1
+    # null pointers
+    assert lib.bw_dequantize(None, one, 0, one, 0, 4, 128, 4, 32, one, 0, 128, None) == -1
+    # M out of range for the decode kernel
+    assert lib.bw_qgemv(one, 0, 17, 128, 128, one, one, one, None, 16, 4, 32, one, 16, None) == -1
+    assert lib.bw_qgemv(one, 0, 0, 128, 128, one, one, one, None, 16, 4, 32, one, 16, None) == -1
+    # bf16 activations are not built
+    assert lib.bw_qgemv(one, 1, 1, 128, 128, one, one, one, None, 16, 4, 32, one, 16, None) == -2
+
+
+def test_host_layer_error_conventions_without_gpu():
+    import bitween_amd
+    with pytest.raises(AssertionError):                       # bitween/functional.py:6
+        bitween_amd.quantize_rtn(torch.zeros(4, 96), 3, 32)
+    with pytest.raises(ValueError):                           # bitween/functional.py:12-17
+        bitween_amd.quantize_rtn(torch.zeros(4, 100), 4, 32)
+    with pytest.raises(ValueError):                           # bitween/modules.py:157-161
+        bitween_amd.QuantizedLinear(64, 64, bits=5)
+    with pytest.raises(ValueError):
+        bitween_amd.QuantizedLinear(64, 64, bits=4, group_size=0)
+    with pytest.raises(AssertionError):                       # bitween/quantizer/quantizer.py:36
+        bitween_amd.Bitween(torch.nn.Linear(8, 8), group_size=0)
+    q = bitween_amd.QuantizedLinear(256, 64, bits=4, group_size=128, bias=True)
+    assert q.qweight.shape == (64, 32) and q.qweight.dtype == torch.int32
+    assert q.scale.shape == (64, 2) and q.scale.dtype == torch.float16 and q.zero_point.dtype == torch.float16
+    assert q.bias.dtype == torch.float16 and q.dtype == torch.float16 and q.requires_grad is False
+    assert bitween_amd.QuantizedLinear(256, 64, bias=False).bias is None
+
+
+@pytest.mark.skipif(torch.cuda.is_available(), reason="checks the no-GPU behaviour")
+def test_no_silent_cpu_fallback():
+    import bitween_amd
+    from bitween_amd.kernels.hip_loader import BitweenHipError
+    with pytest.raises(BitweenHipError):
+        bitween_amd.quantize_rtn(torch.randn(4, 128), 4, 32)
+    with pytest.raises(BitweenHipError):
+        bitween_amd.QuantizedLinear.from_float(torch.nn.Linear(128, 8), 4, 32)
+    q = bitween_amd.QuantizedLinear(128, 8, bits=4, group_size=32)
+    with pytest.raises(BitweenHipError):
+        q(torch.randn(2, 128))
+
+
+def test_product_code_never_touches_the_oracle():
+    pkg = os.path.join(ROOT, "bitween_amd")
+    for dirpath, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".py", ".hip", ".h", ".cpp")):
+                text = open(os.path.join(dirpath, f)).read()
+                assert "oracle" not in text, f"{f} mentions the oracle"
