@@ -1,0 +1,248 @@
+#!/usr/bin/env python3
+"""Headline benchmark: W4A16 g128 fused dequant-GEMM on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-extras]
+
+A step is one decode pass (M = 1) over the seven quantised linears of a
+Llama-2-7B decoder layer (q/k/v/o 4096x4096, gate/up 4096->11008, down
+11008->4096; 4-bit, group 128), inputs resident in HBM.  Successive steps use
+different layers' weights (--layers distinct copies, > 256 MiB in total) so
+the Infinity Cache cannot serve them.  `value` is algorithmic bytes per step
+(packed weights + scales + zero points + activations in + out) over the time
+per step, in GB/s.  The launches of a step are replayed from a HIP graph so
+the Python interpreter is not what is being timed.
+
+Also reported on the same JSON line: the roofline of the decode kernel, the
+CPU restatement timed on the host cores, and (unless --no-extras) per-M decode
+rates, prefill TFLOP/s next to same-run fp16 hipBLASLt, and quantiser rates.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0
+MFMA_F16_PEAK_TFLOPS = 2500.0
+LLAMA7B_LINEARS = [("q_proj", 4096, 4096), ("k_proj", 4096, 4096), ("v_proj", 4096, 4096), ("o_proj", 4096, 4096),
+                   ("gate_proj", 4096, 11008), ("up_proj", 4096, 11008), ("down_proj", 11008, 4096)]   # name, K, N
+
+
+def decode_bytes(m, k, n, bits, g):
+    """Algorithmic bytes of one fused forward: packed weights + scale + zero point + x + y (no bias)."""
+    return n * k * bits // 8 + 2 * n * (k // g) * 2 + m * k * 2 + m * n * 2
+
+
+def make_layer(torch, QuantizedLinear, k, n, bits, g, seed, outliers=False):
+    gen = torch.Generator(device="cuda").manual_seed(seed)
+    w = torch.randn(n, k, device="cuda", generator=gen) * 0.02
+    if outliers:
+        w = torch.where(torch.rand(n, k, device="cuda", generator=gen) < 0.001, w * 10, w)
+    lin = torch.nn.Linear(k, n, bias=False, device="cuda", dtype=torch.float16)
+    lin.weight.data = w.half()
+    q = QuantizedLinear.from_float(lin, bits, g)
+    del lin, w
+    return q
+
+
+def time_calls(torch, fn, iters, warmup):
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(iters):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) * 1e3 / iters      # us per call
+
+
+def graph_of(torch, fn):
+    g = torch.cuda.CUDAGraph()
+    s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s):
+        fn()                                       # warm the launch path outside capture
+    torch.cuda.current_stream().wait_stream(s)
+    torch.cuda.synchronize()
+    with torch.cuda.graph(g):
+        fn()
+    return g
+
+
+def cpu_baseline(bits, g):
+    """The C restatement of the reference path (oracle/rtn_oracle.c: dequantise to float16 values, float64
+    dot, float16 out) timed on this host for one 4096x4096 M=1 forward, OpenMP over the host's cores."""
+    import numpy as np
+    from oracle import c_oracle, rtn_oracle as orc
+    k = n = 4096
+    rng = np.random.default_rng(0)
+    w = (rng.standard_normal((n, k)) * 0.02).astype(np.float16).astype(np.float32)
+    qw, s, z = c_oracle.quantize_rtn_f32(w, bits, g)
+    s16, z16 = orc.store_module_buffers(s, z)
+    x = rng.standard_normal((1, k)).astype(np.float16)
+    cores = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
+    c_oracle.qlinear_forward(x, qw, s16, z16, None, bits, g)
+    t0 = time.perf_counter()
+    reps = 0
+    while time.perf_counter() - t0 < 10.0:
+        c_oracle.qlinear_forward(x, qw, s16, z16, None, bits, g)
+        reps += 1
+    dt = (time.perf_counter() - t0) / reps
+    return {"value": round(decode_bytes(1, k, n, bits, g) / dt / 1e9, 3), "unit": "GB/s", "cores": cores, "kind": "port",
+            "sample": f"{reps} forwards of one 4096x4096 W4 g128 linear, M=1 ({dt * 1e3:.2f} ms each), "
+                      "oracle/rtn_oracle.c orc_qlinear_forward with OpenMP"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=400)
+    ap.add_argument("--warmup", type=int, default=40)
+    ap.add_argument("--layers", type=int, default=8, help="distinct weight sets rotated through")
+    ap.add_argument("--m", type=int, default=1, help="decode batch of the headline number")
+    ap.add_argument("--no-graph", action="store_true")
+    ap.add_argument("--no-extras", action="store_true")
+    ap.add_argument("--no-cpu", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py measures one GPU: this path is a single-device operator and every box here has one GPU; "
+              "run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from bitween_amd import QuantizedLinear
+    from bitween_amd.kernels import hip_loader as hip
+    assert torch.cuda.is_available(), "bench.py needs the GPU"
+    hip.load()
+    torch.cuda.set_device(0)
+    bits, g, m = 4, 128, args.m
+
+    layers = [[make_layer(torch, QuantizedLinear, k, n, bits, g, seed=100 * li + i)
+               for i, (_, k, n) in enumerate(LLAMA7B_LINEARS)] for li in range(args.layers)]
+    xs = {k: torch.randn(m, k, device="cuda", dtype=torch.float16) for k in (4096, 11008)}
+    step_bytes = sum(decode_bytes(m, k, n, bits, g) for _, k, n in LLAMA7B_LINEARS)
+    launches_per_step = len(LLAMA7B_LINEARS)
+
+    def run_layer(li):
+        for q in layers[li]:
+            hip.quantized_gemv_hip(xs[q.in_features], q.qweight, q.scale, q.zero_point, None, bits, g)
+
+    if args.no_graph:
+        def do_steps(first, count):
+            for s in range(first, first + count):
+                run_layer(s % args.layers)
+    else:
+        per_layer = [graph_of(torch, lambda li=li: run_layer(li)) for li in range(args.layers)]
+        full = graph_of(torch, lambda: [run_layer(li) for li in range(args.layers)])
+
+        def do_steps(first, count):
+            s = first
+            while count > 0:
+                if s % args.layers == 0 and count >= args.layers:
+                    full.replay()
+                    s += args.layers
+                    count -= args.layers
+                else:
+                    per_layer[s % args.layers].replay()
+                    s += 1
+                    count -= 1
+
+    do_steps(0, args.warmup)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    do_steps(args.warmup, args.steps)
+    e1.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    dev_ms = e0.elapsed_time(e1)
+    ms_per_step = dev_ms / args.steps
+    gbps = step_bytes / (ms_per_step * 1e-3) / 1e9
+    us_per_launch = ms_per_step * 1e3 / launches_per_step
+    bytes_per_launch = step_bytes / launches_per_step
+
+    result = {
+        "metric": "W4A16 g128 dequant-GEMM: decode HBM GB/s (% peak); prefill TFLOP/s",
+        "value": round(gbps, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f16", "data": "synthetic",
+        "config": {"workload": "Llama-2-7B decoder-layer linears (q/k/v/o 4096x4096, gate/up 4096->11008, down "
+                               "11008->4096), 4-bit g128 RTN, fp16 activations, decode M=%d; one step = the 7 fused "
+                               "forwards of one layer, %d layers' weights rotated" % (m, args.layers),
+                   "M": m, "bits": bits, "group_size": g, "layers_rotated": args.layers,
+                   "bytes_per_step": step_bytes, "launch": "eager" if args.no_graph else "hip_graph"},
+        "pct_hbm_peak": round(100 * gbps / HBM_PEAK_GBPS, 2),
+        "wall_ms_total": round(wall_ms, 3),
+        "roofline": {"bound": "hbm", "achieved": round(bytes_per_launch / (us_per_launch * 1e-6) / 1e9, 1),
+                     "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(bytes_per_launch / (us_per_launch * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4),
+                     "traffic": None, "kernel": "qgemv_kernel<4,128>", "avg_launch_us": round(us_per_launch, 3),
+                     "bytes_per_launch": round(bytes_per_launch)},
+    }
+
+    if not args.no_extras:
+        extras = {}
+        # decode, every shape and M, rotating over the layer copies (eager launches, device time per call)
+        dec = {}
+        for idx, (name, k, n) in enumerate(LLAMA7B_LINEARS):
+            if name in ("k_proj", "v_proj", "o_proj", "up_proj"):
+                continue
+            for mm in (1, 4, 8, 16):
+                x = torch.randn(mm, k, device="cuda", dtype=torch.float16)
+                calls = [lambda li=li: hip.quantized_gemv_hip(x, layers[li][idx].qweight, layers[li][idx].scale,
+                                                              layers[li][idx].zero_point, None, bits, g)
+                         for li in range(args.layers)]
+                gr = graph_of(torch, lambda: [c() for c in calls])
+                us = time_calls(torch, gr.replay, 20, 3) / args.layers
+                dec[f"{name}_{k}x{n}_M{mm}"] = {"us": round(us, 2),
+                                               "GBps": round(decode_bytes(mm, k, n, bits, g) / us / 1e3, 1)}
+        extras["decode"] = dec
+        # same-run fp16 hipBLASLt GEMV on dequantised weights (reads 4x the bytes)
+        blas = {}
+        for name, k, n in (("q_proj", 4096, 4096), ("gate_proj", 4096, 11008)):
+            ws = [torch.randn(n, k, device="cuda", dtype=torch.float16) for _ in range(12)]
+            x = torch.randn(1, k, device="cuda", dtype=torch.float16)
+            gr = graph_of(torch, lambda: [torch.matmul(x, w.T) for w in ws])
+            us = time_calls(torch, gr.replay, 20, 3) / len(ws)
+            blas[f"{name}_{k}x{n}_M1"] = {"us": round(us, 2), "fp16_GBps": round(2 * n * k / us / 1e3, 1)}
+            del ws
+        extras["hipblaslt_fp16_decode"] = blas
+        # prefill: Llama-3-8B MLP shapes
+        pre = {}
+        for k, n in ((4096, 14336), (14336, 4096)):
+            q = make_layer(torch, QuantizedLinear, k, n, bits, g, seed=7)
+            w16 = hip.dequantize(q.qweight, q.scale, q.zero_point, g, bits, torch.float16)
+            for mm in (128, 512, 2048):
+                x = torch.randn(mm, k, device="cuda", dtype=torch.float16)
+                us_q = time_calls(torch, lambda: hip.quantized_gemm_hip(x, q.qweight, q.scale, q.zero_point, None, bits, g), 20, 5)
+                us_b = time_calls(torch, lambda: torch.matmul(x, w16.T), 20, 5)
+                fl = 2.0 * mm * n * k
+                pre[f"{k}x{n}_M{mm}"] = {"us": round(us_q, 1), "TFLOPs": round(fl / us_q / 1e6, 1),
+                                         "hipblaslt_fp16_us": round(us_b, 1), "hipblaslt_fp16_TFLOPs": round(fl / us_b / 1e6, 1),
+                                         "frac_of_hipblaslt": round(us_b / us_q, 3)}
+            del q, w16
+        extras["prefill"] = pre
+        # quantiser: fp16 weights in, packed + fp16 scale/zp out
+        qz = {}
+        for k, n in ((4096, 11008),):
+            ws = [(torch.randn(n, k, device="cuda") * 0.02).half() for _ in range(6)]
+            it = iter(range(10 ** 9))
+            us = time_calls(torch, lambda: hip.quantize_pack(ws[next(it) % 6], bits, g, torch.float32, torch.float16, torch.float16), 30, 6)
+            by = n * k * (2 + bits / 8 + 4 / g)
+            qz[f"{k}x{n}_f16_in"] = {"us": round(us, 1), "GBps": round(by / us / 1e3, 1), "Gweights_per_s": round(n * k / us / 1e3, 1)}
+        extras["quantize"] = qz
+        result["extras"] = extras
+
+    if not args.no_cpu:
+        result["cpu_baseline"] = cpu_baseline(bits, g)
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -37,7 +37,7 @@ def check_matmul(y_gpu, x16, qw, s16, z16, b16, bits, g, tol_rel=1e-2):
         float32 accumulation slack; far tighter than 1e-2, possible because the kernels reproduce W16 exactly.
     """
     y_ref, y64 = orc.qlinear_forward(x16, qw, s16, z16, b16, bits, g)
-    y = y_gpu.float().cpu().numpy().astype(np.float64)
+    y = y_gpu.detach().float().cpu().numpy().astype(np.float64)
     assert np.isfinite(y).all()
     w16 = np.abs(orc.dequantize_f16(qw, s16, z16, g, bits).astype(np.float64))
     mag = np.abs(x16.astype(np.float64)) @ w16.T
