@@ -64,49 +64,73 @@ template <> struct GroupConst<2> {
 
 constexpr uint32_t kMagic = 0x64006400u;   // two float16 1024.0
 
+// (a & mask) | orv in one VALU op.  The VOP3 encoding of gfx950 takes no 32-bit literals, so the
+// compiler emits v_and + v_or for literal operands; with the mask in an SGPR and the magic in a VGPR the
+// fused form is encodable.
+BW_DEV uint32_t and_or(uint32_t a, uint32_t mask, uint32_t orv) {
+    uint32_t d;
+    asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(d) : "v"(a), "s"(mask), "v"(orv));
+    return d;
+}
+
+// SCALE = true: out = fp16(s * (q - z)) (the reference's W16).  SCALE = false: out = q - z exactly
+// (the caller multiplies the group's partial dot product by s afterwards).
+
 // One 4-bit word (nibbles n0..n7) -> 4 pairs in slot order (n0,n4)(n1,n5)(n2,n6)(n3,n7).
+template <bool SCALE>
 BW_DEV void dequant_word4(uint32_t w, const GroupConst<4>& c, h2 out[4]) {
     const h2 k16 = splat((_Float16)0.0625f);
     const uint32_t w8 = w >> 8;
-    h2 a = as_h2((w & 0x000F000Fu) | kMagic);     // 1024 + n
-    h2 b = as_h2((w & 0x00F000F0u) | kMagic);     // 1024 + 16 n
-    h2 d = as_h2((w8 & 0x000F000Fu) | kMagic);
-    h2 e = as_h2((w8 & 0x00F000F0u) | kMagic);
-    out[0] = (a + c.z0) * c.s;
-    out[1] = __builtin_elementwise_fma(b, k16, c.z1) * c.s;
-    out[2] = (d + c.z0) * c.s;
-    out[3] = __builtin_elementwise_fma(e, k16, c.z1) * c.s;
+    h2 a = as_h2(and_or(w, 0x000F000Fu, kMagic));     // 1024 + n
+    h2 b = as_h2(and_or(w, 0x00F000F0u, kMagic));     // 1024 + 16 n
+    h2 d = as_h2(and_or(w8, 0x000F000Fu, kMagic));
+    h2 e = as_h2(and_or(w8, 0x00F000F0u, kMagic));
+    out[0] = a + c.z0;
+    out[1] = __builtin_elementwise_fma(b, k16, c.z1);
+    out[2] = d + c.z0;
+    out[3] = __builtin_elementwise_fma(e, k16, c.z1);
+    if constexpr (SCALE) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) out[i] = out[i] * c.s;
+    }
 }
 
 // One 8-bit word (bytes b0..b3) -> 2 pairs in natural order (b0,b1)(b2,b3).
+template <bool SCALE>
 BW_DEV void dequant_word8(uint32_t w, const GroupConst<8>& c, h2 out[2]) {
     h2 a = as_h2(__builtin_amdgcn_perm(0x64646464u, w, 0x04010400u));
     h2 b = as_h2(__builtin_amdgcn_perm(0x64646464u, w, 0x04030402u));
-    out[0] = (a + c.z0) * c.s;
-    out[1] = (b + c.z0) * c.s;
+    out[0] = a + c.z0;
+    out[1] = b + c.z0;
+    if constexpr (SCALE) { out[0] = out[0] * c.s; out[1] = out[1] * c.s; }
 }
 
 // One 2-bit word (crumbs c0..c15) -> 8 pairs (c_i, c_{i+8}), i = 0..7.
+template <bool SCALE>
 BW_DEV void dequant_word2(uint32_t w, const GroupConst<2>& c, h2 out[8]) {
     const uint32_t w10 = w >> 10;
-    h2 t0 = as_h2((w & 0x00030003u) | kMagic);     // 1024 + c
-    h2 t1 = as_h2((w & 0x000C000Cu) | kMagic);     // 1024 + 4c
-    h2 t2 = as_h2((w & 0x00300030u) | kMagic);     // 1024 + 16c
-    h2 t3 = as_h2((w & 0x00C000C0u) | kMagic);     // 1024 + 64c
-    h2 t4 = as_h2((w & 0x03000300u) | kMagic);     // 1024 + 256c
-    h2 t5 = as_h2((w10 & 0x00030003u) | kMagic);
-    h2 t6 = as_h2((w10 & 0x000C000Cu) | kMagic);
-    h2 t7 = as_h2((w10 & 0x00300030u) | kMagic);
+    h2 t0 = as_h2(and_or(w, 0x00030003u, kMagic));     // 1024 + c
+    h2 t1 = as_h2(and_or(w, 0x000C000Cu, kMagic));     // 1024 + 4c
+    h2 t2 = as_h2(and_or(w, 0x00300030u, kMagic));     // 1024 + 16c
+    h2 t3 = as_h2(and_or(w, 0x00C000C0u, kMagic));     // 1024 + 64c
+    h2 t4 = as_h2(and_or(w, 0x03000300u, kMagic));     // 1024 + 256c
+    h2 t5 = as_h2(and_or(w10, 0x00030003u, kMagic));
+    h2 t6 = as_h2(and_or(w10, 0x000C000Cu, kMagic));
+    h2 t7 = as_h2(and_or(w10, 0x00300030u, kMagic));
     const h2 k4 = splat((_Float16)0.25f), k16 = splat((_Float16)0.0625f), k64 = splat((_Float16)0.015625f),
              k256 = splat((_Float16)0.00390625f);
-    out[0] = (t0 + c.z0) * c.s;
-    out[1] = __builtin_elementwise_fma(t1, k4, c.z1) * c.s;
-    out[2] = __builtin_elementwise_fma(t2, k16, c.z2) * c.s;
-    out[3] = __builtin_elementwise_fma(t3, k64, c.z3) * c.s;
-    out[4] = __builtin_elementwise_fma(t4, k256, c.z4) * c.s;
-    out[5] = (t5 + c.z0) * c.s;
-    out[6] = __builtin_elementwise_fma(t6, k4, c.z1) * c.s;
-    out[7] = __builtin_elementwise_fma(t7, k16, c.z2) * c.s;
+    out[0] = t0 + c.z0;
+    out[1] = __builtin_elementwise_fma(t1, k4, c.z1);
+    out[2] = __builtin_elementwise_fma(t2, k16, c.z2);
+    out[3] = __builtin_elementwise_fma(t3, k64, c.z3);
+    out[4] = __builtin_elementwise_fma(t4, k256, c.z4);
+    out[5] = t5 + c.z0;
+    out[6] = __builtin_elementwise_fma(t6, k4, c.z1);
+    out[7] = __builtin_elementwise_fma(t7, k16, c.z2);
+    if constexpr (SCALE) {
+#pragma unroll
+        for (int i = 0; i < 8; i++) out[i] = out[i] * c.s;
+    }
 }
 
 // Position p of a block of VPI consecutive k holds original element perm(p):
@@ -119,17 +143,17 @@ template <> BW_DEV constexpr int slot_to_k<2>(int p) { return (p >> 1) + ((p & 1
 // Dequantise the 16 bytes a lane loaded (4 words = 128/BITS values) into
 // 128/BITS/2 float16 pairs, MFMA-operand ready: pairs [4t, 4t+4) feed MFMA t.
 // NG = number of quantisation groups those 16 bytes span (1 or 2).
-template <int BITS, int NG>
+template <int BITS, int NG, bool SCALE = true>
 BW_DEV void dequant_lane16(const u4& w, const GroupConst<BITS>* gc, h2* out) {
     if constexpr (BITS == 4) {
 #pragma unroll
-        for (int i = 0; i < 4; i++) dequant_word4(w[i], gc[NG == 1 ? 0 : i / (4 / NG)], out + 4 * i);
+        for (int i = 0; i < 4; i++) dequant_word4<SCALE>(w[i], gc[NG == 1 ? 0 : i / (4 / NG)], out + 4 * i);
     } else if constexpr (BITS == 8) {
 #pragma unroll
-        for (int i = 0; i < 4; i++) dequant_word8(w[i], gc[NG == 1 ? 0 : i / (4 / NG)], out + 2 * i);
+        for (int i = 0; i < 4; i++) dequant_word8<SCALE>(w[i], gc[NG == 1 ? 0 : i / (4 / NG)], out + 2 * i);
     } else {
 #pragma unroll
-        for (int i = 0; i < 4; i++) dequant_word2(w[i], gc[NG == 1 ? 0 : i / (4 / NG)], out + 8 * i);
+        for (int i = 0; i < 4; i++) dequant_word2<SCALE>(w[i], gc[NG == 1 ? 0 : i / (4 / NG)], out + 8 * i);
     }
 }
 

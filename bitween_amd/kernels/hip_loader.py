@@ -12,7 +12,8 @@ import os
 
 import torch
 
-_LIB_PATH = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "csrc", "libbitween_hip.so")
+_LIB_PATH = os.environ.get("BITWEEN_HIP_LIB") or os.path.join(
+    os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "csrc", "libbitween_hip.so")
 _lib = None
 
 BW_F16, BW_BF16, BW_F32, BW_I32 = 0, 1, 2, 3
