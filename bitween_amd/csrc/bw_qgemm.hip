@@ -16,7 +16,7 @@
 // apply (odd K or group size): correct for everything the reference accepts.
 #include "bw_common.h"
 
-bool bw_fast_shape(int64_t K, int bits, int group);
+bool bw_fast_shape(int64_t M, int64_t N, int64_t K, int64_t ldx, int bits, int group);
 
 namespace {
 
@@ -232,7 +232,7 @@ extern "C" int bw_qgemm(const void* x, int act_dtype, int64_t M, int64_t K, int6
     if (!x || !qweight || !scale16 || !zp16 || !y) return BW_EINVAL;
     if (!bw_shape_ok(N, K, bits, group) || M < 1 || M >= ((int64_t)1 << 31) || ldx < K || ldy < N) return BW_EINVAL;
     if (act_dtype != BW_F16) return BW_EUNSUPPORTED;
-    if (!bw_fast_shape(K, bits, group) || !bw_aligned(x, 16) || (ldx * 2) % 16 || !bw_aligned(qweight, 16))
+    if (!bw_fast_shape(M, N, K, ldx, bits, group) || !bw_aligned(x, 16) || (ldx * 2) % 16 || !bw_aligned(qweight, 16))
         return bw_qgemm_generic(x, act_dtype, M, K, ldx, qweight, scale16, zp16, bias, N, bits, group, y, ldy, stream);
     hipStream_t st = (hipStream_t)stream;
 #define BW_CASE(B, G) \
