@@ -108,6 +108,8 @@ def main():
     ap.add_argument("--no-graph", action="store_true")
     ap.add_argument("--no-extras", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="run only a plain 256 MiB device copy a few times (calibrates rocprof FETCH_SIZE/WRITE_SIZE)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one GPU: this path is a single-device operator and every box here has one GPU; "
@@ -121,6 +123,14 @@ def main():
     hip.load()
     torch.cuda.set_device(0)
     bits, g, m = 4, 128, args.m
+    if args.copy_probe:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda").fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"copy_probe_bytes": 256 << 20, "launches": 5}))
+        return
 
     layers = [[make_layer(torch, QuantizedLinear, k, n, bits, g, seed=100 * li + i)
                for i, (_, k, n) in enumerate(LLAMA7B_LINEARS)] for li in range(args.layers)]
@@ -182,7 +192,9 @@ def main():
         "roofline": {"bound": "hbm", "achieved": round(bytes_per_launch / (us_per_launch * 1e-6) / 1e9, 1),
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(bytes_per_launch / (us_per_launch * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4),
-                     "traffic": None, "kernel": "qgemv_kernel<4,128>", "avg_launch_us": round(us_per_launch, 3),
+                     # HBM bytes per launch from rocprofv3 FETCH_SIZE / WRITE_SIZE, scaled by the same counters on
+                     # a plain copy (profiles/qgemv_w4g128_llama7b_decode_M1_hbm_traffic.txt); not measurable live
+                     "traffic": 15531000 if m == 1 else None, "kernel": "qgemv_kernel<4,128>", "avg_launch_us": round(us_per_launch, 3),
                      "bytes_per_launch": round(bytes_per_launch)},
     }
 
