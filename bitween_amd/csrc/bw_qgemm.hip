@@ -18,31 +18,44 @@
 
 bool bw_fast_shape(int64_t M, int64_t N, int64_t K, int64_t ldx, int bits, int group);
 
+#ifdef BW_TRACE
+__device__ unsigned long long bw_gemm_trace[64 * 8];
+extern "C" int bw_debug_gemm_trace(unsigned long long* out) {
+    return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(bw_gemm_trace), sizeof(bw_gemm_trace));
+}
+#define BW_GT(slot) if (blockIdx.x == 3 && blockIdx.y == 0 && tid == 0 && c < 64) { asm volatile("" ::: "memory"); bw_gemm_trace[c * 8 + (slot)] = __builtin_amdgcn_s_memrealtime(); }
+#else
+#define BW_GT(slot)
+#endif
+
 namespace {
 
-constexpr int BM = 128, WAVES = 4, NT = 4, MT = BM / 16, BN = WAVES * NT * 16;
+constexpr int WAVES = 4, NT = 4, MT = 8, BM = MT * 16, BN = WAVES * NT * 16;
 
 template <int BITS, int GROUP>
 struct GemmCfg {
-    static constexpr int VPL = 128 / BITS, CHUNK_K = 4 * VPL, MF = VPL / 8;
+    static constexpr int VPI = 32 / BITS, VPL = 128 / BITS, CHUNK_K = 4 * VPL, MF = VPL / 8;
     static constexpr int NG = (VPL > GROUP) ? VPL / GROUP : 1;
-    static constexpr int PITCH = CHUNK_K + 8;                 // halves per LDS row
+    static constexpr int WPG = (GROUP >= VPL) ? 4 : 4 / NG;      // words of a lane load per group
+    static constexpr int PITCH = CHUNK_K + 8;                    // halves per LDS row
     static constexpr int STAGE_BYTES = BM * PITCH * 2;
+    static constexpr int UNIT = VPI > 8 ? VPI : 8;               // halves permuted together when staging x
+    static constexpr int UW = UNIT / 8;
+    static constexpr int UPR = CHUNK_K / UNIT;                   // staging units per x row
+    static constexpr int XL = BM * UPR / (WAVES * 64);           // staging units per thread
+    static_assert(BM * UPR % (WAVES * 64) == 0, "tile must split evenly over the workgroup");
 };
 
 template <int BITS>
-BW_DEV void permute16(const uint32_t* r, uint32_t* o) {
+BW_DEV void permute_unit(const uint32_t* r, uint32_t* o) {
     if constexpr (BITS == 8) {
 #pragma unroll
-        for (int j = 0; j < 8; j++) o[j] = r[j];
+        for (int j = 0; j < 4; j++) o[j] = r[j];
     } else if constexpr (BITS == 4) {
-#pragma unroll
-        for (int b = 0; b < 2; b++) {
-            o[4 * b + 0] = __builtin_amdgcn_perm(r[4 * b + 2], r[4 * b + 0], 0x05040100u);
-            o[4 * b + 1] = __builtin_amdgcn_perm(r[4 * b + 2], r[4 * b + 0], 0x07060302u);
-            o[4 * b + 2] = __builtin_amdgcn_perm(r[4 * b + 3], r[4 * b + 1], 0x05040100u);
-            o[4 * b + 3] = __builtin_amdgcn_perm(r[4 * b + 3], r[4 * b + 1], 0x07060302u);
-        }
+        o[0] = __builtin_amdgcn_perm(r[2], r[0], 0x05040100u);
+        o[1] = __builtin_amdgcn_perm(r[2], r[0], 0x07060302u);
+        o[2] = __builtin_amdgcn_perm(r[3], r[1], 0x05040100u);
+        o[3] = __builtin_amdgcn_perm(r[3], r[1], 0x07060302u);
     } else {
 #pragma unroll
         for (int j = 0; j < 8; j++)
@@ -50,67 +63,126 @@ BW_DEV void permute16(const uint32_t* r, uint32_t* o) {
     }
 }
 
+// Unpack word t of a lane load (8 values for MFMA step t at 4 bits; two steps' worth at 2 bits, half a
+// step at 8 bits is handled by the caller) - thin wrappers so the K loop can unpack just in time.
+template <int BITS>
+BW_DEV h8 unpack_step(const u4& w, int t, const GroupConst<BITS>* gc, int ng_words) {
+    h2 o[8];
+    if constexpr (BITS == 4) {
+        dequant_word4<true>(w[t], gc[t / ng_words], o);
+        return pack_h8(o);
+    } else if constexpr (BITS == 8) {
+        dequant_word8<true>(w[2 * t], gc[(2 * t) / ng_words], o);
+        dequant_word8<true>(w[2 * t + 1], gc[(2 * t + 1) / ng_words], o + 2);
+        return pack_h8(o);
+    } else {
+        dequant_word2<true>(w[t / 2], gc[(t / 2) / ng_words], o);
+        return pack_h8(o + 4 * (t & 1));
+    }
+}
+
+// The 128 accumulator registers of a wave live in the accumulation register file (AGPRs), leaving all 256
+// architectural VGPRs for operands and prefetch.  The compiler only selects the AGPR form of an MFMA when
+// asked through the operand constraint, hence the inline assembly.  Software-visible hazards of this
+// instruction on gfx950 concern reads of the result by non-MFMA instructions; the only such reads are in
+// the epilogue, hundreds of cycles (an LDS staging pass and a barrier) after the last MFMA.
+BW_DEV void mfma_acc(f4& acc, const h8& a, const h8& b) {
+#ifdef BW_MFMA_BUILTIN
+    acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, acc, 0, 0, 0);
+#else
+    asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
+#endif
+}
+
+struct GemmArgs {
+    const void* x;
+    const void* qweight;
+    const _Float16* scale;
+    const _Float16* zp;
+    const _Float16* bias;
+    _Float16* y;
+    uint32_t x_bytes, w_bytes, meta_bytes;
+    int M, N, K, ldx, ldy;
+    int groups, nchunks, row_bytes;
+};
+
+BW_DEV __amdgpu_buffer_rsrc_t make_rsrc(const void* p, uint32_t bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), (short)0, (int)bytes, 0x00020000);
+}
+
+// Software pipeline, one K step = one chunk:
+//   step c computes from LDS buffer c&1 and weight registers `wr`;
+//   the activations of step c+1 were requested one step earlier and are written to buffer (c+1)&1 after the
+//   MFMAs of step c; the weights of step c+1 likewise sit in `wn` and are moved to `wr`;
+//   then the loads of step c+2 are issued.  Every global load has a full K step (~2000 MFMA cycles) to land.
 template <int BITS, int GROUP>
-__global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(
-    const _Float16* __restrict__ x, int M, int K, int64_t ldx, const uint32_t* __restrict__ qweight,
-    const _Float16* __restrict__ scale, const _Float16* __restrict__ zp, const _Float16* __restrict__ bias, int N,
-    _Float16* __restrict__ y, int64_t ldy) {
+__global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
     using C = GemmCfg<BITS, GROUP>;
+    constexpr uint32_t kOob = 0x80000000u;
     extern __shared__ __attribute__((aligned(16))) char smem[];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int nl = lane & 15, kq = lane >> 4;
     const int m0 = blockIdx.y * BM;
     const int n0 = blockIdx.x * BN + wave * (NT * 16);
-    const int row_bytes = K * BITS / 8, groups = K / GROUP;
-    const int nchunks = (K + C::CHUNK_K - 1) / C::CHUNK_K;
+    const int groups = a.groups;
+    const __amdgpu_buffer_rsrc_t rw = make_rsrc(a.qweight, a.w_bytes), rx = make_rsrc(a.x, a.x_bytes);
 
-    const char* wrow[NT];
-    const _Float16 *srow[NT], *zrow[NT];
+    const __amdgpu_buffer_rsrc_t rs = make_rsrc(a.scale, a.meta_bytes), rz = make_rsrc(a.zp, a.meta_bytes);
+    uint32_t w_off[NT], m_off[NT];
 #pragma unroll
     for (int j = 0; j < NT; j++) {
-        const int row = min(n0 + 16 * j + nl, N - 1);
-        wrow[j] = reinterpret_cast<const char*>(qweight) + (int64_t)row * row_bytes;
-        srow[j] = scale + (int64_t)row * groups;
-        zrow[j] = zp + (int64_t)row * groups;
+        const int row = n0 + 16 * j + nl;
+        w_off[j] = row < a.N ? (uint32_t)row * a.row_bytes + kq * 16 : kOob;
+        m_off[j] = (uint32_t)min(row, a.N - 1) * groups * 2;
+    }
+    uint32_t x_off[C::XL];
+#pragma unroll
+    for (int i = 0; i < C::XL; i++) {
+        const int u = tid + i * WAVES * 64, m = u / C::UPR, ku = u - m * C::UPR;
+        x_off[i] = (m0 + m < a.M) ? (uint32_t)((m0 + m) * a.ldx + ku * C::UNIT) * 2 : kOob;
     }
 
-    // x tile staging: 16 halves per thread step
-    constexpr int BLK_PER_ROW = C::CHUNK_K / 16, STEPS = BM * BLK_PER_ROW / (WAVES * 64);
-    static_assert(BM * BLK_PER_ROW % (WAVES * 64) == 0, "tile must split evenly over the workgroup");
-    auto stage = [&](int chunk, _Float16* xs) {
+    u4 xr[C::XL * C::UW];
+    // Two weight register sets, used alternately by even and odd K steps and never copied: a register move
+    // of an outstanding load would stall on it.
+    struct WSet { u4 w[NT]; uint32_t s[NT][C::NG], z[NT][C::NG]; };   // 16-bit values, one register each
+    WSet set0, set1;
+    auto issue_x = [&](int c) {
+        const uint32_t kb = (uint32_t)c * C::CHUNK_K * 2;
 #pragma unroll
-        for (int s = 0; s < STEPS; s++) {
-            const int i = tid + s * WAVES * 64;
-            const int m = i / BLK_PER_ROW, kb = (i % BLK_PER_ROW) * 16;
-            const int k = chunk * C::CHUNK_K + kb;
-            uint32_t r[8], o[8];
-            if (m0 + m < M && k < K) {
-                const u4* src = reinterpret_cast<const u4*>(x + (int64_t)(m0 + m) * ldx + k);
-                u4 lo = src[0], hi = src[1];
-                r[0] = lo[0]; r[1] = lo[1]; r[2] = lo[2]; r[3] = lo[3];
-                r[4] = hi[0]; r[5] = hi[1]; r[6] = hi[2]; r[7] = hi[3];
-            } else {
+        for (int i = 0; i < C::XL; i++) {
+            const int ku = (tid + i * WAVES * 64) % C::UPR;
+            const uint32_t off = (c * C::CHUNK_K + ku * C::UNIT < a.K) ? x_off[i] + kb : kOob;
 #pragma unroll
-                for (int j = 0; j < 8; j++) r[j] = 0;
-            }
-            permute16<BITS>(r, o);
-            u4* dst = reinterpret_cast<u4*>(xs + m * C::PITCH + kb);
-            dst[0] = u4{o[0], o[1], o[2], o[3]};
-            dst[1] = u4{o[4], o[5], o[6], o[7]};
+            for (int j = 0; j < C::UW; j++) xr[i * C::UW + j] = __builtin_amdgcn_raw_buffer_load_b128(rx, off + j * 16, 0, 0);
         }
     };
-
-    u4 wreg[NT];
-    _Float16 sv[NT][C::NG], zv[NT][C::NG];
-    auto load_w = [&](int chunk) {
-        int kbyte = chunk * 64 + kq * 16;
-        kbyte = kbyte < row_bytes ? kbyte : 0;            // masked lanes: their x is staged as zero
-        const int g0 = (kbyte * 8 / BITS) / GROUP;
+    auto issue_w = [&](int c, WSet& ws) {
+        const bool in = c * 64 + kq * 16 < a.row_bytes;           // lanes past the row end: their x is zero
+        const int g0 = min((c * C::CHUNK_K + kq * C::VPL) / GROUP, groups - C::NG);
 #pragma unroll
         for (int j = 0; j < NT; j++) {
-            wreg[j] = *reinterpret_cast<const u4*>(wrow[j] + kbyte);
+            ws.w[j] = __builtin_amdgcn_raw_buffer_load_b128(rw, in ? w_off[j] + c * 64 : kOob, 0, 0);
 #pragma unroll
-            for (int g = 0; g < C::NG; g++) { sv[j][g] = srow[j][g0 + g]; zv[j][g] = zrow[j][g0 + g]; }
+            for (int g = 0; g < C::NG; g++) {
+                // zero-extending loads into whole registers: a 16-bit load into half a register would have
+                // to wait for the previous load into the other half
+                ws.s[j][g] = __builtin_amdgcn_raw_buffer_load_b16(rs, m_off[j] + (g0 + g) * 2, 0, 0);
+                ws.z[j][g] = __builtin_amdgcn_raw_buffer_load_b16(rz, m_off[j] + (g0 + g) * 2, 0, 0);
+            }
+        }
+    };
+    auto stage = [&](_Float16* xs) {
+#pragma unroll
+        for (int i = 0; i < C::XL; i++) {
+            const int u = tid + i * WAVES * 64, m = u / C::UPR, ku = u - m * C::UPR;
+            uint32_t in[4 * C::UW], o[4 * C::UW];
+#pragma unroll
+            for (int j = 0; j < C::UW; j++) { in[4 * j] = xr[i * C::UW + j][0]; in[4 * j + 1] = xr[i * C::UW + j][1]; in[4 * j + 2] = xr[i * C::UW + j][2]; in[4 * j + 3] = xr[i * C::UW + j][3]; }
+            permute_unit<BITS>(in, o);
+            u4* dst = reinterpret_cast<u4*>(xs + m * C::PITCH + ku * C::UNIT);
+#pragma unroll
+            for (int j = 0; j < C::UW; j++) dst[j] = u4{o[4 * j], o[4 * j + 1], o[4 * j + 2], o[4 * j + 3]};
         }
     };
 
@@ -120,69 +192,180 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(
 #pragma unroll
         for (int j = 0; j < NT; j++) acc[i][j] = f4{0.f, 0.f, 0.f, 0.f};
 
-    _Float16* buf0 = reinterpret_cast<_Float16*>(smem);
-    _Float16* buf1 = reinterpret_cast<_Float16*>(smem + C::STAGE_BYTES);
-    stage(0, buf0);
-    load_w(0);
-    __syncthreads();
-    for (int c = 0; c < nchunks; c++) {
-        _Float16* cur = (c & 1) ? buf1 : buf0;
-        _Float16* nxt = (c & 1) ? buf0 : buf1;
-        // unpack this chunk's weights, then refill the weight registers for the next one
-        h2 wp[NT][C::VPL / 2];
+    // Pieces of the staging / issue work, one per m-tile index, so they can be slotted between MFMA groups.
+    static_assert(C::XL <= MT && NT * 2 == MT, "at most one staging unit and half a weight tile per m-tile slot");
+    auto stage_unit = [&](int i, _Float16* xs) {
+        const int u = tid + i * WAVES * 64, m = u / C::UPR, ku = u - m * C::UPR;
+        uint32_t in[4 * C::UW], o[4 * C::UW];
 #pragma unroll
-        for (int j = 0; j < NT; j++) {
-            GroupConst<BITS> gc[C::NG];
+        for (int j = 0; j < C::UW; j++) { in[4 * j] = xr[i * C::UW + j][0]; in[4 * j + 1] = xr[i * C::UW + j][1]; in[4 * j + 2] = xr[i * C::UW + j][2]; in[4 * j + 3] = xr[i * C::UW + j][3]; }
+        permute_unit<BITS>(in, o);
+        u4* dst = reinterpret_cast<u4*>(xs + m * C::PITCH + ku * C::UNIT);
 #pragma unroll
-            for (int g = 0; g < C::NG; g++) gc[g].set(sv[j][g], zv[j][g]);
-            dequant_lane16<BITS, C::NG>(wreg[j], gc, wp[j]);
+        for (int j = 0; j < C::UW; j++) dst[j] = u4{o[4 * j], o[4 * j + 1], o[4 * j + 2], o[4 * j + 3]};
+    };
+    auto issue_x_unit = [&](int i, int c) {
+        const int ku = (tid + i * WAVES * 64) % C::UPR;
+        const uint32_t off = (c * C::CHUNK_K + ku * C::UNIT < a.K) ? x_off[i] + (uint32_t)c * C::CHUNK_K * 2 : kOob;
+#pragma unroll
+        for (int j = 0; j < C::UW; j++) xr[i * C::UW + j] = __builtin_amdgcn_raw_buffer_load_b128(rx, off + j * 16, 0, 0);
+    };
+    auto issue_w_tile = [&](int j, int c, WSet& ws) {
+        const bool in = c * 64 + kq * 16 < a.row_bytes;
+        ws.w[j] = __builtin_amdgcn_raw_buffer_load_b128(rw, in ? w_off[j] + c * 64 : kOob, 0, 0);
+    };
+    auto issue_meta = [&](int j, int which, int c, WSet& ws) {   // which: 0 = scales, 1 = zero points
+        const int g0 = min((c * C::CHUNK_K + kq * C::VPL) / GROUP, groups - C::NG);
+#pragma unroll
+        for (int g = 0; g < C::NG; g++) {
+            if (which == 0) ws.s[j][g] = __builtin_amdgcn_raw_buffer_load_b16(rs, m_off[j] + (g0 + g) * 2, 0, 0);
+            else ws.z[j][g] = __builtin_amdgcn_raw_buffer_load_b16(rz, m_off[j] + (g0 + g) * 2, 0, 0);
         }
-        if (c + 1 < nchunks) { load_w(c + 1); stage(c + 1, nxt); }
+    };
+
+    // One K step.  The 32 MFMAs of MFMA step t are issued in groups of 4 (one m-tile); between two groups
+    // sits one slice of other work, fenced so the compiler keeps it there:
+    //   t < last : the LDS read of one activation fragment and (every other slot) the unpack of one weight
+    //              fragment of step t+1;
+    //   t = last : one unit of the next chunk's activations (permute, LDS write, re-request for chunk c+2)
+    //              and (every other slot) the re-request of one weight tile for chunk c+2.
+    // Requests past the last chunk are range-checked to zero by the hardware; no branches, so every wait
+    // count is exact.
+    auto step = [&](int c, const _Float16* cur, _Float16* nxt, WSet& ws) {
+        __builtin_amdgcn_sched_barrier(0);
+        BW_GT(0)
+        GroupConst<BITS> gc[NT][C::NG];
+#pragma unroll
+        for (int j = 0; j < NT; j++)
+#pragma unroll
+            for (int g = 0; g < C::NG; g++)
+                gc[j][g].set(__builtin_bit_cast(_Float16, (uint16_t)ws.s[j][g]), __builtin_bit_cast(_Float16, (uint16_t)ws.z[j][g]));
         const _Float16* xp = cur + nl * C::PITCH + kq * C::VPL;
+        h8 xf[2][MT], wf[2][NT];
+#pragma unroll
+        for (int i = 0; i < MT; i++) xf[0][i] = *reinterpret_cast<const h8*>(xp + i * 16 * C::PITCH);
+#pragma unroll
+        for (int j = 0; j < NT; j++) wf[0][j] = unpack_step<BITS>(ws.w[j], 0, gc[j], C::WPG);
 #pragma unroll
         for (int t = 0; t < C::MF; t++) {
-            h8 b[NT];
-#pragma unroll
-            for (int j = 0; j < NT; j++) b[j] = pack_h8(wp[j] + 4 * t);
 #pragma unroll
             for (int i = 0; i < MT; i++) {
-                const h8 a = *reinterpret_cast<const h8*>(xp + i * 16 * C::PITCH + 8 * t);
+                __builtin_amdgcn_sched_barrier(0);
+                if (t == 0 && i == 1) { BW_GT(1) }
+                if (t == C::MF - 1 && i == 0) { BW_GT(2) }
+                if (t == C::MF - 1 && i == MT / 2) { BW_GT(3) }
+                // weights as the A operand: the result fragment holds 4 consecutive n per lane
 #pragma unroll
-                for (int j = 0; j < NT; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b[j], acc[i][j], 0, 0, 0);
+                for (int j = 0; j < NT; j++) mfma_acc(acc[i][j], wf[t & 1][j], xf[t & 1][i]);
+                __builtin_amdgcn_sched_barrier(0);
+                if (t + 1 < C::MF) {
+                    xf[(t + 1) & 1][i] = *reinterpret_cast<const h8*>(xp + i * 16 * C::PITCH + 8 * (t + 1));
+                    if (i & 1) wf[(t + 1) & 1][i / 2] = unpack_step<BITS>(ws.w[i / 2], t + 1, gc[i / 2], C::WPG);
+                }
+                // At most one global request per slot, spread over the whole K step: a burst of requests
+                // backs up the address unit and the wave - which issues in order - stops feeding MFMAs.
+                //   first MFMA step : activations of chunk c+1 (requested a step ago) to LDS, re-request
+                //   middle          : scales and zero points for chunk c+2 (their registers are free once
+                //                     the step's constants are formed)
+                //   last MFMA step  : weights for chunk c+2 (their registers are free after the last unpack)
+                constexpr int T_META = C::MF > 2 ? 1 : C::MF - 1;
+                if (t == 0 && i < C::XL) {
+                    stage_unit(i, nxt);
+                    issue_x_unit(i, c + 2);
+                }
+                if (t == T_META && (C::MF > 2 || (i & 1))) {
+                    const int q = C::MF > 2 ? i : i / 2;          // 0 .. 2*NT-1 when MF > 2, else 0 .. NT-1
+                    if (C::MF > 2) issue_meta(q / 2, q & 1, c + 2, ws);
+                    else { issue_meta(q, 0, c + 2, ws); issue_meta(q, 1, c + 2, ws); }
+                }
+                if (t == C::MF - 1 && !(i & 1)) issue_w_tile(i / 2, c + 2, ws);
+                asm volatile("" ::: "memory");
             }
         }
+        __builtin_amdgcn_sched_barrier(0);
+        BW_GT(4)
         __syncthreads();
+        BW_GT(5)
+    };
+
+    _Float16* buf0 = reinterpret_cast<_Float16*>(smem);
+    _Float16* buf1 = reinterpret_cast<_Float16*>(smem + C::STAGE_BYTES);
+    // Prologue: the same two request batches, in the same order, that a steady-state step finds
+    // outstanding - the compiler merges the wait counts of the loop entry with those of the back edge, and
+    // any difference in order makes the steady state wait for requests it has only just issued.
+    auto issue_batch = [&](int c, WSet& ws) {
+#pragma unroll
+        for (int i = 0; i < C::XL; i++) {
+            issue_x_unit(i, c);
+            asm volatile("" ::: "memory");
+            __builtin_amdgcn_sched_barrier(0);
+        }
+#pragma unroll
+        for (int j = 0; j < NT; j++) {
+            issue_meta(j, 0, c, ws);
+            issue_meta(j, 1, c, ws);
+            asm volatile("" ::: "memory");
+            __builtin_amdgcn_sched_barrier(0);
+        }
+#pragma unroll
+        for (int j = 0; j < NT; j++) {
+            issue_w_tile(j, c, ws);
+            asm volatile("" ::: "memory");
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+    issue_batch(0, set0);
+#pragma unroll
+    for (int i = 0; i < C::XL; i++) stage_unit(i, buf0);
+    __builtin_amdgcn_sched_barrier(0);
+    issue_batch(1, set1);
+    __syncthreads();
+    for (int c = 0; c < a.nchunks; c += 2) {   // an odd chunk count runs one extra step on zeros
+        step(c, buf0, buf1, set0);
+        step(c + 1, buf1, buf0, set1);
     }
-    // acc[i][j][r] = y[m0 + 16 i + 4 kq + r][n0 + 16 j + nl]
+    // acc[i][j][r] = y[m0 + 16 i + nl][n0 + 16 j + 4 kq + r]
 #pragma unroll
     for (int j = 0; j < NT; j++) {
-        const int n = n0 + 16 * j + nl;
-        if (n >= N) continue;
-        const float bv = bias ? (float)bias[n] : 0.f;
+        const int n = n0 + 16 * j + 4 * kq;
+        if (n >= a.N) continue;
+        float bv[4] = {0.f, 0.f, 0.f, 0.f};
+        if (a.bias) {
 #pragma unroll
-        for (int i = 0; i < MT; i++)
+            for (int r = 0; r < 4; r++) bv[r] = n + r < a.N ? (float)a.bias[n + r] : 0.f;
+        }
 #pragma unroll
-            for (int r = 0; r < 4; r++) {
-                const int m = m0 + 16 * i + 4 * kq + r;
-                if (m < M) y[(int64_t)m * ldy + n] = (_Float16)(acc[i][j][r] + bv);
+        for (int i = 0; i < MT; i++) {
+            const int m = m0 + 16 * i + nl;
+            if (m >= a.M) continue;
+            _Float16* dst = a.y + (int64_t)m * a.ldy + n;
+            const _Float16 v0 = (_Float16)(acc[i][j][0] + bv[0]), v1 = (_Float16)(acc[i][j][1] + bv[1]),
+                           v2 = (_Float16)(acc[i][j][2] + bv[2]), v3 = (_Float16)(acc[i][j][3] + bv[3]);
+            if (n + 3 < a.N && (((uintptr_t)dst) & 7) == 0) {
+                *reinterpret_cast<u2*>(dst) = u2{as_u32(h2{v0, v1}), as_u32(h2{v2, v3})};
+            } else {
+                dst[0] = v0;
+                if (n + 1 < a.N) dst[1] = v1;
+                if (n + 2 < a.N) dst[2] = v2;
+                if (n + 3 < a.N) dst[3] = v3;
             }
+        }
     }
 }
 
 template <int BITS, int GROUP>
-int launch_gemm(const void* x, int64_t M, int64_t K, int64_t ldx, const int32_t* qweight, const void* scale,
-                const void* zp, const void* bias, int64_t N, void* y, int64_t ldy, hipStream_t stream) {
+int launch_gemm(const GemmArgs& a, hipStream_t stream) {
     using C = GemmCfg<BITS, GROUP>;
     const size_t lds = 2 * (size_t)C::STAGE_BYTES;
     auto kern = qgemm_kernel<BITS, GROUP>;
-    if (lds > 64 * 1024) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) !=
-            hipSuccess)
+    static bool attr_set = false;
+    if (lds > 64 * 1024 && !attr_set) {
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) != hipSuccess)
             return BW_ELAUNCH;
+        attr_set = true;
     }
-    dim3 grid((unsigned)((N + BN - 1) / BN), (unsigned)((M + BM - 1) / BM)), block(WAVES * 64);
-    hipLaunchKernelGGL(kern, grid, block, lds, stream, (const _Float16*)x, (int)M, (int)K, ldx, (const uint32_t*)qweight,
-                       (const _Float16*)scale, (const _Float16*)zp, (const _Float16*)bias, (int)N, (_Float16*)y, ldy);
+    dim3 grid((unsigned)((a.N + BN - 1) / BN), (unsigned)((a.M + BM - 1) / BM)), block(WAVES * 64);
+    hipLaunchKernelGGL(kern, grid, block, lds, stream, a);
     return hipGetLastError() == hipSuccess ? BW_OK : BW_ELAUNCH;
 }
 
@@ -234,12 +417,25 @@ extern "C" int bw_qgemm(const void* x, int act_dtype, int64_t M, int64_t K, int6
     if (act_dtype != BW_F16) return BW_EUNSUPPORTED;
     if (!bw_fast_shape(M, N, K, ldx, bits, group) || !bw_aligned(x, 16) || (ldx * 2) % 16 || !bw_aligned(qweight, 16))
         return bw_qgemm_generic(x, act_dtype, M, K, ldx, qweight, scale16, zp16, bias, N, bits, group, y, ldy, stream);
+    GemmArgs a;
+    a.x = x; a.qweight = qweight; a.scale = (const _Float16*)scale16; a.zp = (const _Float16*)zp16;
+    a.bias = (const _Float16*)bias; a.y = (_Float16*)y;
+    a.M = (int)M; a.N = (int)N; a.K = (int)K; a.ldx = (int)ldx; a.ldy = (int)ldy;
+    a.groups = (int)(K / group);
+    a.row_bytes = (int)(K * bits / 8);
+    a.nchunks = (a.row_bytes + 63) / 64;
+    a.x_bytes = (uint32_t)(((M - 1) * ldx + K) * 2);
+    a.w_bytes = (uint32_t)(N * a.row_bytes);
+    a.meta_bytes = (uint32_t)(N * a.groups * 2);
     hipStream_t st = (hipStream_t)stream;
 #define BW_CASE(B, G) \
-    if (bits == B && group == G) return launch_gemm<B, G>(x, M, K, ldx, qweight, scale16, zp16, bias, N, y, ldy, st);
-    BW_CASE(4, 128) BW_CASE(4, 64) BW_CASE(4, 32)
+    if (bits == B && group == G) return launch_gemm<B, G>(a, st);
+    BW_CASE(4, 128)
+#ifndef BW_FAST_BUILD
+    BW_CASE(4, 64) BW_CASE(4, 32)
     BW_CASE(8, 128) BW_CASE(8, 64) BW_CASE(8, 32)
     BW_CASE(2, 128) BW_CASE(2, 64) BW_CASE(2, 32)
+#endif
 #undef BW_CASE
     return BW_EUNSUPPORTED;
 }
