@@ -104,6 +104,8 @@ struct GemmArgs {
     uint32_t x_bytes, w_bytes, meta_bytes;
     int M, N, K, ldx, ldy;
     int groups, nchunks, row_bytes;
+    float* ws;            // split-K partial sums [splits][M][N] (float32), or null
+    int chunks_per_split; // K chunks each z-slice of the grid takes
 };
 
 BW_DEV __amdgpu_buffer_rsrc_t make_rsrc(const void* p, uint32_t bytes) {
@@ -125,6 +127,8 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
     const int m0 = blockIdx.y * BM;
     const int n0 = blockIdx.x * BN + wave * (NT * 16);
     const int groups = a.groups;
+    // split-K: this z-slice of the grid takes chunks [c_begin, c_end); requests beyond c_end read as zero
+    const int c_begin = blockIdx.z * a.chunks_per_split, c_end = min(a.nchunks, c_begin + a.chunks_per_split);
     const __amdgpu_buffer_rsrc_t rw = make_rsrc(a.qweight, a.w_bytes), rx = make_rsrc(a.x, a.x_bytes);
 
     const __amdgpu_buffer_rsrc_t rs = make_rsrc(a.scale, a.meta_bytes), rz = make_rsrc(a.zp, a.meta_bytes);
@@ -152,13 +156,13 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
 #pragma unroll
         for (int i = 0; i < C::XL; i++) {
             const int ku = (tid + i * WAVES * 64) % C::UPR;
-            const uint32_t off = (c * C::CHUNK_K + ku * C::UNIT < a.K) ? x_off[i] + kb : kOob;
+            const uint32_t off = (c < c_end && c * C::CHUNK_K + ku * C::UNIT < a.K) ? x_off[i] + kb : kOob;
 #pragma unroll
             for (int j = 0; j < C::UW; j++) xr[i * C::UW + j] = __builtin_amdgcn_raw_buffer_load_b128(rx, off + j * 16, 0, 0);
         }
     };
     auto issue_w = [&](int c, WSet& ws) {
-        const bool in = c * 64 + kq * 16 < a.row_bytes;           // lanes past the row end: their x is zero
+        const bool in = c < c_end && c * 64 + kq * 16 < a.row_bytes;   // lanes past the row end: their x is zero
         const int g0 = min((c * C::CHUNK_K + kq * C::VPL) / GROUP, groups - C::NG);
 #pragma unroll
         for (int j = 0; j < NT; j++) {
@@ -206,12 +210,12 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
     };
     auto issue_x_unit = [&](int i, int c) {
         const int ku = (tid + i * WAVES * 64) % C::UPR;
-        const uint32_t off = (c * C::CHUNK_K + ku * C::UNIT < a.K) ? x_off[i] + (uint32_t)c * C::CHUNK_K * 2 : kOob;
+        const uint32_t off = (c < c_end && c * C::CHUNK_K + ku * C::UNIT < a.K) ? x_off[i] + (uint32_t)c * C::CHUNK_K * 2 : kOob;
 #pragma unroll
         for (int j = 0; j < C::UW; j++) xr[i * C::UW + j] = __builtin_amdgcn_raw_buffer_load_b128(rx, off + j * 16, 0, 0);
     };
     auto issue_w_tile = [&](int j, int c, WSet& ws) {
-        const bool in = c * 64 + kq * 16 < a.row_bytes;
+        const bool in = c < c_end && c * 64 + kq * 16 < a.row_bytes;
         ws.w[j] = __builtin_amdgcn_raw_buffer_load_b128(rw, in ? w_off[j] + c * 64 : kOob, 0, 0);
     };
     auto issue_meta = [&](int j, int which, int c, WSet& ws) {   // which: 0 = scales, 1 = zero points
@@ -241,45 +245,93 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
             for (int g = 0; g < C::NG; g++)
                 gc[j][g].set(__builtin_bit_cast(_Float16, (uint16_t)ws.s[j][g]), __builtin_bit_cast(_Float16, (uint16_t)ws.z[j][g]));
         const _Float16* xp = cur + nl * C::PITCH + kq * C::VPL;
-        h8 xf[2][MT], wf[2][NT];
+        h8 xf[2][MT];
+        h2 wf[2][NT][4];                                  // weight fragments as 4 register pairs each
 #pragma unroll
         for (int i = 0; i < MT; i++) xf[0][i] = *reinterpret_cast<const h8*>(xp + i * 16 * C::PITCH);
 #pragma unroll
-        for (int j = 0; j < NT; j++) wf[0][j] = unpack_step<BITS>(ws.w[j], 0, gc[j], C::WPG);
+        for (int j = 0; j < NT; j++) {
+            const h8 f = unpack_step<BITS>(ws.w[j], 0, gc[j], C::WPG);
+#pragma unroll
+            for (int e = 0; e < 4; e++) wf[0][j][e] = h2{f[2 * e], f[2 * e + 1]};
+        }
+        // At most one global request per slot, spread over the whole K step: a burst of requests backs up
+        // the address unit and the wave - which issues in order - stops feeding MFMAs.
+        //   first MFMA step : activations of chunk c+1 (requested a step ago) to LDS, re-request
+        //   middle          : scales and zero points for chunk c+2 (their registers are free once the
+        //                     step's constants are formed)
+        //   last MFMA step  : weights for chunk c+2 (their registers are free after the last unpack)
+        auto slot_requests = [&](int t, int i) {
+            constexpr int T_META = C::MF > 2 ? 1 : C::MF - 1;
+            if (t == 0 && i < C::XL) {
+                stage_unit(i, nxt);
+                issue_x_unit(i, c + 2);
+            }
+            if (t == T_META && (C::MF > 2 || (i & 1))) {
+                const int q = C::MF > 2 ? i : i / 2;              // 0 .. 2*NT-1 when MF > 2, else 0 .. NT-1
+                if (C::MF > 2) issue_meta(q / 2, q & 1, c + 2, ws);
+                else { issue_meta(q, 0, c + 2, ws); issue_meta(q, 1, c + 2, ws); }
+            }
+            if (t == C::MF - 1 && !(i & 1)) issue_w_tile(i / 2, c + 2, ws);
+            asm volatile("" ::: "memory");
+        };
 #pragma unroll
         for (int t = 0; t < C::MF; t++) {
+            const int cu = t & 1, nx = cu ^ 1;
 #pragma unroll
             for (int i = 0; i < MT; i++) {
-                __builtin_amdgcn_sched_barrier(0);
                 if (t == 0 && i == 1) { BW_GT(1) }
                 if (t == C::MF - 1 && i == 0) { BW_GT(2) }
                 if (t == C::MF - 1 && i == MT / 2) { BW_GT(3) }
-                // weights as the A operand: the result fragment holds 4 consecutive n per lane
+                if constexpr (BITS == 4) {
+                    // An MFMA occupies the matrix pipe for 16 cycles but the issue port for 4: two or three
+                    // VALU operations fit behind each one.  Slot i prepares half a weight fragment of
+                    // MFMA step t+1 (tile i/2, words' low or high byte pair) in four such pieces.
+                    const int jn = i / 2;
+                    const GroupConst<4>& g4 = gc[jn][(t + 1 < C::MF ? t + 1 : t) / C::WPG];
+                    const h2 k16 = splat((_Float16)0.0625f);
+                    uint32_t wsrc = 0;
+                    h2 pa = {0, 0}, pb = {0, 0};
 #pragma unroll
-                for (int j = 0; j < NT; j++) mfma_acc(acc[i][j], wf[t & 1][j], xf[t & 1][i]);
-                __builtin_amdgcn_sched_barrier(0);
-                if (t + 1 < C::MF) {
-                    xf[(t + 1) & 1][i] = *reinterpret_cast<const h8*>(xp + i * 16 * C::PITCH + 8 * (t + 1));
-                    if (i & 1) wf[(t + 1) & 1][i / 2] = unpack_step<BITS>(ws.w[i / 2], t + 1, gc[i / 2], C::WPG);
+                    for (int j = 0; j < NT; j++) {
+                        __builtin_amdgcn_sched_barrier(0);
+                        mfma_acc(acc[i][j], pack_h8(wf[cu][j]), xf[cu][i]);
+                        __builtin_amdgcn_sched_barrier(0);
+                        if (t + 1 < C::MF) {
+                            if (j == 0) {
+                                xf[nx][i] = *reinterpret_cast<const h8*>(xp + i * 16 * C::PITCH + 8 * (t + 1));
+                                wsrc = (i & 1) ? ws.w[jn][t + 1] >> 8 : ws.w[jn][t + 1];
+                                pa = as_h2(and_or(wsrc, 0x000F000Fu, kMagic));
+                            } else if (j == 1) {
+                                pb = as_h2(and_or(wsrc, 0x00F000F0u, kMagic));
+                                pa = pa + g4.z0;
+                            } else if (j == 2) {
+                                pb = __builtin_elementwise_fma(pb, k16, g4.z1);
+                                pa = pa * g4.s;
+                            } else {
+                                pb = pb * g4.s;
+                                wf[nx][jn][2 * (i & 1)] = pa;
+                                wf[nx][jn][2 * (i & 1) + 1] = pb;
+                            }
+                        }
+                        if (j == NT - 1) slot_requests(t, i);
+                    }
+                } else {
+                    __builtin_amdgcn_sched_barrier(0);
+                    // weights as the A operand: the result fragment holds 4 consecutive n per lane
+#pragma unroll
+                    for (int j = 0; j < NT; j++) mfma_acc(acc[i][j], pack_h8(wf[cu][j]), xf[cu][i]);
+                    __builtin_amdgcn_sched_barrier(0);
+                    if (t + 1 < C::MF) {
+                        xf[nx][i] = *reinterpret_cast<const h8*>(xp + i * 16 * C::PITCH + 8 * (t + 1));
+                        if (i & 1) {
+                            const h8 f = unpack_step<BITS>(ws.w[i / 2], t + 1, gc[i / 2], C::WPG);
+#pragma unroll
+                            for (int e = 0; e < 4; e++) wf[nx][i / 2][e] = h2{f[2 * e], f[2 * e + 1]};
+                        }
+                    }
+                    slot_requests(t, i);
                 }
-                // At most one global request per slot, spread over the whole K step: a burst of requests
-                // backs up the address unit and the wave - which issues in order - stops feeding MFMAs.
-                //   first MFMA step : activations of chunk c+1 (requested a step ago) to LDS, re-request
-                //   middle          : scales and zero points for chunk c+2 (their registers are free once
-                //                     the step's constants are formed)
-                //   last MFMA step  : weights for chunk c+2 (their registers are free after the last unpack)
-                constexpr int T_META = C::MF > 2 ? 1 : C::MF - 1;
-                if (t == 0 && i < C::XL) {
-                    stage_unit(i, nxt);
-                    issue_x_unit(i, c + 2);
-                }
-                if (t == T_META && (C::MF > 2 || (i & 1))) {
-                    const int q = C::MF > 2 ? i : i / 2;          // 0 .. 2*NT-1 when MF > 2, else 0 .. NT-1
-                    if (C::MF > 2) issue_meta(q / 2, q & 1, c + 2, ws);
-                    else { issue_meta(q, 0, c + 2, ws); issue_meta(q, 1, c + 2, ws); }
-                }
-                if (t == C::MF - 1 && !(i & 1)) issue_w_tile(i / 2, c + 2, ws);
-                asm volatile("" ::: "memory");
             }
         }
         __builtin_amdgcn_sched_barrier(0);
@@ -314,17 +366,40 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
             __builtin_amdgcn_sched_barrier(0);
         }
     };
-    issue_batch(0, set0);
+    issue_batch(c_begin, set0);
 #pragma unroll
     for (int i = 0; i < C::XL; i++) stage_unit(i, buf0);
     __builtin_amdgcn_sched_barrier(0);
-    issue_batch(1, set1);
+    issue_batch(c_begin + 1, set1);
     __syncthreads();
-    for (int c = 0; c < a.nchunks; c += 2) {   // an odd chunk count runs one extra step on zeros
+    for (int c = c_begin; c < c_end; c += 2) {   // an odd chunk count runs one extra step on zeros
         step(c, buf0, buf1, set0);
         step(c + 1, buf1, buf0, set1);
     }
     // acc[i][j][r] = y[m0 + 16 i + nl][n0 + 16 j + 4 kq + r]
+    if (a.ws) {
+        // split-K: float32 partial sums to the workspace; qgemm_reduce_kernel adds them up
+        float* wz = a.ws + (size_t)blockIdx.z * a.M * a.N;
+#pragma unroll
+        for (int j = 0; j < NT; j++) {
+            const int n = n0 + 16 * j + 4 * kq;
+            if (n >= a.N) continue;
+#pragma unroll
+            for (int i = 0; i < MT; i++) {
+                const int m = m0 + 16 * i + nl;
+                if (m >= a.M) continue;
+                float* dst = wz + (size_t)m * a.N + n;
+                if (n + 3 < a.N && (((uintptr_t)dst) & 15) == 0) {
+                    *reinterpret_cast<f4*>(dst) = acc[i][j];
+                } else {
+#pragma unroll
+                    for (int r = 0; r < 4; r++)
+                        if (n + r < a.N) dst[r] = acc[i][j][r];
+                }
+            }
+        }
+        return;
+    }
 #pragma unroll
     for (int j = 0; j < NT; j++) {
         const int n = n0 + 16 * j + 4 * kq;
@@ -353,8 +428,32 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
     }
 }
 
+// y[m][n] = fp16( sum_z ws[z][m][n] + bias[n] )
+__global__ __launch_bounds__(256) void qgemm_reduce_kernel(const float* __restrict__ ws, int splits, int M, int N,
+                                                           const _Float16* __restrict__ bias, _Float16* __restrict__ y,
+                                                           int ldy) {
+    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t total = (int64_t)M * N;
+    if (idx >= total) return;
+    float v = 0.f;
+    for (int z = 0; z < splits; z++) v += ws[z * total + idx];
+    const int m = (int)(idx / N), n = (int)(idx - (int64_t)m * N);
+    if (bias) v += (float)bias[n];
+    y[(int64_t)m * ldy + n] = (_Float16)v;
+}
+
+// How many z-slices to cut K into.  One workgroup fits per CU, so the grid runs in waves of 256 workgroups:
+// splitting pays only while tiles * splits still fits one wave, and never below 4 chunks per slice.
+inline int gemm_splits(int64_t M, int64_t N, int nchunks) {
+    const int64_t tiles = ((N + BN - 1) / BN) * ((M + BM - 1) / BM);
+    if (tiles > 128) return 1;
+    int s = (int)(256 / tiles);
+    if (s > nchunks / 4) s = nchunks / 4;
+    return s < 2 ? 1 : s;
+}
+
 template <int BITS, int GROUP>
-int launch_gemm(const GemmArgs& a, hipStream_t stream) {
+int launch_gemm(GemmArgs a, void* workspace, size_t workspace_bytes, hipStream_t stream) {
     using C = GemmCfg<BITS, GROUP>;
     const size_t lds = 2 * (size_t)C::STAGE_BYTES;
     auto kern = qgemm_kernel<BITS, GROUP>;
@@ -364,9 +463,22 @@ int launch_gemm(const GemmArgs& a, hipStream_t stream) {
             return BW_ELAUNCH;
         attr_set = true;
     }
-    dim3 grid((unsigned)((a.N + BN - 1) / BN), (unsigned)((a.M + BM - 1) / BM)), block(WAVES * 64);
+    int splits = workspace ? gemm_splits(a.M, a.N, a.nchunks) : 1;
+    if (splits > 1 && workspace_bytes < (size_t)splits * a.M * a.N * sizeof(float)) return BW_EWORKSPACE;
+    a.chunks_per_split = (a.nchunks + splits - 1) / splits;
+    a.chunks_per_split += a.chunks_per_split & 1;             // even: the K loop runs two steps per pass
+    splits = (a.nchunks + a.chunks_per_split - 1) / a.chunks_per_split;
+    a.ws = splits > 1 ? (float*)workspace : nullptr;
+    dim3 grid((unsigned)((a.N + BN - 1) / BN), (unsigned)((a.M + BM - 1) / BM), (unsigned)splits), block(WAVES * 64);
     hipLaunchKernelGGL(kern, grid, block, lds, stream, a);
-    return hipGetLastError() == hipSuccess ? BW_OK : BW_ELAUNCH;
+    if (hipGetLastError() != hipSuccess) return BW_ELAUNCH;
+    if (splits > 1) {
+        const int64_t total = (int64_t)a.M * a.N;
+        hipLaunchKernelGGL(qgemm_reduce_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, a.ws, splits,
+                           a.M, a.N, a.bias, a.y, a.ldy);
+        if (hipGetLastError() != hipSuccess) return BW_ELAUNCH;
+    }
+    return BW_OK;
 }
 
 // Shape-generic fallback: one thread per output element, any group size and
@@ -409,14 +521,22 @@ int bw_qgemm_generic(const void* x, int act_dtype, int64_t M, int64_t K, int64_t
     return hipGetLastError() == hipSuccess ? BW_OK : BW_ELAUNCH;
 }
 
-extern "C" int bw_qgemm(const void* x, int act_dtype, int64_t M, int64_t K, int64_t ldx, const int32_t* qweight,
-                        const void* scale16, const void* zp16, const void* bias, int64_t N, int bits, int group,
-                        void* y, int64_t ldy, void* stream) {
+extern "C" size_t bw_qgemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int bits, int group) {
+    if (!bw_shape_ok(N, K, bits, group) || M < 1 || !bw_fast_shape(M, N, K, K, bits, group)) return 0;
+    const int nchunks = (int)((K * bits / 8 + 63) / 64);
+    const int splits = gemm_splits(M, N, nchunks);
+    return splits > 1 ? (size_t)splits * M * N * sizeof(float) : 0;
+}
+
+extern "C" int bw_qgemm_ws(const void* x, int act_dtype, int64_t M, int64_t K, int64_t ldx, const int32_t* qweight,
+                           const void* scale16, const void* zp16, const void* bias, int64_t N, int bits, int group,
+                           void* y, int64_t ldy, void* workspace, size_t workspace_bytes, void* stream) {
     if (!x || !qweight || !scale16 || !zp16 || !y) return BW_EINVAL;
     if (!bw_shape_ok(N, K, bits, group) || M < 1 || M >= ((int64_t)1 << 31) || ldx < K || ldy < N) return BW_EINVAL;
     if (act_dtype != BW_F16) return BW_EUNSUPPORTED;
     if (!bw_fast_shape(M, N, K, ldx, bits, group) || !bw_aligned(x, 16) || (ldx * 2) % 16 || !bw_aligned(qweight, 16))
         return bw_qgemm_generic(x, act_dtype, M, K, ldx, qweight, scale16, zp16, bias, N, bits, group, y, ldy, stream);
+    if (workspace && !bw_aligned(workspace, 16)) return BW_EALIGN;
     GemmArgs a;
     a.x = x; a.qweight = qweight; a.scale = (const _Float16*)scale16; a.zp = (const _Float16*)zp16;
     a.bias = (const _Float16*)bias; a.y = (_Float16*)y;
@@ -427,9 +547,11 @@ extern "C" int bw_qgemm(const void* x, int act_dtype, int64_t M, int64_t K, int6
     a.x_bytes = (uint32_t)(((M - 1) * ldx + K) * 2);
     a.w_bytes = (uint32_t)(N * a.row_bytes);
     a.meta_bytes = (uint32_t)(N * a.groups * 2);
+    a.ws = nullptr;
+    a.chunks_per_split = a.nchunks;
     hipStream_t st = (hipStream_t)stream;
 #define BW_CASE(B, G) \
-    if (bits == B && group == G) return launch_gemm<B, G>(a, st);
+    if (bits == B && group == G) return launch_gemm<B, G>(a, workspace, workspace_bytes, st);
     BW_CASE(4, 128)
 #ifndef BW_FAST_BUILD
     BW_CASE(4, 64) BW_CASE(4, 32)
@@ -438,6 +560,12 @@ extern "C" int bw_qgemm(const void* x, int act_dtype, int64_t M, int64_t K, int6
 #endif
 #undef BW_CASE
     return BW_EUNSUPPORTED;
+}
+
+extern "C" int bw_qgemm(const void* x, int act_dtype, int64_t M, int64_t K, int64_t ldx, const int32_t* qweight,
+                        const void* scale16, const void* zp16, const void* bias, int64_t N, int bits, int group,
+                        void* y, int64_t ldy, void* stream) {
+    return bw_qgemm_ws(x, act_dtype, M, K, ldx, qweight, scale16, zp16, bias, N, bits, group, y, ldy, nullptr, 0, stream);
 }
 
 extern "C" int bw_qlinear(const void* x, int act_dtype, int64_t M, int64_t K, int64_t ldx, const int32_t* qweight,

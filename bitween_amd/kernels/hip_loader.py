@@ -20,7 +20,7 @@ BW_F16, BW_BF16, BW_F32, BW_I32 = 0, 1, 2, 3
 _DTYPE_CODE = {torch.float16: BW_F16, torch.bfloat16: BW_BF16, torch.float32: BW_F32, torch.int32: BW_I32}
 
 ENTRY_POINTS = ("bw_abi_version", "bw_strerror", "bw_quantize_pack", "bw_dequantize", "bw_qgemv", "bw_qgemm",
-                "bw_qlinear")
+                "bw_qgemm_ws", "bw_qgemm_workspace_bytes", "bw_qlinear")
 
 
 class BitweenHipError(RuntimeError):
@@ -50,7 +50,10 @@ def load():
     mm = [vp, i32, i64, i64, i64, vp, vp, vp, vp, i64, i32, i32, vp, i64, vp]
     for name in ("bw_qgemv", "bw_qgemm", "bw_qlinear"):
         getattr(lib, name).argtypes = mm
-    for name in ("bw_quantize_pack", "bw_dequantize", "bw_qgemv", "bw_qgemm", "bw_qlinear"):
+    lib.bw_qgemm_ws.argtypes = mm[:-1] + [vp, ctypes.c_size_t, vp]
+    lib.bw_qgemm_workspace_bytes.argtypes = [i64, i64, i64, i32, i32]
+    lib.bw_qgemm_workspace_bytes.restype = ctypes.c_size_t
+    for name in ("bw_quantize_pack", "bw_dequantize", "bw_qgemv", "bw_qgemm", "bw_qgemm_ws", "bw_qlinear"):
         getattr(lib, name).restype = i32
     _lib = lib
     return lib
@@ -130,11 +133,21 @@ def _matmul(entry, x, qweight, scale, zero_point, bias, bits, group_size):
     y = torch.empty((m, n), dtype=x.dtype, device=x.device)
     if m == 0:
         return y
+    lib = load()
+    bias_ptr = None if bias is None else bias.contiguous().data_ptr()
     with torch.cuda.device(x.device):
-        st = getattr(load(), entry)(x.data_ptr(), _DTYPE_CODE[x.dtype], m, k, x.stride(0), qweight.data_ptr(),
-                                    scale.data_ptr(), zero_point.data_ptr(),
-                                    None if bias is None else bias.contiguous().data_ptr(), n, bits, group_size,
-                                    y.data_ptr(), n, _stream(x.device))
+        if entry != "bw_qgemv" and m > 16:
+            # prefill: give the library a split-K workspace when the shape wants one
+            nbytes = lib.bw_qgemm_workspace_bytes(m, n, k, bits, group_size)
+            ws = torch.empty(nbytes, dtype=torch.uint8, device=x.device) if nbytes else None
+            st = lib.bw_qgemm_ws(x.data_ptr(), _DTYPE_CODE[x.dtype], m, k, x.stride(0), qweight.data_ptr(),
+                                 scale.data_ptr(), zero_point.data_ptr(), bias_ptr, n, bits, group_size,
+                                 y.data_ptr(), n, None if ws is None else ws.data_ptr(), nbytes, _stream(x.device))
+            entry = "bw_qgemm_ws"
+        else:
+            st = getattr(lib, entry)(x.data_ptr(), _DTYPE_CODE[x.dtype], m, k, x.stride(0), qweight.data_ptr(),
+                                     scale.data_ptr(), zero_point.data_ptr(), bias_ptr, n, bits, group_size,
+                                     y.data_ptr(), n, _stream(x.device))
     _check(st, entry)
     return y
 

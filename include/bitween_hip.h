@@ -94,6 +94,19 @@ int bw_qgemm(const void* x, int act_dtype, int64_t M, int64_t K, int64_t ldx,
              const int32_t* qweight, const void* scale16, const void* zp16, const void* bias,
              int64_t N, int bits, int group, void* y, int64_t ldy, void* stream);
 
+/* Prefill with split-K.  When the (M, N) tile grid alone would leave most of the chip idle (small M*N,
+ * long K) bw_qgemm_ws cuts K into slices that run in parallel and adds their float32 partial sums in a
+ * second kernel; the partial sums live in a caller-provided device workspace of at least
+ * bw_qgemm_workspace_bytes(...) bytes (16-byte aligned; 0 = this shape needs none).  With workspace ==
+ * NULL it behaves exactly like bw_qgemm.  No counterpart in the reference (its forward is one library
+ * GEMM, bitween/modules.py:97). */
+size_t bw_qgemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int bits, int group);
+
+int bw_qgemm_ws(const void* x, int act_dtype, int64_t M, int64_t K, int64_t ldx,
+                const int32_t* qweight, const void* scale16, const void* zp16, const void* bias,
+                int64_t N, int bits, int group, void* y, int64_t ldy,
+                void* workspace, size_t workspace_bytes, void* stream);
+
 int bw_qlinear(const void* x, int act_dtype, int64_t M, int64_t K, int64_t ldx,
                const int32_t* qweight, const void* scale16, const void* zp16, const void* bias,
                int64_t N, int bits, int group, void* y, int64_t ldy, void* stream);

@@ -48,6 +48,29 @@ def test_entry_points_reject_bad_arguments_before_touching_the_gpu():
     assert lib.bw_qgemv(one, 0, 0, 128, 128, one, one, one, None, 16, 4, 32, one, 16, None) == -1
     # bf16 activations are not built
     assert lib.bw_qgemv(one, 1, 1, 128, 128, one, one, one, None, 16, 4, 32, one, 16, None) == -2
+    # split-K prefill: same checks as bw_qgemm, before the workspace is looked at
+    assert lib.bw_qgemm_ws(None, 0, 128, 128, 128, one, one, one, None, 16, 4, 32, one, 16, None, 0, None) == -1
+    assert lib.bw_qgemm_ws(one, 0, 128, 128, 64, one, one, one, None, 16, 4, 32, one, 16, None, 0, None) == -1
+    assert lib.bw_qgemm_ws(one, 1, 128, 128, 128, one, one, one, None, 16, 4, 32, one, 16, None, 0, None) == -2
+
+
+def test_split_k_workspace_size_is_a_pure_host_function():
+    from bitween_amd.kernels import hip_loader
+    lib = hip_loader.load()
+    ws = lib.bw_qgemm_workspace_bytes
+    # a grid of 128 x 256 tiles that fills the chip by itself needs no workspace
+    assert ws(2048, 14336, 4096, 4, 128) == 0
+    assert ws(4096, 4096, 4096, 4, 128) == 0
+    # few tiles and a long K: splits * M * N float32 partial sums, splits >= 2
+    for m, n, k, bits in ((128, 4096, 14336, 4), (512, 4096, 14336, 4), (128, 14336, 4096, 4), (64, 1024, 2048, 8)):
+        b = ws(m, n, k, bits, 128)
+        assert b % (m * n * 4) == 0 and b // (m * n * 4) >= 2
+        tiles = -(-n // 256) * -(-m // 128)
+        assert tiles * (b // (m * n * 4)) <= 256
+    # too short a K to split, invalid shapes, shapes the generic kernel takes
+    assert ws(128, 256, 128, 4, 128) == 0
+    assert ws(128, 256, 100, 4, 32) == 0
+    assert ws(128, 20, 96, 4, 48) == 0
 
 
 def test_host_layer_error_conventions_without_gpu():

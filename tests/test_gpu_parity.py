@@ -153,6 +153,42 @@ def test_gemm_vs_oracle(bits, g):
             check_matmul(y, x, qw, s16, z16, b16, bits, g)
 
 
+@pytest.mark.parametrize("bits,g,m,k,n", [(4, 128, 128, 14336, 512), (4, 64, 200, 4096, 768), (8, 128, 96, 4096, 300),
+                                          (2, 32, 128, 8192, 256), (4, 32, 17, 2048 + 128, 40)])
+def test_gemm_split_k_vs_unsplit_and_oracle(bits, g, m, k, n):
+    """bw_qgemm_ws through the C ABI: with a workspace K is cut into parallel slices, without one it is
+    bw_qgemm; both must meet the oracle, and a workspace that is too small is refused before any launch."""
+    import ctypes
+    from bitween_amd.kernels import hip_loader
+    lib = hip_loader.load()
+    _, qw, s16, z16, b16 = quantized_layer(n, k, bits, g, seed=m + k + n, outliers=True)
+    x = np.random.default_rng(k + m).standard_normal((m, k)).astype(np.float16)
+    d = [to_gpu(a) for a in (x, qw, s16, z16, b16)]
+    need = lib.bw_qgemm_workspace_bytes(m, n, k, bits, g)
+    assert need >= 2 * m * n * 4, "case is meant to split"
+    ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+    st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    def run(ws_ptr, ws_bytes, y):
+        return lib.bw_qgemm_ws(d[0].data_ptr(), 0, m, k, k, d[1].data_ptr(), d[2].data_ptr(), d[3].data_ptr(),
+                               d[4].data_ptr(), n, bits, g, y.data_ptr(), n, ws_ptr, ws_bytes, st)
+
+    y_split = torch.full((m, n), float("nan"), dtype=torch.float16, device="cuda")
+    y_plain = torch.full((m, n), float("nan"), dtype=torch.float16, device="cuda")
+    y_small = torch.full((m, n), 7.0, dtype=torch.float16, device="cuda")
+    assert run(ws.data_ptr(), need, y_split) == 0
+    assert run(None, 0, y_plain) == 0
+    assert run(ws.data_ptr(), need - 4, y_small) == -5          # BW_EWORKSPACE, nothing launched
+    assert run(ws.data_ptr() + 4, need, y_small) == -3          # BW_EALIGN
+    torch.cuda.synchronize()
+    assert (y_small == 7.0).all()
+    check_matmul(y_split, x, qw, s16, z16, b16, bits, g)
+    check_matmul(y_plain, x, qw, s16, z16, b16, bits, g)
+    # the two differ only in the float32 summation order
+    diff = (y_split.float() - y_plain.float()).abs().max().item()
+    assert diff <= 2.0 ** -9 * y_plain.float().abs().max().item()
+
+
 def test_reference_acceptance_recipe():
     """main.py:394-477: M=512, N=1024, K=2048, 8-bit g128, nn.Linear default init, mean-relative error < 1 %."""
     import bitween_amd
