@@ -217,6 +217,217 @@ __global__ __launch_bounds__((64 * GemvCfg<BITS, GROUP, MT>::MAX_WAVES)) void qg
     }
 }
 
+// ---- 4-bit, group 128, M <= 2: integer operands, zero point taken out of the inner loop ----------------
+//
+// A masked packed word is already a float16: bits 0-3 of a half are the subnormal q * 2^-24, bits 4-7 the
+// subnormal q * 2^-20, and the matrix core keeps subnormal inputs exactly.  So a word unpacks with one shift
+// and four ANDs, the products x * q are exact, and per group (= per chunk)
+//     sum_k x_k (q_k - z) = 2^24 * (E + O / 16) - z * S,     S = sum_k x_k,
+// with E and O the accumulators of the even and the odd nibbles.  S comes from the lanes that stage x (a
+// 16-lane reduction per chunk and row), so the inner loop holds no per-weight arithmetic at all; that
+// staging cost grows with M, which is why wider activation tiles stay on the kernel above.
+// Results agree with the per-weight float16 dequantisation to float32 rounding: a one-hot x still returns
+// the reference's W16 column bit for bit.
+BW_DEV float half_of(uint32_t word, int hi) {
+    return (float)__builtin_bit_cast(_Float16, (uint16_t)(hi ? word >> 16 : word));
+}
+
+BW_DEV float row16_sum(float v) {
+    // sum over the 16 lanes of a DPP row; every lane of the row ends up with the total
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true));
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, true));
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xF, 0xF, true));
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x140, 0xF, 0xF, true));
+    return v;
+}
+
+template <int MT, int KB>
+__global__ __launch_bounds__(1024) void qgemv_w4g128_kernel(const GemvArgs a) {
+    static_assert(MT == 1 || MT == 2 || MT == 4, "rows of one MFMA row quad");
+    constexpr int UPR = KB * 16;                          // 8-half units per activation row and round
+    constexpr int XL = (MT * UPR + 63) / 64;              // unit loads per lane and round
+    constexpr int ROW_BYTES = KB * 256 + 16, X_BYTES = MT * ROW_BYTES;
+    constexpr uint32_t kOob = 0x80000000u;
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nwaves = blockDim.x >> 6;
+    const int nl = lane & 15, kq = lane >> 4;
+    const int n0 = blockIdx.x * 16;
+    // LDS: [(scale, zero point) pairs, 16 rows x GP][x tile of wave 0] ... [x tile of wave n-1][partial sums]
+    const int gcols = (a.groups + 31) & ~31, GP = gcols + 1;     // odd pitch: the 16 rows hit different banks
+    uint32_t* meta = reinterpret_cast<uint32_t*>(smem);
+    char* after_meta = smem + ((16 * GP * 4 + 15) & ~15);
+    char* xs = after_meta + wave * X_BYTES;
+    float* red = reinterpret_cast<float*>(after_meta + nwaves * X_BYTES);
+    const __amdgpu_buffer_rsrc_t rw = make_rsrc(a.qweight, a.w_bytes), rx = make_rsrc(a.x, a.x_bytes),
+                                 rs = make_rsrc(a.scale, a.meta_bytes), rz = make_rsrc(a.zp, a.meta_bytes);
+
+    // scales / zero points of the 16 rows: thread e takes row (e / 32) % 16, column e % 32 + 32 * (e / 512)
+    const uint32_t meta_base = (uint32_t)n0 * a.groups * 2;
+    const int mr = (tid >> 5) & 15, mc = (tid & 31) + 32 * (tid >> 9);
+    uint32_t ms = 0, mz = 0;
+    if (mc < gcols) {
+        const uint32_t off = mc < a.groups ? meta_base + (mr * a.groups + mc) * 2 : kOob;
+        ms = __builtin_amdgcn_raw_buffer_load_b16(rs, off, 0, 0);
+        mz = __builtin_amdgcn_raw_buffer_load_b16(rz, off, 0, 0);
+    }
+
+    const uint32_t w_lane = (uint32_t)(n0 + nl) * a.row_bytes + kq * 16;
+    // where this lane's unit u = lane + 64 i of the round goes: row u / UPR, unit ku = u % UPR
+    uint32_t x_off[XL], x_dst[XL];
+#pragma unroll
+    for (int i = 0; i < XL; i++) {
+        const int u = lane + 64 * i, m = u / UPR, ku = u % UPR;
+        x_off[i] = m < a.M ? (uint32_t)(m * a.ldx + ku * 8) * 2 : kOob;
+        x_dst[i] = m * ROW_BYTES + (ku >> 2) * 64 + (ku & 3) * 8;
+    }
+    u4 xr[XL], wr[KB];
+    // Requests of a round: the weights, then x.  Every workgroup of the grid reads the same few KB of x at
+    // the same time and those hot lines come back late; loads return in order, so weights queued behind
+    // them would be held up too.  The unpack below needs only the weights and runs while x is on its way.
+    // x before the weights: loads return in order and the staging of x should overlap the weight stream
+    auto issue = [&](int c0) {
+#pragma unroll
+        for (int i = 0; i < XL; i++) {
+            const int ku = (lane + 64 * i) % UPR;
+            const uint32_t xo = (x_off[i] != kOob && c0 * 128 + ku * 8 < a.K) ? x_off[i] + c0 * 256 : kOob;
+            xr[i] = __builtin_amdgcn_raw_buffer_load_b128(rx, xo, 0, 0);
+        }
+        asm volatile("" ::: "memory");
+        const uint32_t off = c0 * 64 < a.row_bytes ? w_lane + c0 * 64 : kOob;
+#pragma unroll
+        for (int b = 0; b < KB; b++) wr[b] = __builtin_amdgcn_raw_buffer_load_b128(rw, off + b * 64, 0, 0);
+        asm volatile("" ::: "memory");
+    };
+    int c0 = wave * KB;
+    issue(c0);
+
+    if (mc < gcols) meta[mr * GP + mc] = ms | (mz << 16);
+    for (int e = tid + blockDim.x; e < 16 * gcols; e += blockDim.x) {   // more pairs than threads
+        const int r = (e >> 5) & 15, c = (e & 31) + 32 * (e >> 9);
+        const uint32_t off = c < a.groups ? meta_base + (r * a.groups + c) * 2 : kOob;
+        const uint32_t s2 = __builtin_amdgcn_raw_buffer_load_b16(rs, off, 0, 0);
+        const uint32_t z2 = __builtin_amdgcn_raw_buffer_load_b16(rz, off, 0, 0);
+        meta[r * GP + c] = s2 | (z2 << 16);
+    }
+    __syncthreads();
+
+    float acc[MT];
+#pragma unroll
+    for (int r = 0; r < MT; r++) acc[r] = 0.f;
+    const char* xrow = xs + (nl < MT ? nl : MT - 1) * ROW_BYTES + kq * 64;
+    const uint32_t* mrow = meta + nl * GP;
+    constexpr uint32_t kEven = 0x000F000Fu, kOdd = 0x00F000F0u;
+    while (true) {
+        // stage the round's activations: even-k quartets (x0,x4,x2,x6) and odd-k quartets (x1,x5,x3,x7) of
+        // every 8 values, in the order the masks below emit the nibbles; and -2^-24 * sum(x) per chunk
+        float nsum[XL];
+#pragma unroll
+        for (int i = 0; i < XL; i++) {
+            const u4 v = xr[i];
+            u2 ev, od;
+            ev[0] = __builtin_amdgcn_perm(v[2], v[0], 0x05040100u);
+            ev[1] = __builtin_amdgcn_perm(v[3], v[1], 0x05040100u);
+            od[0] = __builtin_amdgcn_perm(v[2], v[0], 0x07060302u);
+            od[1] = __builtin_amdgcn_perm(v[3], v[1], 0x07060302u);
+            if (MT * UPR >= 64 * (i + 1) || lane + 64 * i < MT * UPR) {
+                *reinterpret_cast<u2*>(xs + x_dst[i]) = ev;
+                *reinterpret_cast<u2*>(xs + x_dst[i] + 32) = od;
+            }
+            float t = 0.f;
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const h2 p = __builtin_bit_cast(h2, (uint32_t)v[j]);
+                t -= (float)p[0];
+                t -= (float)p[1];
+            }
+            nsum[i] = row16_sum(t) * 0x1p-24f;
+        }
+        __builtin_amdgcn_wave_barrier();
+        const uint32_t* mp = mrow + c0;
+#pragma unroll
+        for (int b = 0; b < KB; b++) {
+            const u4 w = wr[b];
+            u4 e0, e1, o0, o1;                            // B operands: even / odd nibbles of words 0,1 and 2,3
+#pragma unroll
+            for (int j = 0; j < 2; j++) {
+                const uint32_t wa = w[j], sa = wa >> 8, wb = w[2 + j], sb = wb >> 8;
+                e0[2 * j] = wa & kEven; e0[2 * j + 1] = sa & kEven;
+                o0[2 * j] = wa & kOdd;  o0[2 * j + 1] = sa & kOdd;
+                e1[2 * j] = wb & kEven; e1[2 * j + 1] = sb & kEven;
+                o1[2 * j] = wb & kOdd;  o1[2 * j + 1] = sb & kOdd;
+            }
+            const h8* xp = reinterpret_cast<const h8*>(xrow + b * 256);
+            f4 pe = {0.f, 0.f, 0.f, 0.f}, po = {0.f, 0.f, 0.f, 0.f};
+            pe = __builtin_amdgcn_mfma_f32_16x16x32_f16(xp[0], __builtin_bit_cast(h8, e0), pe, 0, 0, 0);
+            po = __builtin_amdgcn_mfma_f32_16x16x32_f16(xp[2], __builtin_bit_cast(h8, o0), po, 0, 0, 0);
+            pe = __builtin_amdgcn_mfma_f32_16x16x32_f16(xp[1], __builtin_bit_cast(h8, e1), pe, 0, 0, 0);
+            po = __builtin_amdgcn_mfma_f32_16x16x32_f16(xp[3], __builtin_bit_cast(h8, o1), po, 0, 0, 0);
+            const uint32_t sz = mp[b];
+            const float sf = half_of(sz, 0), zf = half_of(sz, 1);
+#pragma unroll
+            for (int r = 0; r < MT; r++) {
+                // unit (row r, chunk b) of the round was reduced in the DPP row that starts at lane u % 64 of load u / 64
+                const int u = r * UPR + 16 * b;
+                const float ns = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, nsum[u / 64]), u % 64));
+                const float t = __builtin_fmaf(po[r], 0.0625f, pe[r]);
+                acc[r] = __builtin_fmaf(sf, __builtin_fmaf(zf, ns, t), acc[r]);
+            }
+        }
+        c0 += nwaves * KB;
+        if (c0 >= a.nchunks) break;                       // wave-uniform
+        __builtin_amdgcn_wave_barrier();
+        issue(c0);
+    }
+
+    // acc[r] = 2^-24 * partial y[m = r][n = nl] in the lanes with kq == 0
+    if (kq == 0) {
+#pragma unroll
+        for (int r = 0; r < MT; r++) red[(wave * MT + r) * 16 + nl] = acc[r];
+    }
+    __syncthreads();
+    // one wave per output row: the four 16-lane quarters each add every fourth partial sum, then fold
+    for (int m = wave; m < MT; m += nwaves) {
+        float v = 0.f;
+        for (int w = kq; w < nwaves; w += 4) v += red[(w * MT + m) * 16 + nl];
+        v += __shfl_xor(v, 16);
+        v += __shfl_xor(v, 32);
+        const int n = n0 + nl;
+        if (kq == 0 && m < a.M && n < a.N) {
+            v *= 0x1p24f;
+            if (a.bias) v += (float)a.bias[n];
+            a.y[(int64_t)m * a.ldy + n] = (_Float16)v;
+        }
+    }
+}
+
+template <int MT, int KB>
+int launch_w4g128_kb(const GemvArgs& a, hipStream_t stream) {
+    int nwaves = (a.nchunks + KB - 1) / KB;
+    if (nwaves > 16) nwaves = 16;
+    const int gcols = (a.groups + 31) & ~31;
+    const size_t lds = (size_t)((16 * (gcols + 1) * 4 + 15) & ~15) + (size_t)nwaves * (MT * (KB * 256 + 16) + MT * 64);
+    auto kern = qgemv_w4g128_kernel<MT, KB>;
+    static bool attr_set = false;                          // per instantiation; benign if raced
+    if (lds > 64 * 1024 && !attr_set) {
+        if (lds > 150 * 1024) return BW_EUNSUPPORTED;
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) != hipSuccess)
+            return BW_ELAUNCH;
+        attr_set = true;
+    }
+    hipLaunchKernelGGL(kern, dim3((unsigned)((a.N + 15) / 16)), dim3(nwaves * 64), lds, stream, a);
+    return hipGetLastError() == hipSuccess ? BW_OK : BW_ELAUNCH;
+}
+
+template <int MT>
+int launch_w4g128(const GemvArgs& a, hipStream_t stream) {
+    static const int force_kb = getenv("BW_GEMV_KB") ? atoi(getenv("BW_GEMV_KB")) : 0;
+    int kb = (a.nchunks <= 32 && a.N <= 4096) ? 2 : 4;
+    if (force_kb) kb = force_kb;
+    if (kb >= 8) return launch_w4g128_kb<MT, 8>(a, stream);
+    if (kb >= 4) return launch_w4g128_kb<MT, 4>(a, stream);
+    return launch_w4g128_kb<MT, 2>(a, stream);
+}
+
 constexpr int kLdsBudget = 150 * 1024;
 
 template <int BITS, int GROUP, int MT, int KB>
@@ -261,6 +472,10 @@ int launch_gemv_mt(const GemvArgs& a, hipStream_t stream) {
 
 template <int BITS, int GROUP>
 int launch_gemv(const GemvArgs& a, hipStream_t stream) {
+    if constexpr (BITS == 4 && GROUP == 128) {
+        if (a.M == 1) return launch_w4g128<1>(a, stream);
+        if (a.M == 2) return launch_w4g128<2>(a, stream);
+    }
     if (a.M == 1) return launch_gemv_mt<BITS, GROUP, 1>(a, stream);
     if (a.M <= 4) return launch_gemv_mt<BITS, GROUP, 4>(a, stream);
     if (a.M <= 8) return launch_gemv_mt<BITS, GROUP, 8>(a, stream);
