@@ -98,6 +98,154 @@ def cpu_baseline(bits, g):
                       "oracle/rtn_oracle.c orc_qlinear_forward with OpenMP"}
 
 
+# ---- extras: every section takes (torch, hip, QuantizedLinear, layers) and returns a JSON-able dict; `layers`
+# are the headline's rotating W4 g128 layer copies --------------------------------------------------------------
+
+def extras_decode(torch, hip, QuantizedLinear, layers):
+    """Decode for every Llama-2-7B shape and M, rotating over the layer copies (graph replay, device time per call)."""
+    bits, g, out = 4, 128, {}
+    for idx, (name, k, n) in enumerate(LLAMA7B_LINEARS):
+        if name in ("k_proj", "v_proj", "o_proj", "up_proj"):
+            continue
+        for mm in (1, 2, 4, 8, 16):
+            x = torch.randn(mm, k, device="cuda", dtype=torch.float16)
+            calls = [lambda li=li: hip.quantized_gemv_hip(x, layers[li][idx].qweight, layers[li][idx].scale,
+                                                          layers[li][idx].zero_point, None, bits, g)
+                     for li in range(len(layers))]
+            reps = max(1, 96 // len(calls))                   # >= 96 launches per replay: graph launch cost amortised
+            gr = graph_of(torch, lambda: [c() for _ in range(reps) for c in calls])
+            us = time_calls(torch, gr.replay, 10, 2) / (reps * len(calls))
+            out[f"{name}_{k}x{n}_M{mm}"] = {"us": round(us, 2), "GBps": round(decode_bytes(mm, k, n, bits, g) / us / 1e3, 1)}
+    return out
+
+
+def extras_decode_hot(torch, hip, QuantizedLinear, layers):
+    """The same launches on one layer copy over and over: weights come from the 256 MiB Infinity Cache, not HBM."""
+    bits, g, out = 4, 128, {}
+    for idx, (name, k, n) in enumerate(LLAMA7B_LINEARS):
+        if name in ("k_proj", "v_proj", "o_proj", "up_proj"):
+            continue
+        x = torch.randn(1, k, device="cuda", dtype=torch.float16)
+        q = layers[0][idx]
+        gr = graph_of(torch, lambda: [hip.quantized_gemv_hip(x, q.qweight, q.scale, q.zero_point, None, bits, g) for _ in range(96)])
+        us = time_calls(torch, gr.replay, 10, 2) / 96
+        out[f"{name}_{k}x{n}_M1"] = {"us": round(us, 2), "GBps": round(decode_bytes(1, k, n, bits, g) / us / 1e3, 1)}
+    return out
+
+
+def extras_decode_other_formats(torch, hip, QuantizedLinear, layers):
+    """K=4096 -> N=11008 at 8-bit g128, 4-bit g64, 2-bit g32 (weights with 0.1 % outliers x10), M = 1 and 16."""
+    k, n, out = 4096, 11008, {}
+    for bits, g in ((8, 128), (4, 64), (2, 32)):
+        copies = 16 if bits < 8 else 8                          # > 256 MiB of packed weights in rotation
+        qs = [make_layer(torch, QuantizedLinear, k, n, bits, g, seed=31 * bits + i, outliers=True) for i in range(copies)]
+        for mm in (1, 16):
+            x = torch.randn(mm, k, device="cuda", dtype=torch.float16)
+            reps = 96 // copies
+            gr = graph_of(torch, lambda: [hip.quantized_gemv_hip(x, q.qweight, q.scale, q.zero_point, None, bits, g)
+                                          for _ in range(reps) for q in qs])
+            us = time_calls(torch, gr.replay, 10, 2) / (reps * copies)
+            out[f"w{bits}g{g}_{k}x{n}_M{mm}"] = {"us": round(us, 2), "GBps": round(decode_bytes(mm, k, n, bits, g) / us / 1e3, 1)}
+        del qs
+    return out
+
+
+def extras_hipblaslt_decode(torch, hip, QuantizedLinear, layers):
+    """Same-run fp16 hipBLASLt GEMV on dequantised weights (reads 4x the bytes)."""
+    out = {}
+    for name, k, n in (("q_proj", 4096, 4096), ("gate_proj", 4096, 11008)):
+        ws = [torch.randn(n, k, device="cuda", dtype=torch.float16) for _ in range(12)]
+        x = torch.randn(1, k, device="cuda", dtype=torch.float16)
+        gr = graph_of(torch, lambda: [torch.matmul(x, w.T) for _ in range(8) for w in ws])
+        us = time_calls(torch, gr.replay, 10, 2) / (8 * len(ws))
+        out[f"{name}_{k}x{n}_M1"] = {"us": round(us, 2), "fp16_GBps": round(2 * n * k / us / 1e3, 1)}
+        del ws
+    return out
+
+
+def extras_prefill(torch, hip, QuantizedLinear, layers):
+    """Prefill on the Llama-3-8B MLP shapes, W4 g128, next to fp16 hipBLASLt on the dequantised weights."""
+    bits, g, out = 4, 128, {}
+    for k, n in ((4096, 14336), (14336, 4096)):
+        q = make_layer(torch, QuantizedLinear, k, n, bits, g, seed=7)
+        w16 = hip.dequantize(q.qweight, q.scale, q.zero_point, g, bits, torch.float16)
+        for mm in (128, 512, 2048):
+            x = torch.randn(mm, k, device="cuda", dtype=torch.float16)
+            us_q = time_calls(torch, lambda: hip.quantized_gemm_hip(x, q.qweight, q.scale, q.zero_point, None, bits, g), 20, 5)
+            us_b = time_calls(torch, lambda: torch.matmul(x, w16.T), 20, 5)
+            fl = 2.0 * mm * n * k
+            out[f"{k}x{n}_M{mm}"] = {"us": round(us_q, 1), "TFLOPs": round(fl / us_q / 1e6, 1),
+                                     "pct_mfma_f16_peak": round(100 * fl / us_q / 1e6 / MFMA_F16_PEAK_TFLOPS, 1),
+                                     "hipblaslt_fp16_us": round(us_b, 1), "hipblaslt_fp16_TFLOPs": round(fl / us_b / 1e6, 1),
+                                     "frac_of_hipblaslt": round(us_b / us_q, 3)}
+        del q, w16
+    return out
+
+
+def extras_quantize(torch, hip, QuantizedLinear, layers):
+    """Quantiser: fp16 weights in, packed words + fp16 scale / zero point out (the from_float path)."""
+    out = {}
+    for bits, g in ((4, 128), (8, 128), (2, 32)):
+        k, n = 4096, 11008
+        ws = [(torch.randn(n, k, device="cuda") * 0.02).half() for _ in range(6)]
+        it = iter(range(10 ** 9))
+        us = time_calls(torch, lambda: hip.quantize_pack(ws[next(it) % 6], bits, g, torch.float32, torch.float16, torch.float16), 30, 6)
+        by = n * k * (2 + bits / 8 + 4 / g)
+        out[f"w{bits}g{g}_{k}x{n}_f16_in"] = {"us": round(us, 1), "GBps": round(by / us / 1e3, 1),
+                                             "pct_hbm_peak": round(100 * by / us / 1e3 / HBM_PEAK_GBPS, 1),
+                                             "Gweights_per_s": round(n * k / us / 1e3, 1)}
+        del ws
+    return out
+
+
+def extras_mixed_precision_model(torch, hip, QuantizedLinear, layers):
+    """The linears of a 32-layer, hidden-4096, MLP-11008 decoder with the mixed recipe: attention 8-bit g128,
+    gate/up/down 4-bit g128, down_proj of layers 0, 1, 30, 31 2-bit g32.  Reports the time to quantise all of
+    them (fp16 in) and the time of one decode token through all of them (M = 1, one HIP graph, nothing but the
+    quantised linears: no attention, norms, embeddings or lm_head), next to fp16 hipBLASLt on the same shapes."""
+    nlayers, low = 32, (0, 1, 30, 31)
+    gen = torch.Generator(device="cuda").manual_seed(5)
+    src = {(k, n): (torch.randn(n, k, device="cuda", generator=gen) * 0.02).half() for _, k, n in LLAMA7B_LINEARS[3:]}
+    plan = []
+    for li in range(nlayers):
+        for name, k, n in LLAMA7B_LINEARS:
+            if name in ("q_proj", "k_proj", "v_proj", "o_proj"):
+                plan.append((k, n, 8, 128))
+            elif name == "down_proj" and li in low:
+                plan.append((k, n, 2, 32))
+            else:
+                plan.append((k, n, 4, 128))
+    # quantise: one launch per linear, same random source per shape (the values do not change the timing)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    packed = [hip.quantize_pack(src[(k, n)], b, g, torch.float32, torch.float16, torch.float16) for k, n, b, g in plan]
+    e1.record()
+    torch.cuda.synchronize()
+    quant_ms = e0.elapsed_time(e1)
+    weights = sum(k * n for k, n, _, _ in plan)
+    xs = {k: torch.randn(1, k, device="cuda", dtype=torch.float16) for k in (4096, 11008)}
+    gr = graph_of(torch, lambda: [hip.quantized_gemv_hip(xs[k], qw, s, z, None, b, g)
+                                  for (k, n, b, g), (qw, s, z) in zip(plan, packed)])
+    tok_us = time_calls(torch, gr.replay, 20, 3)
+    by = sum(decode_bytes(1, k, n, b, g) for k, n, b, g in plan)
+    del gr
+    # fp16 hipBLASLt over the same shapes: one set of fp16 weights per layer would be 13 GB; rotate 4 layers' worth
+    w16 = [[torch.randn(n, k, device="cuda", dtype=torch.float16) for _, k, n in LLAMA7B_LINEARS] for _ in range(4)]
+    gr = graph_of(torch, lambda: [torch.matmul(xs[w.shape[1]], w.T) for li in range(nlayers) for w in w16[li % 4]])
+    blas_us = time_calls(torch, gr.replay, 10, 2)
+    return {"linears": len(plan), "weights_G": round(weights / 1e9, 3), "quantize_all_ms": round(quant_ms, 2),
+            "quantize_Gweights_per_s": round(weights / quant_ms / 1e6, 1),
+            "decode_token_us_linears_only": round(tok_us, 1), "decode_tokens_per_s_linears_only": round(1e6 / tok_us, 1),
+            "decode_GBps": round(by / tok_us / 1e3, 1), "decode_bytes_per_token": by,
+            "hipblaslt_fp16_token_us_linears_only": round(blas_us, 1)}
+
+
+EXTRAS = {"decode": extras_decode, "decode_infinity_cache_hot": extras_decode_hot,
+          "decode_other_formats": extras_decode_other_formats, "hipblaslt_fp16_decode": extras_hipblaslt_decode,
+          "prefill": extras_prefill, "quantize": extras_quantize, "mixed_precision_model": extras_mixed_precision_model}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -108,6 +256,8 @@ def main():
     ap.add_argument("--no-graph", action="store_true")
     ap.add_argument("--no-extras", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--only", choices=sorted(EXTRAS), default=None,
+                    help="run just this section of the extras and print it (used for profiling one kernel)")
     ap.add_argument("--copy-probe", action="store_true",
                     help="run only a plain 256 MiB device copy a few times (calibrates rocprof FETCH_SIZE/WRITE_SIZE)")
     args = ap.parse_args()
@@ -134,6 +284,9 @@ def main():
 
     layers = [[make_layer(torch, QuantizedLinear, k, n, bits, g, seed=100 * li + i)
                for i, (_, k, n) in enumerate(LLAMA7B_LINEARS)] for li in range(args.layers)]
+    if args.only:
+        print(json.dumps({args.only: EXTRAS[args.only](torch, hip, QuantizedLinear, layers)}))
+        return
     xs = {k: torch.randn(m, k, device="cuda", dtype=torch.float16) for k in (4096, 11008)}
     step_bytes = sum(decode_bytes(m, k, n, bits, g) for _, k, n in LLAMA7B_LINEARS)
     launches_per_step = len(LLAMA7B_LINEARS)
@@ -142,6 +295,7 @@ def main():
         for q in layers[li]:
             hip.quantized_gemv_hip(xs[q.in_features], q.qweight, q.scale, q.zero_point, None, bits, g)
 
+    per_layer_graphs = None
     if args.no_graph:
         def do_steps(first, count):
             for s in range(first, first + count):
@@ -149,6 +303,7 @@ def main():
     else:
         per_layer = [graph_of(torch, lambda li=li: run_layer(li)) for li in range(args.layers)]
         full = graph_of(torch, lambda: [run_layer(li) for li in range(args.layers)])
+        per_layer_graphs = (per_layer, full)
 
         def do_steps(first, count):
             s = first
@@ -199,57 +354,8 @@ def main():
     }
 
     if not args.no_extras:
-        extras = {}
-        # decode, every shape and M, rotating over the layer copies (eager launches, device time per call)
-        dec = {}
-        for idx, (name, k, n) in enumerate(LLAMA7B_LINEARS):
-            if name in ("k_proj", "v_proj", "o_proj", "up_proj"):
-                continue
-            for mm in (1, 4, 8, 16):
-                x = torch.randn(mm, k, device="cuda", dtype=torch.float16)
-                calls = [lambda li=li: hip.quantized_gemv_hip(x, layers[li][idx].qweight, layers[li][idx].scale,
-                                                              layers[li][idx].zero_point, None, bits, g)
-                         for li in range(args.layers)]
-                gr = graph_of(torch, lambda: [c() for c in calls])
-                us = time_calls(torch, gr.replay, 20, 3) / args.layers
-                dec[f"{name}_{k}x{n}_M{mm}"] = {"us": round(us, 2),
-                                               "GBps": round(decode_bytes(mm, k, n, bits, g) / us / 1e3, 1)}
-        extras["decode"] = dec
-        # same-run fp16 hipBLASLt GEMV on dequantised weights (reads 4x the bytes)
-        blas = {}
-        for name, k, n in (("q_proj", 4096, 4096), ("gate_proj", 4096, 11008)):
-            ws = [torch.randn(n, k, device="cuda", dtype=torch.float16) for _ in range(12)]
-            x = torch.randn(1, k, device="cuda", dtype=torch.float16)
-            gr = graph_of(torch, lambda: [torch.matmul(x, w.T) for w in ws])
-            us = time_calls(torch, gr.replay, 20, 3) / len(ws)
-            blas[f"{name}_{k}x{n}_M1"] = {"us": round(us, 2), "fp16_GBps": round(2 * n * k / us / 1e3, 1)}
-            del ws
-        extras["hipblaslt_fp16_decode"] = blas
-        # prefill: Llama-3-8B MLP shapes
-        pre = {}
-        for k, n in ((4096, 14336), (14336, 4096)):
-            q = make_layer(torch, QuantizedLinear, k, n, bits, g, seed=7)
-            w16 = hip.dequantize(q.qweight, q.scale, q.zero_point, g, bits, torch.float16)
-            for mm in (128, 512, 2048):
-                x = torch.randn(mm, k, device="cuda", dtype=torch.float16)
-                us_q = time_calls(torch, lambda: hip.quantized_gemm_hip(x, q.qweight, q.scale, q.zero_point, None, bits, g), 20, 5)
-                us_b = time_calls(torch, lambda: torch.matmul(x, w16.T), 20, 5)
-                fl = 2.0 * mm * n * k
-                pre[f"{k}x{n}_M{mm}"] = {"us": round(us_q, 1), "TFLOPs": round(fl / us_q / 1e6, 1),
-                                         "hipblaslt_fp16_us": round(us_b, 1), "hipblaslt_fp16_TFLOPs": round(fl / us_b / 1e6, 1),
-                                         "frac_of_hipblaslt": round(us_b / us_q, 3)}
-            del q, w16
-        extras["prefill"] = pre
-        # quantiser: fp16 weights in, packed + fp16 scale/zp out
-        qz = {}
-        for k, n in ((4096, 11008),):
-            ws = [(torch.randn(n, k, device="cuda") * 0.02).half() for _ in range(6)]
-            it = iter(range(10 ** 9))
-            us = time_calls(torch, lambda: hip.quantize_pack(ws[next(it) % 6], bits, g, torch.float32, torch.float16, torch.float16), 30, 6)
-            by = n * k * (2 + bits / 8 + 4 / g)
-            qz[f"{k}x{n}_f16_in"] = {"us": round(us, 1), "GBps": round(by / us / 1e3, 1), "Gweights_per_s": round(n * k / us / 1e3, 1)}
-        extras["quantize"] = qz
-        result["extras"] = extras
+        del per_layer_graphs
+        result["extras"] = {name: fn(torch, hip, QuantizedLinear, layers) for name, fn in EXTRAS.items()}
 
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(bits, g)
