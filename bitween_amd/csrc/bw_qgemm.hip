@@ -428,18 +428,33 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
     }
 }
 
-// y[m][n] = fp16( sum_z ws[z][m][n] + bias[n] )
+// y[m][n] = fp16( sum_z ws[z][m][n] + bias[n] ); VEC consecutive n per thread (VEC = 4 needs N % 4 == 0)
+template <int VEC>
 __global__ __launch_bounds__(256) void qgemm_reduce_kernel(const float* __restrict__ ws, int splits, int M, int N,
                                                            const _Float16* __restrict__ bias, _Float16* __restrict__ y,
                                                            int ldy) {
-    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t idx = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * VEC;
     const int64_t total = (int64_t)M * N;
     if (idx >= total) return;
-    float v = 0.f;
-    for (int z = 0; z < splits; z++) v += ws[z * total + idx];
     const int m = (int)(idx / N), n = (int)(idx - (int64_t)m * N);
-    if (bias) v += (float)bias[n];
-    y[(int64_t)m * ldy + n] = (_Float16)v;
+    float v[VEC];
+#pragma unroll
+    for (int i = 0; i < VEC; i++) v[i] = 0.f;
+    for (int z = 0; z < splits; z++) {
+        if constexpr (VEC == 4) {
+            const f4 t = *reinterpret_cast<const f4*>(ws + z * total + idx);
+#pragma unroll
+            for (int i = 0; i < 4; i++) v[i] += t[i];
+        } else {
+            v[0] += ws[z * total + idx];
+        }
+    }
+    _Float16* dst = y + (int64_t)m * ldy + n;
+#pragma unroll
+    for (int i = 0; i < VEC; i++) {
+        if (bias) v[i] += (float)bias[n + i];
+        dst[i] = (_Float16)v[i];
+    }
 }
 
 // How many z-slices to cut K into.  One workgroup fits per CU, so the grid runs in waves of 256 workgroups:
@@ -474,8 +489,12 @@ int launch_gemm(GemmArgs a, void* workspace, size_t workspace_bytes, hipStream_t
     if (hipGetLastError() != hipSuccess) return BW_ELAUNCH;
     if (splits > 1) {
         const int64_t total = (int64_t)a.M * a.N;
-        hipLaunchKernelGGL(qgemm_reduce_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, a.ws, splits,
-                           a.M, a.N, a.bias, a.y, a.ldy);
+        if (a.N % 4 == 0)
+            hipLaunchKernelGGL(qgemm_reduce_kernel<4>, dim3((unsigned)((total / 4 + 255) / 256)), dim3(256), 0, stream, a.ws,
+                               splits, a.M, a.N, a.bias, a.y, a.ldy);
+        else
+            hipLaunchKernelGGL(qgemm_reduce_kernel<1>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, a.ws,
+                               splits, a.M, a.N, a.bias, a.y, a.ldy);
         if (hipGetLastError() != hipSuccess) return BW_ELAUNCH;
     }
     return BW_OK;
