@@ -191,8 +191,10 @@ def extras_quantize(torch, hip, QuantizedLinear, layers):
     for bits, g in ((4, 128), (8, 128), (2, 32)):
         k, n = 4096, 11008
         ws = [(torch.randn(n, k, device="cuda") * 0.02).half() for _ in range(6)]
-        it = iter(range(10 ** 9))
-        us = time_calls(torch, lambda: hip.quantize_pack(ws[next(it) % 6], bits, g, torch.float32, torch.float16, torch.float16), 30, 6)
+        # graph replay: the Python call (three output allocations, ctypes) costs as much as the kernel
+        gr = graph_of(torch, lambda: [hip.quantize_pack(w, bits, g, torch.float32, torch.float16, torch.float16)
+                                      for _ in range(4) for w in ws])
+        us = time_calls(torch, gr.replay, 10, 2) / 24
         by = n * k * (2 + bits / 8 + 4 / g)
         out[f"w{bits}g{g}_{k}x{n}_f16_in"] = {"us": round(us, 1), "GBps": round(by / us / 1e3, 1),
                                              "pct_hbm_peak": round(100 * by / us / 1e3 / HBM_PEAK_GBPS, 1),

@@ -1,16 +1,16 @@
 // RTN per-group quantise + pack, and the stand-alone dequantise.
 //
 // bw_quantize_pack restates bitween/functional.py:3-45 as ONE kernel: a
-// thread owns one packed output word (32/bits consecutive weights), the
-// group/(32/bits) threads of a group agree on min and max with cross-lane
-// shuffles, and every thread then forms scale, zero point and its own
-// quantised values with the same sequence of correctly rounded IEEE
-// operations eager torch performs: (max-min)/Qmax, clamp(1e-8), -min/scale,
-// round-half-even, clamp; then w/scale, a separate add of the zero point,
-// round-half-even, clamp.  Divisions are true IEEE divisions (x/15 differs
-// from x*(1/15)), nothing is contracted into FMAs, denormals are kept.
+// thread owns a few packed output words, the threads of a group agree on min
+// and max with cross-lane shuffles, and every thread then forms scale, zero
+// point and its own quantised values with the results of the same sequence
+// of correctly rounded IEEE operations eager torch performs: (max-min)/Qmax,
+// clamp(1e-8), -min/scale, round-half-even, clamp; then w/scale, a separate
+// add of the zero point, round-half-even, clamp.  Divisions are true IEEE
+// divisions (x/15 differs from x*(1/15)) or provably give the same rounded
+// integer, nothing else is contracted into FMAs, denormals are kept.
 // The weights are read once (2 or 4 bytes each) and bits/8 + 4/group bytes are
-// written: HBM-bound, with the divide sequence as the ALU cost.
+// written: HBM-bound.
 #include "bw_common.h"
 
 namespace {
@@ -60,81 +60,136 @@ BW_DEV void load_vals(const void* w, int64_t off, float* v) {
     }
 }
 
-// One thread per packed word; LPG = group / VPI threads (a power of two <= 64,
-// aligned inside the wave) cooperate on one group.
-template <int BITS, int WDT, int MATH>
+// scale and zero point of one group from its extrema, exactly as functional.py:25-26
+template <int MATH>
+BW_DEV void group_params(float lo, float hi, float qmax, float& s, float& zf) {
+    s = rnd<MATH>(__fdiv_rn(rnd<MATH>(__fsub_rn(hi, lo)), qmax));
+    s = fmaxf(s, rnd<MATH>(1e-8f));
+    zf = rintf(rnd<MATH>(__fdiv_rn(-lo, s)));
+    zf = fminf(fmaxf(zf, 0.f), qmax);
+}
+
+// round(w / s + zf) before the clamp, exactly as functional.py:29: an IEEE divide, then a separate add
+template <int MATH>
+BW_DEV float quant_exact(float w, float s, float zf) {
+    return rintf(rnd<MATH>(__fadd_rn(rnd<MATH>(__fdiv_rn(w, s)), zf)));
+}
+
+// A thread owns WPT consecutive packed words (VPT = WPT * 32/bits weights, 32 bytes of 16-bit input where
+// the shape allows); the lpg = group / VPT threads of a group (a power of two <= 64, aligned inside the
+// wave) agree on min and max with cross-lane shuffles.
+//
+// float32 math takes a short cut that cannot change a result: q1 = fma(w - q0 s, r, q0) with q0 = w r and
+// r = 1/s refined once is within one ulp of the correctly rounded w / s, and for |q1| < 1024 the sum
+// t = q1 + zf is then within 2^-12 of what the exact quotient gives.  Unless t lies within 2^-11 of a
+// half-integer, round(t) is therefore the reference's value; the rare elements that do (and anything
+// large, infinite or NaN) are redone with the true IEEE divide.
+template <int BITS, int WDT, int MATH, int WPT>
 __global__ __launch_bounds__(256) void quantize_pack_kernel(const void* __restrict__ w, int64_t N, int K, int64_t ldw,
                                                             int group, int lpg, int32_t* __restrict__ qweight,
                                                             void* __restrict__ scale, int scale_dtype,
                                                             void* __restrict__ zp, int zp_dtype) {
-    constexpr int VPI = 32 / BITS;
+    constexpr int VPI = 32 / BITS, VPT = VPI * WPT;
     constexpr float QMAX = (float)((1 << BITS) - 1);
-    const int words = K / VPI;
-    const int64_t total = N * (int64_t)words;
-    int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    const bool live = idx < total;
-    if (!live) idx = total - 1;          // keep the whole wave in the shuffles; stores are masked
-    const int64_t row = idx / words;
-    const int wcol = (int)(idx - row * words);
-    float v[VPI];
-    load_vals<WDT, VPI>(w, row * ldw + (int64_t)wcol * VPI, v);
-    float lo = v[0], hi = v[0];
+    const int tpr = K / VPT;                             // threads per row; grid.x covers them, grid.y the rows
+    int tcol = (int)(blockIdx.x * blockDim.x + threadIdx.x);
+    const bool live = tcol < tpr;
+    if (!live) tcol = tpr - 1;           // keep the whole wave in the shuffles; stores are masked
+    const int groups = K / group;
+    for (int64_t row = blockIdx.y; row < N; row += gridDim.y) {
+        float v[VPT];
+        load_vals<WDT, VPT>(w, row * ldw + (int64_t)tcol * VPT, v);
 #pragma unroll
-    for (int i = 0; i < VPI; i++) { v[i] = rnd<MATH>(v[i]); }
-    lo = hi = v[0];
+        for (int i = 0; i < VPT; i++) { v[i] = rnd<MATH>(v[i]); }
+        float lo = v[0], hi = v[0];
 #pragma unroll
-    for (int i = 1; i < VPI; i++) { lo = fminf(lo, v[i]); hi = fmaxf(hi, v[i]); }
-    for (int d = 1; d < lpg; d <<= 1) {
-        lo = fminf(lo, __shfl_xor(lo, d));
-        hi = fmaxf(hi, __shfl_xor(hi, d));
-    }
-    float s = rnd<MATH>(__fdiv_rn(rnd<MATH>(__fsub_rn(hi, lo)), QMAX));          // functional.py:25
-    s = fmaxf(s, rnd<MATH>(1e-8f));
-    float zf = rintf(rnd<MATH>(__fdiv_rn(-lo, s)));                                // functional.py:26
-    zf = fminf(fmaxf(zf, 0.f), QMAX);
-    uint32_t word = 0;
+        for (int i = 1; i < VPT; i++) { lo = fminf(lo, v[i]); hi = fmaxf(hi, v[i]); }
+        for (int d = 1; d < lpg; d <<= 1) {
+            lo = fminf(lo, __shfl_xor(lo, d));
+            hi = fmaxf(hi, __shfl_xor(hi, d));
+        }
+        float s, zf;
+        group_params<MATH>(lo, hi, QMAX, s, zf);
+        float t[VPT];
+        if constexpr (MATH == BW_F32) {
+            const float r0 = __builtin_amdgcn_rcpf(s);
+            const float r = __builtin_fmaf(__builtin_fmaf(-s, r0, 1.0f), r0, r0);
 #pragma unroll
-    for (int i = 0; i < VPI; i++) {
-        float t = rnd<MATH>(__fdiv_rn(v[i], s));                                   // functional.py:29: divide,
-        t = rnd<MATH>(__fadd_rn(t, zf));                                           // then a separate add
-        t = fminf(fmaxf(rintf(t), 0.f), QMAX);
-        word |= (uint32_t)(int)t << (i * BITS);
-    }
-    if (live) {
-        qweight[idx] = (int32_t)word;
-        const int k = wcol * VPI;
-        if (k % group == 0) {
-            const int64_t gi = row * (K / group) + k / group;
-            store_meta(scale, scale_dtype, gi, s);
-            store_meta(zp, zp_dtype, gi, zf);
+            for (int i = 0; i < VPT; i++) {
+                const float q0 = __fmul_rn(v[i], r);
+                const float q1 = __builtin_fmaf(__builtin_fmaf(-q0, s, v[i]), r, q0);
+                const float sum = __fadd_rn(q1, zf);
+                t[i] = rintf(sum);
+                // far from a tie (a huge |q1| has no fraction and clamps the same either way; NaN fails the test)
+                if (!(fabsf(__fsub_rn(sum, t[i])) < 0.5f - 0x1p-11f)) t[i] = quant_exact<MATH>(v[i], s, zf);
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < VPT; i++) t[i] = quant_exact<MATH>(v[i], s, zf);
+        }
+        // pack: the clamped values are small integers, so 16 bits' worth of fields add up exactly in float32
+        constexpr int FPH = 16 / BITS;                    // fields per 16-bit half word
+        uint32_t word[WPT];
+#pragma unroll
+        for (int j = 0; j < WPT; j++) {
+            float half[2] = {0.f, 0.f};
+#pragma unroll
+            for (int i = 0; i < VPI; i++)
+                half[i / FPH] = __builtin_fmaf(fminf(fmaxf(t[j * VPI + i], 0.f), QMAX), (float)(1 << ((i % FPH) * BITS)), half[i / FPH]);
+            word[j] = (uint32_t)half[0] | ((uint32_t)half[1] << 16);
+        }
+        if (live) {
+            uint32_t* dst = reinterpret_cast<uint32_t*>(qweight) + (row * tpr + tcol) * WPT;
+            if constexpr (WPT == 4) *reinterpret_cast<u4*>(dst) = u4{word[0], word[1], word[2], word[3]};
+            else if constexpr (WPT == 2) *reinterpret_cast<u2*>(dst) = u2{word[0], word[1]};
+            else dst[0] = word[0];
+            const int k = tcol * VPT;
+            if (k % group == 0) {
+                const int64_t gi = row * groups + k / group;
+                store_meta(scale, scale_dtype, gi, s);
+                store_meta(zp, zp_dtype, gi, zf);
+            }
         }
     }
 }
 
-// Any group size (including ones that are not a power-of-two multiple of the
-// word width): one thread per group, two passes over its values.
+// Any group size: one thread per packed word, which scans the whole group of each of its values for the
+// extrema (re-using them while consecutive values share a group).  Slow, exact, no scratch memory.
 template <int WDT, int MATH>
-__global__ void quantize_group_generic_kernel(const void* __restrict__ w, int64_t N, int K, int64_t ldw, int bits, int group,
-                                              uint8_t* __restrict__ qtmp, void* __restrict__ scale, int scale_dtype,
-                                              void* __restrict__ zp, int zp_dtype) {
-    const int groups = K / group;
-    const int64_t gi = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (gi >= N * groups) return;
-    const int64_t row = gi / groups;
-    const int64_t base = row * ldw + (gi - row * groups) * group;
+__global__ __launch_bounds__(256) void quantize_pack_generic_kernel(const void* __restrict__ w, int64_t N, int K, int64_t ldw,
+                                                                    int bits, int group, int32_t* __restrict__ qweight,
+                                                                    void* __restrict__ scale, int scale_dtype,
+                                                                    void* __restrict__ zp, int zp_dtype) {
+    const int vpi = 32 / bits, words = K / vpi, groups = K / group;
     const float qmax = (float)((1 << bits) - 1);
-    float lo = rnd<MATH>(Elem<WDT>::load(w, base)), hi = lo;
-    for (int i = 1; i < group; i++) { const float t = rnd<MATH>(Elem<WDT>::load(w, base + i)); lo = fminf(lo, t); hi = fmaxf(hi, t); }
-    float s = rnd<MATH>(__fdiv_rn(rnd<MATH>(__fsub_rn(hi, lo)), qmax));
-    s = fmaxf(s, rnd<MATH>(1e-8f));
-    float zf = fminf(fmaxf(rintf(rnd<MATH>(__fdiv_rn(-lo, s))), 0.f), qmax);
-    store_meta(scale, scale_dtype, gi, s);
-    store_meta(zp, zp_dtype, gi, zf);
-    for (int i = 0; i < group; i++) {
-        float t = rnd<MATH>(__fdiv_rn(rnd<MATH>(Elem<WDT>::load(w, base + i)), s));
-        t = rnd<MATH>(__fadd_rn(t, zf));
-        qtmp[row * K + (gi - row * groups) * group + i] = (uint8_t)(int)fminf(fmaxf(rintf(t), 0.f), qmax);
+    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= N * (int64_t)words) return;
+    const int64_t row = idx / words;
+    const int wcol = (int)(idx - row * words);
+    uint32_t word = 0;
+    int gprev = -1;
+    float s = 0.f, zf = 0.f;
+    for (int i = 0; i < vpi; i++) {
+        const int k = wcol * vpi + i, g = k / group;
+        if (g != gprev) {
+            const int64_t base = row * ldw + (int64_t)g * group;
+            float lo = rnd<MATH>(Elem<WDT>::load(w, base)), hi = lo;
+            for (int e = 1; e < group; e++) {
+                const float x = rnd<MATH>(Elem<WDT>::load(w, base + e));
+                lo = fminf(lo, x);
+                hi = fmaxf(hi, x);
+            }
+            group_params<MATH>(lo, hi, qmax, s, zf);
+            gprev = g;
+            if (k == g * group) {                        // the thread holding a group's first value stores its parameters
+                store_meta(scale, scale_dtype, row * groups + g, s);
+                store_meta(zp, zp_dtype, row * groups + g, zf);
+            }
+        }
+        const float t = quant_exact<MATH>(rnd<MATH>(Elem<WDT>::load(w, row * ldw + k)), s, zf);
+        word |= (uint32_t)(int)fminf(fmaxf(t, 0.f), qmax) << (i * bits);
     }
+    qweight[idx] = (int32_t)word;
 }
 
 // out[n][k] = scale * (q - zp): float32 product, rounded once to the output type.
@@ -177,22 +232,54 @@ __global__ __launch_bounds__(256) void dequantize_kernel(const uint32_t* __restr
     }
 }
 
-template <int BITS, int WDT, int MATH>
+// Can a launch with WPT words per thread take this shape?  Vector loads / stores need their alignment, the
+// threads of a group must be a power of two inside one wave.
+template <int BITS, int WDT, int WPT>
+bool quantize_fits(const void* w, int64_t K, int64_t ldw, int group, const void* qweight) {
+    constexpr int VPT = 32 / BITS * WPT;
+    constexpr size_t esz = WDT == BW_F32 ? 4 : 2;
+    constexpr size_t need = (VPT * esz >= 16) ? 16 : VPT * esz;
+    const int lpg = group / VPT;
+    return group % VPT == 0 && K % VPT == 0 && lpg >= 1 && lpg <= 64 && (lpg & (lpg - 1)) == 0 && bw_aligned(w, need) &&
+           (ldw * esz) % need == 0 && bw_aligned(qweight, 4 * WPT);
+}
+
+template <int BITS, int WDT, int MATH, int WPT>
 int launch_quantize(const void* w, int64_t N, int64_t K, int64_t ldw, int group, int32_t* qweight, void* scale, int sdt,
                     void* zp, int zdt, hipStream_t st) {
-    const int vpi = 32 / BITS;
-    const int64_t total = N * (K / vpi);
-    hipLaunchKernelGGL((quantize_pack_kernel<BITS, WDT, MATH>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, w, N,
-                       (int)K, ldw, group, group / vpi, qweight, scale, sdt, zp, zdt);
+    constexpr int VPT = 32 / BITS * WPT;
+    const int tpr = (int)(K / VPT);
+    const int block = tpr >= 256 ? 256 : ((tpr + 63) / 64) * 64;
+    dim3 grid((unsigned)((tpr + block - 1) / block), (unsigned)(N < 65535 ? N : 65535));
+    hipLaunchKernelGGL((quantize_pack_kernel<BITS, WDT, MATH, WPT>), grid, dim3(block), 0, st, w, N, (int)K, ldw, group,
+                       group / VPT, qweight, scale, sdt, zp, zdt);
+    return hipGetLastError() == hipSuccess ? BW_OK : BW_ELAUNCH;
+}
+
+template <int BITS, int WDT, int MATH>
+int launch_quantize_bits(const void* w, int64_t N, int64_t K, int64_t ldw, int group, int32_t* qweight, void* scale, int sdt,
+                         void* zp, int zdt, hipStream_t st) {
+    // 32 bytes of input per thread where the shape allows, else one word per thread, else the generic kernel
+    constexpr int VPI = 32 / BITS;
+    constexpr int WIDE = (WDT == BW_F32 ? 8 : 16) / VPI;
+    if constexpr (WIDE > 1) {
+        if (quantize_fits<BITS, WDT, WIDE>(w, K, ldw, group, qweight))
+            return launch_quantize<BITS, WDT, MATH, WIDE>(w, N, K, ldw, group, qweight, scale, sdt, zp, zdt, st);
+    }
+    if (quantize_fits<BITS, WDT, 1>(w, K, ldw, group, qweight))
+        return launch_quantize<BITS, WDT, MATH, 1>(w, N, K, ldw, group, qweight, scale, sdt, zp, zdt, st);
+    const int64_t total = N * (K / VPI);
+    hipLaunchKernelGGL((quantize_pack_generic_kernel<WDT, MATH>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, w, N,
+                       (int)K, ldw, BITS, group, qweight, scale, sdt, zp, zdt);
     return hipGetLastError() == hipSuccess ? BW_OK : BW_ELAUNCH;
 }
 
 template <int WDT, int MATH>
 int dispatch_bits(int bits, const void* w, int64_t N, int64_t K, int64_t ldw, int group, int32_t* qweight, void* scale,
                   int sdt, void* zp, int zdt, hipStream_t st) {
-    if (bits == 2) return launch_quantize<2, WDT, MATH>(w, N, K, ldw, group, qweight, scale, sdt, zp, zdt, st);
-    if (bits == 4) return launch_quantize<4, WDT, MATH>(w, N, K, ldw, group, qweight, scale, sdt, zp, zdt, st);
-    return launch_quantize<8, WDT, MATH>(w, N, K, ldw, group, qweight, scale, sdt, zp, zdt, st);
+    if (bits == 2) return launch_quantize_bits<2, WDT, MATH>(w, N, K, ldw, group, qweight, scale, sdt, zp, zdt, st);
+    if (bits == 4) return launch_quantize_bits<4, WDT, MATH>(w, N, K, ldw, group, qweight, scale, sdt, zp, zdt, st);
+    return launch_quantize_bits<8, WDT, MATH>(w, N, K, ldw, group, qweight, scale, sdt, zp, zdt, st);
 }
 
 }  // namespace
@@ -207,14 +294,8 @@ extern "C" int bw_quantize_pack(const void* w, int w_dtype, int math_dtype, int6
     if (zp_dtype != BW_I32 && zp_dtype != BW_F16 && zp_dtype != BW_BF16) return BW_EINVAL;
     // math in a 16-bit type only makes sense on weights of that type (eager torch never mixes them)
     if (math_dtype != BW_F32 && math_dtype != w_dtype) return BW_EINVAL;
-    const int vpi = 32 / bits;
-    const int lpg = group / vpi;
-    const bool pow2 = group % vpi == 0 && lpg >= 1 && lpg <= 64 && (lpg & (lpg - 1)) == 0;
-    // vector loads of one word's worth of weights: 16-byte (or 8-byte for 4 halves) alignment
-    const size_t esz = w_dtype == BW_F32 ? 4 : 2;
-    const size_t need = (vpi * esz >= 16) ? 16 : vpi * esz;
-    if (!pow2) return BW_EUNSUPPORTED;   // needs a byte scratch plane; see bw_quantize_pack in the header
-    if (!bw_aligned(w, need) || (ldw * esz) % need) return BW_EALIGN;
+    // every entry of scale / zp needs natural alignment; the kernels pick their own vector widths
+    if (!bw_aligned(w, w_dtype == BW_F32 ? 4 : 2) || !bw_aligned(qweight, 4)) return BW_EALIGN;
     hipStream_t st = (hipStream_t)stream;
 #define BW_Q(WD, MD) \
     if (w_dtype == WD && math_dtype == MD) return dispatch_bits<WD, MD>(bits, w, N, K, ldw, group, qweight, scale, scale_dtype, zp, zp_dtype, st);
@@ -247,7 +328,7 @@ extern "C" int bw_dequantize(const int32_t* qweight, const void* scale, int scal
     return BW_EINVAL;
 }
 
-extern "C" int bw_abi_version(void) { return 1; }
+extern "C" int bw_abi_version(void) { return 2; }
 
 extern "C" const char* bw_strerror(int status) {
     switch (status) {

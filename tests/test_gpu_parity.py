@@ -122,6 +122,48 @@ def test_quantize_random_vs_oracle(bits, g, wdtype):
         assert np.array_equal(_bits_of(got), expect)
 
 
+def _tie_heavy_weights(n, k, bits, g, seed):
+    """float32 weights whose quotient w / scale + zp sits on, or within a few ulps of, a half-integer: the
+    inputs where a quotient that is off by one ulp changes the rounded integer."""
+    rng = np.random.default_rng(seed)
+    qmax = np.float32(2 ** bits - 1)
+    w = np.empty((n, k), dtype=np.float32)
+    for r in range(n):
+        for c in range(k // g):
+            mag = np.float32(10.0 ** rng.uniform(-6, 4))
+            lo = np.float32(-mag * rng.uniform(0.05, 1.0))
+            hi = np.float32(mag * rng.uniform(0.05, 1.0))
+            s = max(np.float32(np.float32(hi - lo) / qmax), np.float32(1e-8))
+            zf = np.float32(min(max(np.rint(np.float32(-lo / s)), 0), qmax))
+            j = rng.integers(0, int(qmax), size=g).astype(np.float32)
+            vals = (s * (j + np.float32(0.5) - zf)).astype(np.float32)       # quotient + zp = j + 0.5 (up to rounding)
+            for _ in range(3):                                               # walk up to 3 ulps either way
+                step = rng.integers(-1, 2, size=g)
+                vals = np.where(step > 0, np.nextafter(vals, np.float32(np.inf)),
+                                np.where(step < 0, np.nextafter(vals, np.float32(-np.inf)), vals)).astype(np.float32)
+            vals = np.clip(vals, lo, hi)
+            vals[0], vals[1] = lo, hi                                        # pin the group's extrema, hence its scale
+            w[r, c * g:(c + 1) * g] = vals
+    return w
+
+
+@pytest.mark.parametrize("bits,g", COMBOS)
+def test_quantize_near_ties_vs_oracle(bits, g):
+    """The quantiser's short division is only taken away from rounding ties; this feeds it ties."""
+    hip = _hip()
+    w = _tie_heavy_weights(48, 1024, bits, g, seed=17 * bits + g)
+    for wt in (torch.from_numpy(w), torch.from_numpy(w).half()):
+        w_eff = wt.float().numpy()
+        finite = np.isfinite(w_eff).all(axis=1)
+        qw_o, s_o, z_o, _ = orc.quantize_rtn(w_eff, bits, g)
+        qw, sc, z = hip.quantize_pack(wt.cuda(), bits, g, math_dtype=torch.float32, scale_dtype=torch.float32,
+                                      zp_dtype=torch.int32)
+        assert finite.sum() >= 40
+        assert np.array_equal(qw.cpu().numpy()[finite], qw_o[finite])
+        assert np.array_equal(_bits_of(sc)[finite], s_o.view(np.uint32)[finite])
+        assert np.array_equal(z.cpu().numpy()[finite], z_o[finite])
+
+
 GEMV_SHAPES = [(768, 3072), (256, 40), (4096, 512), (11008, 64), (2048, 16), (1024, 1000)]
 
 
@@ -206,10 +248,15 @@ def test_reference_acceptance_recipe():
 
 
 def test_generic_shapes_any_group():
-    """Group sizes / K outside the fast layouts take the shape-generic kernel."""
+    """Group sizes / K outside the fast layouts take the shape-generic kernels."""
     hip = _hip()
     for bits, g, k, n in ((4, 48, 96, 20), (8, 20, 40, 33), (2, 16, 48, 7)):
-        _, qw, s16, z16, b16 = quantized_layer(n, k, bits, g, seed=g + k)
+        w, qw, s16, z16, b16 = quantized_layer(n, k, bits, g, seed=g + k)
+        # quantiser: any group size the reference accepts, bit-exact
+        qw_g, s_g, z_g = hip.quantize_pack(to_gpu(w), bits, g, math_dtype=torch.float32, scale_dtype=torch.float16,
+                                           zp_dtype=torch.float16)
+        assert np.array_equal(qw_g.cpu().numpy(), qw)
+        assert np.array_equal(_bits_of(s_g), s16.view(np.uint16)) and np.array_equal(_bits_of(z_g), z16.view(np.uint16))
         x = np.random.default_rng(g).standard_normal((5, k)).astype(np.float16)
         y = hip.quantized_matmul_hip(to_gpu(x), to_gpu(qw), to_gpu(s16), to_gpu(z16), to_gpu(b16), bits, g)
         check_matmul(y, x, qw, s16, z16, b16, bits, g)
