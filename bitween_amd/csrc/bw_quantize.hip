@@ -85,7 +85,8 @@ BW_DEV float quant_exact(float w, float s, float zf) {
 // half-integer, round(t) is therefore the reference's value; the rare elements that do (and anything
 // large, infinite or NaN) are redone with the true IEEE divide.
 template <int BITS, int WDT, int MATH, int WPT>
-__global__ __launch_bounds__(256) void quantize_pack_kernel(const void* __restrict__ w, int64_t N, int K, int64_t ldw,
+__global__ __launch_bounds__(256) void quantize_pack_kernel(const void* __restrict__ w, const void* __restrict__ delta,
+                                                            int64_t N, int K, int64_t ldw, int64_t ldd,
                                                             int group, int lpg, int32_t* __restrict__ qweight,
                                                             void* __restrict__ scale, int scale_dtype,
                                                             void* __restrict__ zp, int zp_dtype) {
@@ -99,6 +100,12 @@ __global__ __launch_bounds__(256) void quantize_pack_kernel(const void* __restri
     for (int64_t row = blockIdx.y; row < N; row += gridDim.y) {
         float v[VPT];
         load_vals<WDT, VPT>(w, row * ldw + (int64_t)tcol * VPT, v);
+        if (delta) {                                     // w + delta, one rounding to the weights' own type
+            float dv[VPT];
+            load_vals<WDT, VPT>(delta, row * ldd + (int64_t)tcol * VPT, dv);
+#pragma unroll
+            for (int i = 0; i < VPT; i++) v[i] = rnd<WDT>(__fadd_rn(v[i], dv[i]));
+        }
 #pragma unroll
         for (int i = 0; i < VPT; i++) { v[i] = rnd<MATH>(v[i]); }
         float lo = v[0], hi = v[0];
@@ -156,7 +163,8 @@ __global__ __launch_bounds__(256) void quantize_pack_kernel(const void* __restri
 // Any group size: one thread per packed word, which scans the whole group of each of its values for the
 // extrema (re-using them while consecutive values share a group).  Slow, exact, no scratch memory.
 template <int WDT, int MATH>
-__global__ __launch_bounds__(256) void quantize_pack_generic_kernel(const void* __restrict__ w, int64_t N, int K, int64_t ldw,
+__global__ __launch_bounds__(256) void quantize_pack_generic_kernel(const void* __restrict__ w, const void* __restrict__ delta,
+                                                                    int64_t N, int K, int64_t ldw, int64_t ldd,
                                                                     int bits, int group, int32_t* __restrict__ qweight,
                                                                     void* __restrict__ scale, int scale_dtype,
                                                                     void* __restrict__ zp, int zp_dtype) {
@@ -169,13 +177,17 @@ __global__ __launch_bounds__(256) void quantize_pack_generic_kernel(const void* 
     uint32_t word = 0;
     int gprev = -1;
     float s = 0.f, zf = 0.f;
+    auto value = [&](int k) {
+        float x = Elem<WDT>::load(w, row * ldw + k);
+        if (delta) x = rnd<WDT>(__fadd_rn(x, Elem<WDT>::load(delta, row * ldd + k)));
+        return rnd<MATH>(x);
+    };
     for (int i = 0; i < vpi; i++) {
         const int k = wcol * vpi + i, g = k / group;
         if (g != gprev) {
-            const int64_t base = row * ldw + (int64_t)g * group;
-            float lo = rnd<MATH>(Elem<WDT>::load(w, base)), hi = lo;
+            float lo = value(g * group), hi = lo;
             for (int e = 1; e < group; e++) {
-                const float x = rnd<MATH>(Elem<WDT>::load(w, base + e));
+                const float x = value(g * group + e);
                 lo = fminf(lo, x);
                 hi = fmaxf(hi, x);
             }
@@ -186,7 +198,7 @@ __global__ __launch_bounds__(256) void quantize_pack_generic_kernel(const void* 
                 store_meta(zp, zp_dtype, row * groups + g, zf);
             }
         }
-        const float t = quant_exact<MATH>(rnd<MATH>(Elem<WDT>::load(w, row * ldw + k)), s, zf);
+        const float t = quant_exact<MATH>(value(k), s, zf);
         word |= (uint32_t)(int)fminf(fmaxf(t, 0.f), qmax) << (i * bits);
     }
     qweight[idx] = (int32_t)word;
@@ -235,73 +247,83 @@ __global__ __launch_bounds__(256) void dequantize_kernel(const uint32_t* __restr
 // Can a launch with WPT words per thread take this shape?  Vector loads / stores need their alignment, the
 // threads of a group must be a power of two inside one wave.
 template <int BITS, int WDT, int WPT>
-bool quantize_fits(const void* w, int64_t K, int64_t ldw, int group, const void* qweight) {
+bool quantize_fits(const void* w, const void* delta, int64_t K, int64_t ldw, int64_t ldd, int group, const void* qweight) {
     constexpr int VPT = 32 / BITS * WPT;
     constexpr size_t esz = WDT == BW_F32 ? 4 : 2;
     constexpr size_t need = (VPT * esz >= 16) ? 16 : VPT * esz;
     const int lpg = group / VPT;
     return group % VPT == 0 && K % VPT == 0 && lpg >= 1 && lpg <= 64 && (lpg & (lpg - 1)) == 0 && bw_aligned(w, need) &&
-           (ldw * esz) % need == 0 && bw_aligned(qweight, 4 * WPT);
+           (ldw * esz) % need == 0 && bw_aligned(qweight, 4 * WPT) &&
+           (!delta || (bw_aligned(delta, need) && (ldd * esz) % need == 0));
 }
 
 template <int BITS, int WDT, int MATH, int WPT>
-int launch_quantize(const void* w, int64_t N, int64_t K, int64_t ldw, int group, int32_t* qweight, void* scale, int sdt,
-                    void* zp, int zdt, hipStream_t st) {
+int launch_quantize(const void* w, const void* delta, int64_t N, int64_t K, int64_t ldw, int64_t ldd, int group,
+                    int32_t* qweight, void* scale, int sdt, void* zp, int zdt, hipStream_t st) {
     constexpr int VPT = 32 / BITS * WPT;
     const int tpr = (int)(K / VPT);
     const int block = tpr >= 256 ? 256 : ((tpr + 63) / 64) * 64;
     dim3 grid((unsigned)((tpr + block - 1) / block), (unsigned)(N < 65535 ? N : 65535));
-    hipLaunchKernelGGL((quantize_pack_kernel<BITS, WDT, MATH, WPT>), grid, dim3(block), 0, st, w, N, (int)K, ldw, group,
-                       group / VPT, qweight, scale, sdt, zp, zdt);
+    hipLaunchKernelGGL((quantize_pack_kernel<BITS, WDT, MATH, WPT>), grid, dim3(block), 0, st, w, delta, N, (int)K, ldw, ldd,
+                       group, group / VPT, qweight, scale, sdt, zp, zdt);
     return hipGetLastError() == hipSuccess ? BW_OK : BW_ELAUNCH;
 }
 
 template <int BITS, int WDT, int MATH>
-int launch_quantize_bits(const void* w, int64_t N, int64_t K, int64_t ldw, int group, int32_t* qweight, void* scale, int sdt,
-                         void* zp, int zdt, hipStream_t st) {
+int launch_quantize_bits(const void* w, const void* delta, int64_t N, int64_t K, int64_t ldw, int64_t ldd, int group,
+                         int32_t* qweight, void* scale, int sdt, void* zp, int zdt, hipStream_t st) {
     // 32 bytes of input per thread where the shape allows, else one word per thread, else the generic kernel
     constexpr int VPI = 32 / BITS;
     constexpr int WIDE = (WDT == BW_F32 ? 8 : 16) / VPI;
     if constexpr (WIDE > 1) {
-        if (quantize_fits<BITS, WDT, WIDE>(w, K, ldw, group, qweight))
-            return launch_quantize<BITS, WDT, MATH, WIDE>(w, N, K, ldw, group, qweight, scale, sdt, zp, zdt, st);
+        if (quantize_fits<BITS, WDT, WIDE>(w, delta, K, ldw, ldd, group, qweight))
+            return launch_quantize<BITS, WDT, MATH, WIDE>(w, delta, N, K, ldw, ldd, group, qweight, scale, sdt, zp, zdt, st);
     }
-    if (quantize_fits<BITS, WDT, 1>(w, K, ldw, group, qweight))
-        return launch_quantize<BITS, WDT, MATH, 1>(w, N, K, ldw, group, qweight, scale, sdt, zp, zdt, st);
+    if (quantize_fits<BITS, WDT, 1>(w, delta, K, ldw, ldd, group, qweight))
+        return launch_quantize<BITS, WDT, MATH, 1>(w, delta, N, K, ldw, ldd, group, qweight, scale, sdt, zp, zdt, st);
     const int64_t total = N * (K / VPI);
-    hipLaunchKernelGGL((quantize_pack_generic_kernel<WDT, MATH>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, w, N,
-                       (int)K, ldw, BITS, group, qweight, scale, sdt, zp, zdt);
+    hipLaunchKernelGGL((quantize_pack_generic_kernel<WDT, MATH>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, w,
+                       delta, N, (int)K, ldw, ldd, BITS, group, qweight, scale, sdt, zp, zdt);
     return hipGetLastError() == hipSuccess ? BW_OK : BW_ELAUNCH;
 }
 
 template <int WDT, int MATH>
-int dispatch_bits(int bits, const void* w, int64_t N, int64_t K, int64_t ldw, int group, int32_t* qweight, void* scale,
-                  int sdt, void* zp, int zdt, hipStream_t st) {
-    if (bits == 2) return launch_quantize_bits<2, WDT, MATH>(w, N, K, ldw, group, qweight, scale, sdt, zp, zdt, st);
-    if (bits == 4) return launch_quantize_bits<4, WDT, MATH>(w, N, K, ldw, group, qweight, scale, sdt, zp, zdt, st);
-    return launch_quantize_bits<8, WDT, MATH>(w, N, K, ldw, group, qweight, scale, sdt, zp, zdt, st);
+int dispatch_bits(int bits, const void* w, const void* delta, int64_t N, int64_t K, int64_t ldw, int64_t ldd, int group,
+                  int32_t* qweight, void* scale, int sdt, void* zp, int zdt, hipStream_t st) {
+    if (bits == 2) return launch_quantize_bits<2, WDT, MATH>(w, delta, N, K, ldw, ldd, group, qweight, scale, sdt, zp, zdt, st);
+    if (bits == 4) return launch_quantize_bits<4, WDT, MATH>(w, delta, N, K, ldw, ldd, group, qweight, scale, sdt, zp, zdt, st);
+    return launch_quantize_bits<8, WDT, MATH>(w, delta, N, K, ldw, ldd, group, qweight, scale, sdt, zp, zdt, st);
 }
 
 }  // namespace
 
-extern "C" int bw_quantize_pack(const void* w, int w_dtype, int math_dtype, int64_t N, int64_t K, int64_t ldw, int bits,
-                                int group, int32_t* qweight, void* scale, int scale_dtype, void* zp, int zp_dtype,
-                                void* stream) {
+extern "C" int bw_quantize_pack_add(const void* w, const void* delta, int w_dtype, int math_dtype, int64_t N, int64_t K,
+                                    int64_t ldw, int64_t ldd, int bits, int group, int32_t* qweight, void* scale,
+                                    int scale_dtype, void* zp, int zp_dtype, void* stream) {
     if (!w || !qweight || !scale || !zp) return BW_EINVAL;
-    if (!bw_shape_ok(N, K, bits, group) || ldw < K) return BW_EINVAL;
+    if (!bw_shape_ok(N, K, bits, group) || ldw < K || (delta && ldd < K)) return BW_EINVAL;
     if (w_dtype != BW_F16 && w_dtype != BW_BF16 && w_dtype != BW_F32) return BW_EINVAL;
     if (scale_dtype != BW_F32 && scale_dtype != BW_F16 && scale_dtype != BW_BF16) return BW_EINVAL;
     if (zp_dtype != BW_I32 && zp_dtype != BW_F16 && zp_dtype != BW_BF16) return BW_EINVAL;
     // math in a 16-bit type only makes sense on weights of that type (eager torch never mixes them)
     if (math_dtype != BW_F32 && math_dtype != w_dtype) return BW_EINVAL;
-    // every entry of scale / zp needs natural alignment; the kernels pick their own vector widths
-    if (!bw_aligned(w, w_dtype == BW_F32 ? 4 : 2) || !bw_aligned(qweight, 4)) return BW_EALIGN;
+    // every element needs its natural alignment; the kernels pick their own vector widths
+    const size_t esz = w_dtype == BW_F32 ? 4 : 2;
+    if (!bw_aligned(w, esz) || !bw_aligned(qweight, 4) || (delta && !bw_aligned(delta, esz))) return BW_EALIGN;
     hipStream_t st = (hipStream_t)stream;
 #define BW_Q(WD, MD) \
-    if (w_dtype == WD && math_dtype == MD) return dispatch_bits<WD, MD>(bits, w, N, K, ldw, group, qweight, scale, scale_dtype, zp, zp_dtype, st);
+    if (w_dtype == WD && math_dtype == MD) \
+        return dispatch_bits<WD, MD>(bits, w, delta, N, K, ldw, ldd, group, qweight, scale, scale_dtype, zp, zp_dtype, st);
     BW_Q(BW_F32, BW_F32) BW_Q(BW_F16, BW_F32) BW_Q(BW_BF16, BW_F32) BW_Q(BW_F16, BW_F16) BW_Q(BW_BF16, BW_BF16)
 #undef BW_Q
     return BW_EINVAL;
+}
+
+extern "C" int bw_quantize_pack(const void* w, int w_dtype, int math_dtype, int64_t N, int64_t K, int64_t ldw, int bits,
+                                int group, int32_t* qweight, void* scale, int scale_dtype, void* zp, int zp_dtype,
+                                void* stream) {
+    return bw_quantize_pack_add(w, nullptr, w_dtype, math_dtype, N, K, ldw, 0, bits, group, qweight, scale, scale_dtype, zp,
+                                zp_dtype, stream);
 }
 
 extern "C" int bw_dequantize(const int32_t* qweight, const void* scale, int scale_dtype, const void* zp, int zp_dtype,

@@ -18,6 +18,14 @@ def _gpu_for(t):
 
 
 @torch.no_grad()
+def quantize_rtn_perturbed(weight: torch.Tensor, value: torch.Tensor, bits: int = 8, group_size: int = 32):
+    """quantize_rtn(weight + value, bits, group_size) in one kernel: the hand-off of a tuned layer to its
+    inference form (WrapperLinear.to_quantized_linear, bitween/wrapper.py:222-232).  `value` must have the
+    shape and dtype of `weight`; the sum is rounded once to that dtype, as the eager add is."""
+    return _quantize(weight, bits, group_size, value)
+
+
+@torch.no_grad()
 def quantize_rtn(weight: torch.Tensor, bits: int = 8, group_size: int = 32):
     """Round-to-nearest asymmetric per-group quantisation and packing.
 
@@ -26,6 +34,10 @@ def quantize_rtn(weight: torch.Tensor, bits: int = 8, group_size: int = 32):
     of bitween/functional.py:45.  Arithmetic is carried out in weight.dtype,
     as the reference's eager ops do.
     """
+    return _quantize(weight, bits, group_size, None)
+
+
+def _quantize(weight, bits, group_size, value):
     assert bits in [2, 4, 8], "Only 2, 4, or 8-bit quantization supported."
     if weight.dim() != 2:
         raise ValueError("weight must be [out_features, in_features]")
@@ -40,7 +52,7 @@ def quantize_rtn(weight: torch.Tensor, bits: int = 8, group_size: int = 32):
     dev = _gpu_for(weight)
     w = weight.to(dev)
     qweight, scale, zp = _hip.quantize_pack(w, bits, group_size, math_dtype=weight.dtype, scale_dtype=weight.dtype,
-                                            zp_dtype=torch.int32)
+                                            zp_dtype=torch.int32, delta=None if value is None else value.to(dev))
     if not weight.is_cuda:
         qweight, scale, zp = qweight.to(weight.device), scale.to(weight.device), zp.to(weight.device)
     return qweight, scale, zp, group_size

@@ -19,7 +19,7 @@ _lib = None
 BW_F16, BW_BF16, BW_F32, BW_I32 = 0, 1, 2, 3
 _DTYPE_CODE = {torch.float16: BW_F16, torch.bfloat16: BW_BF16, torch.float32: BW_F32, torch.int32: BW_I32}
 
-ENTRY_POINTS = ("bw_abi_version", "bw_strerror", "bw_quantize_pack", "bw_dequantize", "bw_qgemv", "bw_qgemm",
+ENTRY_POINTS = ("bw_abi_version", "bw_strerror", "bw_quantize_pack", "bw_quantize_pack_add", "bw_dequantize", "bw_qgemv", "bw_qgemm",
                 "bw_qgemm_ws", "bw_qgemm_workspace_bytes", "bw_qlinear")
 
 
@@ -46,6 +46,7 @@ def load():
     lib.bw_strerror.restype = ctypes.c_char_p
     lib.bw_strerror.argtypes = [i32]
     lib.bw_quantize_pack.argtypes = [vp, i32, i32, i64, i64, i64, i32, i32, vp, vp, i32, vp, i32, vp]
+    lib.bw_quantize_pack_add.argtypes = [vp, vp, i32, i32, i64, i64, i64, i64, i32, i32, vp, vp, i32, vp, i32, vp]
     lib.bw_dequantize.argtypes = [vp, vp, i32, vp, i32, i64, i64, i32, i32, vp, i32, i64, vp]
     mm = [vp, i32, i64, i64, i64, vp, vp, vp, vp, i64, i32, i32, vp, i64, vp]
     for name in ("bw_qgemv", "bw_qgemm", "bw_qlinear"):
@@ -53,7 +54,7 @@ def load():
     lib.bw_qgemm_ws.argtypes = mm[:-1] + [vp, ctypes.c_size_t, vp]
     lib.bw_qgemm_workspace_bytes.argtypes = [i64, i64, i64, i32, i32]
     lib.bw_qgemm_workspace_bytes.restype = ctypes.c_size_t
-    for name in ("bw_quantize_pack", "bw_dequantize", "bw_qgemv", "bw_qgemm", "bw_qgemm_ws", "bw_qlinear"):
+    for name in ("bw_quantize_pack", "bw_quantize_pack_add", "bw_dequantize", "bw_qgemv", "bw_qgemm", "bw_qgemm_ws", "bw_qlinear"):
         getattr(lib, name).restype = i32
     _lib = lib
     return lib
@@ -78,21 +79,30 @@ def _stream(device):
     return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
 
 
-def quantize_pack(weight, bits, group_size, math_dtype, scale_dtype, zp_dtype):
-    """weight [N,K] on GPU (f16/bf16/f32) -> (qweight int32, scale, zero_point) per bw_quantize_pack."""
+def quantize_pack(weight, bits, group_size, math_dtype, scale_dtype, zp_dtype, delta=None):
+    """weight [N,K] on GPU (f16/bf16/f32) -> (qweight int32, scale, zero_point) per bw_quantize_pack; with
+    `delta` (same shape and dtype) the kernel quantises weight + delta (bw_quantize_pack_add)."""
     require_gpu(weight, "quantize_pack")
     if weight.stride(-1) != 1:
         weight = weight.contiguous()
     n, k = weight.shape
     vpi = 32 // bits
     dev = weight.device
+    if delta is not None:
+        require_gpu(delta, "quantize_pack")
+        if delta.shape != weight.shape or delta.dtype != weight.dtype:
+            raise ValueError("delta must have the shape and dtype of weight")
+        if delta.stride(-1) != 1:
+            delta = delta.contiguous()
     qweight = torch.empty((n, k // vpi), dtype=torch.int32, device=dev)
     scale = torch.empty((n, k // group_size), dtype=scale_dtype, device=dev)
     zp = torch.empty((n, k // group_size), dtype=zp_dtype, device=dev)
     with torch.cuda.device(dev):
-        st = load().bw_quantize_pack(weight.data_ptr(), _DTYPE_CODE[weight.dtype], _DTYPE_CODE[math_dtype], n, k,
-                                     weight.stride(0), bits, group_size, qweight.data_ptr(), scale.data_ptr(),
-                                     _DTYPE_CODE[scale_dtype], zp.data_ptr(), _DTYPE_CODE[zp_dtype], _stream(dev))
+        st = load().bw_quantize_pack_add(weight.data_ptr(), None if delta is None else delta.data_ptr(),
+                                         _DTYPE_CODE[weight.dtype], _DTYPE_CODE[math_dtype], n, k, weight.stride(0),
+                                         0 if delta is None else delta.stride(0), bits, group_size, qweight.data_ptr(),
+                                         scale.data_ptr(), _DTYPE_CODE[scale_dtype], zp.data_ptr(),
+                                         _DTYPE_CODE[zp_dtype], _stream(dev))
     _check(st, "bw_quantize_pack")
     return qweight, scale, zp
 

@@ -1,1 +1,1 @@
-from .quantizer import Bitween
+from .quantizer import Bitween, apply_precision_map

@@ -62,6 +62,14 @@ int bw_quantize_pack(const void* w, int w_dtype, int math_dtype, int64_t N, int6
                      int bits, int group, int32_t* qweight, void* scale, int scale_dtype,
                      void* zp, int zp_dtype, void* stream);
 
+/* quantize_rtn(orig_weight + value, bits, group_size): the hand-off of a tuned layer,
+ * WrapperLinear.to_quantized_linear (bitween/wrapper.py:222-232), without materialising the sum.
+ *   delta  [N][ldd] of w_dtype, or NULL (then identical to bw_quantize_pack); the sum w + delta is rounded
+ *          once to w_dtype, as the eager tensor add does, before the arithmetic above. */
+int bw_quantize_pack_add(const void* w, const void* delta, int w_dtype, int math_dtype, int64_t N, int64_t K,
+                         int64_t ldw, int64_t ldd, int bits, int group, int32_t* qweight,
+                         void* scale, int scale_dtype, void* zp, int zp_dtype, void* stream);
+
 /* dequantize_rtn(q_packed, scale, zero_point, group_size, bits) -> weight
  * replaces bitween/functional.py:47-71 (out_dtype BW_F32) and the per-forward
  * dequantize kernel bitween/modules.py:10-58 (out_dtype BW_F16: one rounding

