@@ -18,16 +18,6 @@
 
 bool bw_fast_shape(int64_t M, int64_t N, int64_t K, int64_t ldx, int bits, int group);
 
-#ifdef BW_TRACE
-__device__ unsigned long long bw_gemm_trace[64 * 8];
-extern "C" int bw_debug_gemm_trace(unsigned long long* out) {
-    return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(bw_gemm_trace), sizeof(bw_gemm_trace));
-}
-#define BW_GT(slot) if (blockIdx.x == 3 && blockIdx.y == 0 && tid == 0 && c < 64) { asm volatile("" ::: "memory"); bw_gemm_trace[c * 8 + (slot)] = __builtin_amdgcn_s_memrealtime(); }
-#else
-#define BW_GT(slot)
-#endif
-
 namespace {
 
 constexpr int WAVES = 4, NT = 4, MT = 8, BM = MT * 16, BN = WAVES * NT * 16;
@@ -87,11 +77,7 @@ BW_DEV h8 unpack_step(const u4& w, int t, const GroupConst<BITS>* gc, int ng_wor
 // instruction on gfx950 concern reads of the result by non-MFMA instructions; the only such reads are in
 // the epilogue, hundreds of cycles (an LDS staging pass and a barrier) after the last MFMA.
 BW_DEV void mfma_acc(f4& acc, const h8& a, const h8& b) {
-#ifdef BW_MFMA_BUILTIN
-    acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, acc, 0, 0, 0);
-#else
     asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
-#endif
 }
 
 struct GemmArgs {
@@ -151,44 +137,6 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
     // of an outstanding load would stall on it.
     struct WSet { u4 w[NT]; uint32_t s[NT][C::NG], z[NT][C::NG]; };   // 16-bit values, one register each
     WSet set0, set1;
-    auto issue_x = [&](int c) {
-        const uint32_t kb = (uint32_t)c * C::CHUNK_K * 2;
-#pragma unroll
-        for (int i = 0; i < C::XL; i++) {
-            const int ku = (tid + i * WAVES * 64) % C::UPR;
-            const uint32_t off = (c < c_end && c * C::CHUNK_K + ku * C::UNIT < a.K) ? x_off[i] + kb : kOob;
-#pragma unroll
-            for (int j = 0; j < C::UW; j++) xr[i * C::UW + j] = __builtin_amdgcn_raw_buffer_load_b128(rx, off + j * 16, 0, 0);
-        }
-    };
-    auto issue_w = [&](int c, WSet& ws) {
-        const bool in = c < c_end && c * 64 + kq * 16 < a.row_bytes;   // lanes past the row end: their x is zero
-        const int g0 = min((c * C::CHUNK_K + kq * C::VPL) / GROUP, groups - C::NG);
-#pragma unroll
-        for (int j = 0; j < NT; j++) {
-            ws.w[j] = __builtin_amdgcn_raw_buffer_load_b128(rw, in ? w_off[j] + c * 64 : kOob, 0, 0);
-#pragma unroll
-            for (int g = 0; g < C::NG; g++) {
-                // zero-extending loads into whole registers: a 16-bit load into half a register would have
-                // to wait for the previous load into the other half
-                ws.s[j][g] = __builtin_amdgcn_raw_buffer_load_b16(rs, m_off[j] + (g0 + g) * 2, 0, 0);
-                ws.z[j][g] = __builtin_amdgcn_raw_buffer_load_b16(rz, m_off[j] + (g0 + g) * 2, 0, 0);
-            }
-        }
-    };
-    auto stage = [&](_Float16* xs) {
-#pragma unroll
-        for (int i = 0; i < C::XL; i++) {
-            const int u = tid + i * WAVES * 64, m = u / C::UPR, ku = u - m * C::UPR;
-            uint32_t in[4 * C::UW], o[4 * C::UW];
-#pragma unroll
-            for (int j = 0; j < C::UW; j++) { in[4 * j] = xr[i * C::UW + j][0]; in[4 * j + 1] = xr[i * C::UW + j][1]; in[4 * j + 2] = xr[i * C::UW + j][2]; in[4 * j + 3] = xr[i * C::UW + j][3]; }
-            permute_unit<BITS>(in, o);
-            u4* dst = reinterpret_cast<u4*>(xs + m * C::PITCH + ku * C::UNIT);
-#pragma unroll
-            for (int j = 0; j < C::UW; j++) dst[j] = u4{o[4 * j], o[4 * j + 1], o[4 * j + 2], o[4 * j + 3]};
-        }
-    };
 
     f4 acc[MT][NT];
 #pragma unroll
@@ -237,7 +185,6 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
     // count is exact.
     auto step = [&](int c, const _Float16* cur, _Float16* nxt, WSet& ws) {
         __builtin_amdgcn_sched_barrier(0);
-        BW_GT(0)
         GroupConst<BITS> gc[NT][C::NG];
 #pragma unroll
         for (int j = 0; j < NT; j++)
@@ -280,9 +227,6 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
             const int cu = t & 1, nx = cu ^ 1;
 #pragma unroll
             for (int i = 0; i < MT; i++) {
-                if (t == 0 && i == 1) { BW_GT(1) }
-                if (t == C::MF - 1 && i == 0) { BW_GT(2) }
-                if (t == C::MF - 1 && i == MT / 2) { BW_GT(3) }
                 if constexpr (BITS == 4) {
                     // An MFMA occupies the matrix pipe for 16 cycles but the issue port for 4: two or three
                     // VALU operations fit behind each one.  Slot i prepares half a weight fragment of
@@ -335,9 +279,7 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
             }
         }
         __builtin_amdgcn_sched_barrier(0);
-        BW_GT(4)
         __syncthreads();
-        BW_GT(5)
     };
 
     _Float16* buf0 = reinterpret_cast<_Float16*>(smem);
