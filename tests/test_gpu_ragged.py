@@ -1,0 +1,77 @@
+"""Seeded sweep over ragged shapes: N that is not a multiple of the 16-row tile, K that ends inside a chunk,
+every M from 1 to past the decode / prefill switch, padded activation rows, bias on and off.  Each case goes
+through the C ABI (bw_qlinear picks the kernel) and is checked against the oracle."""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+from gpu_util import check_matmul, quantized_layer, to_gpu
+from oracle import rtn_oracle as orc
+
+pytestmark = pytest.mark.gpu
+
+
+def _cases():
+    rng = np.random.default_rng(2024)
+    out = []
+    for i in range(48):
+        bits = int(rng.choice([2, 4, 8]))
+        g = int(rng.choice([32, 64, 128]))
+        k = g * int(rng.integers(1, 20))
+        n = int(rng.integers(1, 200))
+        m = int(rng.choice([1, 2, 3, 4, 5, 8, 9, 15, 16, 17, 31, 33, 64, 129]))
+        pad = int(rng.choice([0, 0, 8, 24]))
+        out.append((i, bits, g, k, n, m, pad, bool(rng.integers(0, 2))))
+    return out
+
+
+@pytest.mark.parametrize("case", _cases(), ids=lambda c: "b%d_g%d_K%d_N%d_M%d_pad%d_%s" % (c[1:7] + ("bias" if c[7] else "nobias",)))
+def test_ragged_shapes_through_the_abi(case):
+    from bitween_amd.kernels import hip_loader
+    lib = hip_loader.load()
+    i, bits, g, k, n, m, pad, use_bias = case
+    _, qw, s16, z16, b16 = quantized_layer(n, k, bits, g, seed=900 + i, outliers=True)
+    x = np.random.default_rng(i).standard_normal((m, k)).astype(np.float16)
+    ldx = k + pad
+    xbuf = torch.full((m, ldx), float("nan"), dtype=torch.float16, device="cuda")      # the padding must never be read
+    xbuf[:, :k] = to_gpu(x)
+    d = [to_gpu(a) for a in (qw, s16, z16, b16)]
+    ldy = n + 3
+    y = torch.full((m, ldy), 7.0, dtype=torch.float16, device="cuda")
+    st = lib.bw_qlinear(xbuf.data_ptr(), 0, m, k, ldx, d[0].data_ptr(), d[1].data_ptr(), d[2].data_ptr(),
+                        d[3].data_ptr() if use_bias else None, n, bits, g, y.data_ptr(), ldy,
+                        ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    assert st == 0
+    torch.cuda.synchronize()
+    assert (y[:, n:] == 7.0).all()                        # nothing written past a row's N outputs
+    check_matmul(y[:, :n], x, qw, s16, z16, b16 if use_bias else None, bits, g)
+
+
+@pytest.mark.parametrize("bits,g,n,k", [(4, 128, 5, 256), (8, 32, 33, 96), (2, 64, 17, 192), (4, 32, 1, 32)])
+def test_quantize_dequantize_ragged(bits, g, n, k):
+    """Row counts that leave waves partly empty, with a padded row pitch on the way in and out."""
+    from bitween_amd.kernels import hip_loader as hip
+    lib = hip.load()
+    rng = np.random.default_rng(n * k)
+    w = (rng.standard_normal((n, k)) * 0.05).astype(np.float32)
+    ldw = k + 16
+    wbuf = torch.full((n, ldw), float("nan"), dtype=torch.float32, device="cuda")
+    wbuf[:, :k] = to_gpu(w)
+    vpi = 32 // bits
+    qw = torch.empty((n, k // vpi), dtype=torch.int32, device="cuda")
+    sc = torch.empty((n, k // g), dtype=torch.float32, device="cuda")
+    zp = torch.empty((n, k // g), dtype=torch.int32, device="cuda")
+    st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    assert lib.bw_quantize_pack(wbuf.data_ptr(), 2, 2, n, k, ldw, bits, g, qw.data_ptr(), sc.data_ptr(), 2, zp.data_ptr(), 3, st) == 0
+    qw_o, s_o, z_o, _ = orc.quantize_rtn(w, bits, g)
+    assert np.array_equal(qw.cpu().numpy(), qw_o) and np.array_equal(zp.cpu().numpy(), z_o)
+    assert np.array_equal(sc.cpu().numpy().view(np.uint32), s_o.view(np.uint32))
+    ldo = k + 5
+    out = torch.full((n, ldo), 3.0, dtype=torch.float32, device="cuda")
+    assert lib.bw_dequantize(qw.data_ptr(), sc.data_ptr(), 2, zp.data_ptr(), 3, n, k, bits, g, out.data_ptr(), 2, ldo, st) == 0
+    torch.cuda.synchronize()
+    assert (out[:, k:] == 3.0).all()
+    expect = (s_o.repeat(g, axis=1) * (orc.unpack_words(qw_o, bits).astype(np.float32) - z_o.repeat(g, axis=1).astype(np.float32)))
+    assert np.array_equal(out[:, :k].cpu().numpy().view(np.uint32), expect.astype(np.float32).view(np.uint32))
