@@ -90,8 +90,11 @@ struct GemmArgs {
     uint32_t x_bytes, w_bytes, meta_bytes;
     int M, N, K, ldx, ldy;
     int groups, nchunks, row_bytes;
-    float* ws;            // split-K partial sums [splits][M][N] (float32), or null
-    int chunks_per_split; // K chunks each z-slice of the grid takes
+    // Grid plan: workgroup ids [0, full_tiles) each own a whole output tile; the remaining ids come in runs of
+    // `splits`, each run sharing one tile and cutting K into slices of chunks_per_split chunks whose float32
+    // partial tiles go to ws (one BM x BN block per id) for qgemm_reduce_kernel to add up.
+    float* ws;
+    int tiles_n, full_tiles, splits, chunks_per_split;
 };
 
 BW_DEV __amdgpu_buffer_rsrc_t make_rsrc(const void* p, uint32_t bytes) {
@@ -110,11 +113,16 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
     extern __shared__ __attribute__((aligned(16))) char smem[];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int nl = lane & 15, kq = lane >> 4;
-    const int m0 = blockIdx.y * BM;
-    const int n0 = blockIdx.x * BN + wave * (NT * 16);
+    const int id = (int)blockIdx.x;
+    const bool partial = id >= a.full_tiles;
+    const int run = partial ? id - a.full_tiles : 0;
+    const int tile = partial ? a.full_tiles + run / a.splits : id;
+    const int m0 = (tile / a.tiles_n) * BM;
+    const int n0 = (tile % a.tiles_n) * BN + wave * (NT * 16);
     const int groups = a.groups;
-    // split-K: this z-slice of the grid takes chunks [c_begin, c_end); requests beyond c_end read as zero
-    const int c_begin = blockIdx.z * a.chunks_per_split, c_end = min(a.nchunks, c_begin + a.chunks_per_split);
+    // a partial workgroup takes chunks [c_begin, c_end); requests beyond c_end read as zero
+    const int c_begin = partial ? (run % a.splits) * a.chunks_per_split : 0;
+    const int c_end = partial ? min(a.nchunks, c_begin + a.chunks_per_split) : a.nchunks;
     const __amdgpu_buffer_rsrc_t rw = make_rsrc(a.qweight, a.w_bytes), rx = make_rsrc(a.x, a.x_bytes);
 
     const __amdgpu_buffer_rsrc_t rs = make_rsrc(a.scale, a.meta_bytes), rz = make_rsrc(a.zp, a.meta_bytes);
@@ -319,27 +327,13 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
         step(c + 1, buf1, buf0, set1);
     }
     // acc[i][j][r] = y[m0 + 16 i + nl][n0 + 16 j + 4 kq + r]
-    if (a.ws) {
-        // split-K: float32 partial sums to the workspace; qgemm_reduce_kernel adds them up
-        float* wz = a.ws + (size_t)blockIdx.z * a.M * a.N;
+    if (partial) {
+        // float32 partial tile to this workgroup's block of the workspace (tile-shaped, so no bounds to check)
+        float* blk = a.ws + (size_t)run * (BM * BN) + wave * (NT * 16) + 4 * kq;
 #pragma unroll
-        for (int j = 0; j < NT; j++) {
-            const int n = n0 + 16 * j + 4 * kq;
-            if (n >= a.N) continue;
+        for (int j = 0; j < NT; j++)
 #pragma unroll
-            for (int i = 0; i < MT; i++) {
-                const int m = m0 + 16 * i + nl;
-                if (m >= a.M) continue;
-                float* dst = wz + (size_t)m * a.N + n;
-                if (n + 3 < a.N && (((uintptr_t)dst) & 15) == 0) {
-                    *reinterpret_cast<f4*>(dst) = acc[i][j];
-                } else {
-#pragma unroll
-                    for (int r = 0; r < 4; r++)
-                        if (n + r < a.N) dst[r] = acc[i][j][r];
-                }
-            }
-        }
+            for (int i = 0; i < MT; i++) *reinterpret_cast<f4*>(blk + (16 * i + nl) * BN + 16 * j) = acc[i][j];
         return;
     }
 #pragma unroll
@@ -370,43 +364,78 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
     }
 }
 
-// y[m][n] = fp16( sum_z ws[z][m][n] + bias[n] ); VEC consecutive n per thread (VEC = 4 needs N % 4 == 0)
-template <int VEC>
-__global__ __launch_bounds__(256) void qgemm_reduce_kernel(const float* __restrict__ ws, int splits, int M, int N,
-                                                           const _Float16* __restrict__ bias, _Float16* __restrict__ y,
-                                                           int ldy) {
-    const int64_t idx = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * VEC;
-    const int64_t total = (int64_t)M * N;
-    if (idx >= total) return;
-    const int m = (int)(idx / N), n = (int)(idx - (int64_t)m * N);
-    float v[VEC];
+// Adds up the partial tiles of the split workgroups: block (x, y) handles 1024 outputs of split tile y,
+// a thread four consecutive n.  y[m][n] = fp16( sum_z partial_z[m][n] + bias[n] ).
+__global__ __launch_bounds__(256) void qgemm_reduce_kernel(const GemmArgs a) {
+    const int tile = a.full_tiles + (int)blockIdx.y;
+    const int quad = (int)(blockIdx.x * blockDim.x + threadIdx.x);          // < BM * BN / 4
+    const int ml = quad / (BN / 4), nl4 = (quad % (BN / 4)) * 4;
+    const int m = (tile / a.tiles_n) * BM + ml, n = (tile % a.tiles_n) * BN + nl4;
+    if (m >= a.M || n >= a.N) return;
+    const float* src = a.ws + (size_t)blockIdx.y * a.splits * (BM * BN) + ml * BN + nl4;
+    f4 v = {0.f, 0.f, 0.f, 0.f};
+    for (int z = 0; z < a.splits; z++) {
+        const f4 t = *reinterpret_cast<const f4*>(src + (size_t)z * (BM * BN));
 #pragma unroll
-    for (int i = 0; i < VEC; i++) v[i] = 0.f;
-    for (int z = 0; z < splits; z++) {
-        if constexpr (VEC == 4) {
-            const f4 t = *reinterpret_cast<const f4*>(ws + z * total + idx);
-#pragma unroll
-            for (int i = 0; i < 4; i++) v[i] += t[i];
-        } else {
-            v[0] += ws[z * total + idx];
-        }
+        for (int i = 0; i < 4; i++) v[i] += t[i];
     }
-    _Float16* dst = y + (int64_t)m * ldy + n;
+    _Float16* dst = a.y + (int64_t)m * a.ldy + n;
+    _Float16 o[4];
 #pragma unroll
-    for (int i = 0; i < VEC; i++) {
-        if (bias) v[i] += (float)bias[n + i];
-        dst[i] = (_Float16)v[i];
+    for (int i = 0; i < 4; i++) o[i] = (_Float16)(v[i] + ((a.bias && n + i < a.N) ? (float)a.bias[n + i] : 0.f));
+    if (n + 3 < a.N && (((uintptr_t)dst) & 7) == 0) {
+        *reinterpret_cast<u2*>(dst) = u2{as_u32(h2{o[0], o[1]}), as_u32(h2{o[2], o[3]})};
+    } else {
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+            if (n + i < a.N) dst[i] = o[i];
     }
 }
 
-// How many z-slices to cut K into.  One workgroup fits per CU, so the grid runs in waves of 256 workgroups:
-// splitting pays only while tiles * splits still fits one wave, and never below 4 chunks per slice.
-inline int gemm_splits(int64_t M, int64_t N, int nchunks) {
-    const int64_t tiles = ((N + BN - 1) / BN) * ((M + BM - 1) / BM);
-    if (tiles > 128) return 1;
-    int s = (int)(256 / tiles);
+// One workgroup fits per CU, so a grid runs in rounds of `cus` workgroups.  Two cases cut K:
+//   * a grid of at most half a round (small M * N, long K): every tile is split so that one round is filled;
+//   * a last round that is at most half full: its tiles are split so that it takes a fraction of a tile's time.
+// Never below 4 chunks per slice.  Without a workspace nothing is split.
+struct GemmPlan {
+    int tiles_n, tiles, full_tiles, splits, chunks_per_split;
+    size_t ws_bytes;
+};
+
+inline int device_cus() {
+    static const int cus = [] {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess)
+            n = 0;
+        return n > 0 ? n : 256;
+    }();
+    return cus;
+}
+
+inline GemmPlan gemm_plan(int64_t M, int64_t N, int nchunks, bool have_workspace) {
+    GemmPlan p;
+    p.tiles_n = (int)((N + BN - 1) / BN);
+    p.tiles = p.tiles_n * (int)((M + BM - 1) / BM);
+    p.full_tiles = p.tiles;
+    p.splits = 1;
+    p.chunks_per_split = nchunks;
+    p.ws_bytes = 0;
+    if (!have_workspace) return p;
+    const int cus = device_cus();
+    const int rest = p.tiles <= cus / 2 ? p.tiles : p.tiles % cus;          // tiles of the (only or last) short round
+    if (rest == 0 || rest > cus / 2) return p;
+    int s = cus / rest;
     if (s > nchunks / 4) s = nchunks / 4;
-    return s < 2 ? 1 : s;
+    if (s > 16) s = 16;
+    if (s < 2) return p;
+    int cps = (nchunks + s - 1) / s;
+    cps += cps & 1;                                                          // even: the K loop runs two steps per pass
+    s = (nchunks + cps - 1) / cps;
+    if (s < 2) return p;
+    p.full_tiles = p.tiles - rest;
+    p.splits = s;
+    p.chunks_per_split = cps;
+    p.ws_bytes = (size_t)rest * s * BM * BN * sizeof(float);
+    return p;
 }
 
 template <int BITS, int GROUP>
@@ -420,23 +449,18 @@ int launch_gemm(GemmArgs a, void* workspace, size_t workspace_bytes, hipStream_t
             return BW_ELAUNCH;
         attr_set = true;
     }
-    int splits = workspace ? gemm_splits(a.M, a.N, a.nchunks) : 1;
-    if (splits > 1 && workspace_bytes < (size_t)splits * a.M * a.N * sizeof(float)) return BW_EWORKSPACE;
-    a.chunks_per_split = (a.nchunks + splits - 1) / splits;
-    a.chunks_per_split += a.chunks_per_split & 1;             // even: the K loop runs two steps per pass
-    splits = (a.nchunks + a.chunks_per_split - 1) / a.chunks_per_split;
-    a.ws = splits > 1 ? (float*)workspace : nullptr;
-    dim3 grid((unsigned)((a.N + BN - 1) / BN), (unsigned)((a.M + BM - 1) / BM), (unsigned)splits), block(WAVES * 64);
-    hipLaunchKernelGGL(kern, grid, block, lds, stream, a);
+    const GemmPlan p = gemm_plan(a.M, a.N, a.nchunks, workspace != nullptr);
+    if (p.ws_bytes > workspace_bytes) return BW_EWORKSPACE;
+    a.ws = (float*)workspace;
+    a.tiles_n = p.tiles_n;
+    a.full_tiles = p.full_tiles;
+    a.splits = p.splits;
+    a.chunks_per_split = p.chunks_per_split;
+    const int split_tiles = p.tiles - p.full_tiles;
+    hipLaunchKernelGGL(kern, dim3((unsigned)(p.full_tiles + split_tiles * p.splits)), dim3(WAVES * 64), lds, stream, a);
     if (hipGetLastError() != hipSuccess) return BW_ELAUNCH;
-    if (splits > 1) {
-        const int64_t total = (int64_t)a.M * a.N;
-        if (a.N % 4 == 0)
-            hipLaunchKernelGGL(qgemm_reduce_kernel<4>, dim3((unsigned)((total / 4 + 255) / 256)), dim3(256), 0, stream, a.ws,
-                               splits, a.M, a.N, a.bias, a.y, a.ldy);
-        else
-            hipLaunchKernelGGL(qgemm_reduce_kernel<1>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, a.ws,
-                               splits, a.M, a.N, a.bias, a.y, a.ldy);
+    if (split_tiles) {
+        hipLaunchKernelGGL(qgemm_reduce_kernel, dim3(BM * BN / 4 / 256, (unsigned)split_tiles), dim3(256), 0, stream, a);
         if (hipGetLastError() != hipSuccess) return BW_ELAUNCH;
     }
     return BW_OK;
@@ -483,10 +507,8 @@ int bw_qgemm_generic(const void* x, int act_dtype, int64_t M, int64_t K, int64_t
 }
 
 extern "C" size_t bw_qgemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int bits, int group) {
-    if (!bw_shape_ok(N, K, bits, group) || M < 1 || !bw_fast_shape(M, N, K, K, bits, group)) return 0;
-    const int nchunks = (int)((K * bits / 8 + 63) / 64);
-    const int splits = gemm_splits(M, N, nchunks);
-    return splits > 1 ? (size_t)splits * M * N * sizeof(float) : 0;
+    if (!bw_shape_ok(N, K, bits, group) || M < 1 || M >= ((int64_t)1 << 31) || !bw_fast_shape(M, N, K, K, bits, group)) return 0;
+    return gemm_plan(M, N, (int)((K * bits / 8 + 63) / 64), true).ws_bytes;
 }
 
 extern "C" int bw_qgemm_ws(const void* x, int act_dtype, int64_t M, int64_t K, int64_t ldx, const int32_t* qweight,
@@ -509,6 +531,8 @@ extern "C" int bw_qgemm_ws(const void* x, int act_dtype, int64_t M, int64_t K, i
     a.w_bytes = (uint32_t)(N * a.row_bytes);
     a.meta_bytes = (uint32_t)(N * a.groups * 2);
     a.ws = nullptr;
+    a.tiles_n = a.full_tiles = 0;
+    a.splits = 1;
     a.chunks_per_split = a.nchunks;
     hipStream_t st = (hipStream_t)stream;
 #define BW_CASE(B, G) \

@@ -58,15 +58,18 @@ def test_split_k_workspace_size_is_a_pure_host_function():
     from bitween_amd.kernels import hip_loader
     lib = hip_loader.load()
     ws = lib.bw_qgemm_workspace_bytes
-    # a grid of 128 x 256 tiles that fills the chip by itself needs no workspace
-    assert ws(2048, 14336, 4096, 4, 128) == 0
-    assert ws(4096, 4096, 4096, 4, 128) == 0
-    # few tiles and a long K: splits * M * N float32 partial sums, splits >= 2
+    tile = 128 * 256 * 4                                        # one float32 partial tile
+    # whole rounds of 256 tiles (one workgroup per CU), or a last round that is more than half full: no workspace
+    assert ws(2048, 4096, 14336, 4, 128) == 0                   # 16 x 16 tiles = exactly one round
+    assert ws(4096, 4096, 4096, 4, 128) == 0                    # 512 tiles
+    assert ws(512, 14336, 4096, 4, 128) == 0                    # 224 tiles: 0.875 of a round
+    # few tiles and a long K: every tile split so that one round is filled
     for m, n, k, bits in ((128, 4096, 14336, 4), (512, 4096, 14336, 4), (128, 14336, 4096, 4), (64, 1024, 2048, 8)):
         b = ws(m, n, k, bits, 128)
-        assert b % (m * n * 4) == 0 and b // (m * n * 4) >= 2
         tiles = -(-n // 256) * -(-m // 128)
-        assert tiles * (b // (m * n * 4)) <= 256
+        assert b % (tiles * tile) == 0 and 2 <= b // (tiles * tile) and tiles * (b // (tiles * tile)) <= 256
+    # a last round that is at most half full: only its tiles are split (896 tiles = 3 rounds + 128 tiles, cut in two)
+    assert ws(2048, 14336, 4096, 4, 128) == 128 * 2 * tile
     # too short a K to split, invalid shapes, shapes the generic kernel takes
     assert ws(128, 256, 128, 4, 128) == 0
     assert ws(128, 256, 100, 4, 32) == 0

@@ -207,7 +207,7 @@ def test_gemm_split_k_vs_unsplit_and_oracle(bits, g, m, k, n):
     x = np.random.default_rng(k + m).standard_normal((m, k)).astype(np.float16)
     d = [to_gpu(a) for a in (x, qw, s16, z16, b16)]
     need = lib.bw_qgemm_workspace_bytes(m, n, k, bits, g)
-    assert need >= 2 * m * n * 4, "case is meant to split"
+    assert need >= 2 * 128 * 256 * 4, "case is meant to split"
     ws = torch.empty(need, dtype=torch.uint8, device="cuda")
     st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
 
@@ -229,6 +229,36 @@ def test_gemm_split_k_vs_unsplit_and_oracle(bits, g, m, k, n):
     # the two differ only in the float32 summation order
     diff = (y_split.float() - y_plain.float()).abs().max().item()
     assert diff <= 2.0 ** -9 * y_plain.float().abs().max().item()
+
+
+def test_gemm_short_last_round_is_split():
+    """258 tiles on 256 CUs: the two tiles of the last round are cut along K (partial tiles + reduce kernel), the
+    other 256 are not.  Checked against the un-split run everywhere and against the oracle on rows of both kinds."""
+    import ctypes
+    from bitween_amd.kernels import hip_loader
+    lib = hip_loader.load()
+    bits, g, m, k, n = 4, 128, 128 * 86, 2048, 768
+    need = lib.bw_qgemm_workspace_bytes(m, n, k, bits, g)
+    if need == 0:
+        pytest.skip("this device's CU count leaves no short last round for 258 tiles")
+    assert need % (128 * 256 * 4) == 0 and need < 64 * 128 * 256 * 4      # a few tiles' worth, not the whole matrix
+    _, qw, s16, z16, b16 = quantized_layer(n, k, bits, g, seed=77, outliers=True)
+    x = np.random.default_rng(78).standard_normal((m, k)).astype(np.float16)
+    d = [to_gpu(a) for a in (x, qw, s16, z16, b16)]
+    ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+    st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    ys = []
+    for ws_ptr, ws_bytes in ((ws.data_ptr(), need), (None, 0)):
+        y = torch.full((m, n), float("nan"), dtype=torch.float16, device="cuda")
+        assert lib.bw_qgemm_ws(d[0].data_ptr(), 0, m, k, k, d[1].data_ptr(), d[2].data_ptr(), d[3].data_ptr(), d[4].data_ptr(),
+                               n, bits, g, y.data_ptr(), n, ws_ptr, ws_bytes, st) == 0
+        ys.append(y)
+    torch.cuda.synchronize()
+    assert torch.isfinite(ys[0]).all()
+    diff = (ys[0].float() - ys[1].float()).abs().max().item()
+    assert diff <= 2.0 ** -9 * ys[1].float().abs().max().item()
+    rows = np.r_[0:40, m - 300:m - 260, m - 40:m]                           # first tile, and both tiles of the last round
+    check_matmul(ys[0][torch.from_numpy(rows).cuda()], x[rows], qw, s16, z16, b16, bits, g)
 
 
 def test_reference_acceptance_recipe():
