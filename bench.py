@@ -246,9 +246,31 @@ def extras_mixed_precision_model(torch, hip, QuantizedLinear, layers):
             "hipblaslt_fp16_token_us_linears_only": round(blas_us, 1)}
 
 
+def extras_eager_call(torch, hip, QuantizedLinear, layers):
+    """Host side of the drop-in: wall time per QuantizedLinear.forward call issued eagerly from Python (no graph),
+    M = 1, next to torch's own fp16 nn.Linear of the same shape.  The kernel itself runs for ~4 us."""
+    q = layers[0][0]
+    x = torch.randn(1, q.in_features, device="cuda", dtype=torch.float16)
+    lin = torch.nn.Linear(q.in_features, q.out_features, bias=False, device="cuda", dtype=torch.float16)
+
+    def wall(fn, n=3000):
+        for _ in range(300):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(n):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / n * 1e6
+
+    with torch.no_grad():
+        return {"quantized_linear_forward_us": round(wall(lambda: q(x)), 1),
+                "torch_fp16_linear_forward_us": round(wall(lambda: lin(x)), 1)}
+
+
 EXTRAS = {"decode": extras_decode, "decode_infinity_cache_hot": extras_decode_hot,
           "decode_other_formats": extras_decode_other_formats, "hipblaslt_fp16_decode": extras_hipblaslt_decode,
-          "prefill": extras_prefill, "quantize": extras_quantize, "mixed_precision_model": extras_mixed_precision_model}
+          "prefill": extras_prefill, "quantize": extras_quantize, "mixed_precision_model": extras_mixed_precision_model, "eager_call": extras_eager_call}
 
 
 def main():

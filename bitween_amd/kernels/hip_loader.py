@@ -56,8 +56,13 @@ def load():
     lib.bw_qgemm_workspace_bytes.restype = ctypes.c_size_t
     for name in ("bw_quantize_pack", "bw_quantize_pack_add", "bw_dequantize", "bw_qgemv", "bw_qgemm", "bw_qgemm_ws", "bw_qlinear"):
         getattr(lib, name).restype = i32
+    for name in ("bw_qgemv", "bw_qgemm", "bw_qlinear"):
+        _ENTRY[name] = getattr(lib, name)
     _lib = lib
     return lib
+
+
+_ENTRY = {}
 
 
 def _check(status, what):
@@ -76,7 +81,7 @@ def require_gpu(t, what):
 
 
 def _stream(device):
-    return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+    return torch._C._cuda_getCurrentRawStream(device.index if device.index is not None else torch.cuda.current_device())
 
 
 def quantize_pack(weight, bits, group_size, math_dtype, scale_dtype, zp_dtype, delta=None):
@@ -122,43 +127,80 @@ def dequantize(qweight, scale, zero_point, group_size, bits, out_dtype):
     return out
 
 
+def _raw_stream(index):
+    return torch._C._cuda_getCurrentRawStream(index)
+
+
+class _on_device:
+    """torch.cuda.device(), skipped when the device is already current (the common case: saves microseconds
+    on a call whose kernel runs for a few)."""
+    __slots__ = ("index", "ctx")
+
+    def __init__(self, device):
+        self.index = device.index if device.index is not None else torch.cuda.current_device()
+        self.ctx = None
+
+    def __enter__(self):
+        if torch.cuda.current_device() != self.index:
+            self.ctx = torch.cuda.device(self.index)
+            self.ctx.__enter__()
+        return self.index
+
+    def __exit__(self, *exc):
+        if self.ctx is not None:
+            self.ctx.__exit__(*exc)
+        return False
+
+
 def _matmul(entry, x, qweight, scale, zero_point, bias, bits, group_size):
-    require_gpu(x, entry)
+    if not x.is_cuda:
+        require_gpu(x, entry)
     if x.dim() != 2:
         raise ValueError("x must be [M, K]")
-    if qweight.dtype != torch.int32 or scale.dtype != torch.float16 or zero_point.dtype != torch.float16:
+    if qweight.dtype is not torch.int32 or scale.dtype is not torch.float16 or zero_point.dtype is not torch.float16:
         raise TypeError("qweight must be int32 and scale / zero_point float16 (the QuantizedLinear buffers)")
-    if x.dtype != torch.float16:
+    if x.dtype is not torch.float16:
         raise TypeError("x must be float16")
-    if bias is not None and bias.dtype != x.dtype:
+    if bias is not None and bias.dtype is not torch.float16:
         raise TypeError("bias must have the dtype of x")
-    x = x if x.stride(-1) == 1 and (x.stride(0) * 2) % 16 == 0 and x.data_ptr() % 16 == 0 else x.contiguous().clone()
-    qweight, scale, zero_point = qweight.contiguous(), scale.contiguous(), zero_point.contiguous()
+    ldx = x.stride(0)
+    if x.stride(1) != 1 or (ldx * 2) % 16 or x.data_ptr() % 16:
+        x = x.contiguous().clone()
+        ldx = x.stride(0)
+    if not qweight.is_contiguous():
+        qweight = qweight.contiguous()
+    if not scale.is_contiguous():
+        scale = scale.contiguous()
+    if not zero_point.is_contiguous():
+        zero_point = zero_point.contiguous()
     m, k = x.shape
     n, words = qweight.shape
     if words * (32 // bits) != k:
         raise ValueError(f"x has K={k} but qweight packs K={words * (32 // bits)}")
-    if scale.shape != (n, k // group_size) or zero_point.shape != scale.shape:
+    groups = k // group_size
+    if scale.shape != (n, groups) or zero_point.shape != (n, groups):
         raise ValueError("scale / zero_point must be [N, K // group_size]")
-    y = torch.empty((m, n), dtype=x.dtype, device=x.device)
+    y = torch.empty((m, n), dtype=torch.float16, device=x.device)
     if m == 0:
         return y
     lib = load()
-    bias_ptr = None if bias is None else bias.contiguous().data_ptr()
-    with torch.cuda.device(x.device):
+    bias_ptr = None
+    if bias is not None:
+        bias_ptr = (bias if bias.is_contiguous() else bias.contiguous()).data_ptr()
+    with _on_device(x.device) as index:
         if entry != "bw_qgemv" and m > 16:
             # prefill: give the library a split-K workspace when the shape wants one
             nbytes = lib.bw_qgemm_workspace_bytes(m, n, k, bits, group_size)
             ws = torch.empty(nbytes, dtype=torch.uint8, device=x.device) if nbytes else None
-            st = lib.bw_qgemm_ws(x.data_ptr(), _DTYPE_CODE[x.dtype], m, k, x.stride(0), qweight.data_ptr(),
-                                 scale.data_ptr(), zero_point.data_ptr(), bias_ptr, n, bits, group_size,
-                                 y.data_ptr(), n, None if ws is None else ws.data_ptr(), nbytes, _stream(x.device))
+            st = lib.bw_qgemm_ws(x.data_ptr(), BW_F16, m, k, ldx, qweight.data_ptr(), scale.data_ptr(),
+                                 zero_point.data_ptr(), bias_ptr, n, bits, group_size, y.data_ptr(), n,
+                                 None if ws is None else ws.data_ptr(), nbytes, _raw_stream(index))
             entry = "bw_qgemm_ws"
         else:
-            st = getattr(lib, entry)(x.data_ptr(), _DTYPE_CODE[x.dtype], m, k, x.stride(0), qweight.data_ptr(),
-                                     scale.data_ptr(), zero_point.data_ptr(), bias_ptr, n, bits, group_size,
-                                     y.data_ptr(), n, _stream(x.device))
-    _check(st, entry)
+            st = _ENTRY[entry](x.data_ptr(), BW_F16, m, k, ldx, qweight.data_ptr(), scale.data_ptr(),
+                               zero_point.data_ptr(), bias_ptr, n, bits, group_size, y.data_ptr(), n, _raw_stream(index))
+    if st:
+        _check(st, entry)
     return y
 
 

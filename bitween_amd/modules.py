@@ -65,8 +65,16 @@ class QuantizedLinear(nn.Module):
             self.bias = None
 
     def forward(self, x):
-        return QuantizedLinearFunction.apply(x, self.qweight, self.scale, self.zero_point, self.bias, self.bits,
-                                             self.group_size)
+        if x.requires_grad and torch.is_grad_enabled():
+            return QuantizedLinearFunction.apply(x, self.qweight, self.scale, self.zero_point, self.bias, self.bits,
+                                                 self.group_size)
+        # nothing to differentiate (the buffers never require grad): same arithmetic without the autograd node
+        shape = x.shape
+        x2 = x.reshape(-1, shape[-1])
+        if x2.dtype is not torch.float16:
+            x2 = x2.to(torch.float16)
+        y = _hip.quantized_matmul_hip(x2, self.qweight, self.scale, self.zero_point, self.bias, self.bits, self.group_size)
+        return y.view(*shape[:-1], self.out_features)
 
     @classmethod
     def from_float(cls, float_layer: nn.Linear, bits=8, group_size=32):
