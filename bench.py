@@ -246,6 +246,40 @@ def extras_mixed_precision_model(torch, hip, QuantizedLinear, layers):
             "hipblaslt_fp16_token_us_linears_only": round(blas_us, 1)}
 
 
+def extras_decode_fused_siblings(torch, hip, QuantizedLinear, layers):
+    """The headline step again with q/k/v and gate/up grouped by fuse_sibling_linears: the model still calls seven
+    modules per layer, four launches run (a launch costs ~2.5 us before its first byte arrives).  Not the headline:
+    the caller has to opt in.  Run last: it re-points the layers' buffers at concatenated copies."""
+    import bitween_amd
+    names = [n for n, _, _ in LLAMA7B_LINEARS]
+    blocks = []
+    for layer in layers:
+        blk = torch.nn.Module()
+        for n, q in zip(names, layer):
+            setattr(blk, n, q)
+        blocks.append(blk)
+    groups = sum(bitween_amd.fuse_sibling_linears(b) for b in blocks)
+    xs = {k: torch.randn(1, k, device="cuda", dtype=torch.float16) for k in (4096, 11008)}
+
+    def run():
+        with torch.no_grad():
+            for _ in range(2):
+                for blk in blocks:
+                    # a new tensor object per block and pass, as in a real model: a group only re-uses its result
+                    # for the very tensor it was computed from
+                    x_attn, x_o, x_mlp, x_down = xs[4096][:], xs[4096][:], xs[4096][:], xs[11008][:]
+                    blk.q_proj(x_attn), blk.k_proj(x_attn), blk.v_proj(x_attn)
+                    blk.o_proj(x_o)
+                    blk.gate_proj(x_mlp), blk.up_proj(x_mlp)
+                    blk.down_proj(x_down)
+
+    gr = graph_of(torch, run)
+    us = time_calls(torch, gr.replay, 20, 3) / (2 * len(blocks))
+    by = sum(decode_bytes(1, k, n, 4, 128) for _, k, n in LLAMA7B_LINEARS)
+    return {"groups_per_layer": groups // len(blocks), "launches_per_layer": len(names) - 3, "us_per_layer": round(us, 2),
+            "GBps": round(by / us / 1e3, 1), "pct_hbm_peak": round(100 * by / us / 1e3 / HBM_PEAK_GBPS, 1)}
+
+
 def extras_eager_call(torch, hip, QuantizedLinear, layers):
     """Host side of the drop-in: wall time per QuantizedLinear.forward call issued eagerly from Python (no graph),
     M = 1, next to torch's own fp16 nn.Linear of the same shape.  The kernel itself runs for ~4 us."""
@@ -270,7 +304,8 @@ def extras_eager_call(torch, hip, QuantizedLinear, layers):
 
 EXTRAS = {"decode": extras_decode, "decode_infinity_cache_hot": extras_decode_hot,
           "decode_other_formats": extras_decode_other_formats, "hipblaslt_fp16_decode": extras_hipblaslt_decode,
-          "prefill": extras_prefill, "quantize": extras_quantize, "mixed_precision_model": extras_mixed_precision_model, "eager_call": extras_eager_call}
+          "prefill": extras_prefill, "quantize": extras_quantize, "mixed_precision_model": extras_mixed_precision_model, "eager_call": extras_eager_call,
+          "decode_fused_siblings": extras_decode_fused_siblings}
 
 
 def main():

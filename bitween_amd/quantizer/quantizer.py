@@ -10,7 +10,7 @@ import copy
 
 import torch.nn as nn
 
-from ..modules import QuantizedLinear
+from ..modules import QuantizedLinear, fuse_sibling_linears
 from .func import _set_module
 
 
@@ -68,10 +68,12 @@ class Bitween:
 
     def quantize(self, evaluate_perplexity=False, eval_samples=100, rtn=False, trainable=False, calib_dataset="pile-10k",
                  nsamples=None, cache_to_disk=None, max_memory_mb=None, ignore_layers=None, batch_size=None,
-                 verbose=True, layer_config=None, **eval_kwargs):
+                 verbose=True, layer_config=None, fuse_siblings=False, **eval_kwargs):
         """Returns a deep copy of the model with its linear layers RTN-quantised.  As in the reference,
         trainable=False selects RTN whatever `rtn` says (quantizer.py:67).  `layer_config` (not in the
-        reference's signature) overrides bits / group_size per layer or block, see apply_precision_map."""
+        reference's signature) overrides bits / group_size per layer or block, see apply_precision_map;
+        `fuse_siblings=True` (also not in the reference) groups q/k/v and gate/up children so that they share
+        one launch, see modules.fuse_sibling_linears."""
         if trainable:
             raise NotImplementedError("trainable quantisation is outside this package (RTN only)")
         if evaluate_perplexity and self.tokenizer is not None and eval_samples > 0:
@@ -93,6 +95,8 @@ class Bitween:
                     print(f"  - Quantizing layer: {name}")
                 bits, group_size = _precision_for(name, layer_config or {}, (self.bits, self.group_size))
                 _set_module(quantized_model, name, QuantizedLinear.from_float(module, bits, group_size))
+            if fuse_siblings:
+                fuse_sibling_linears(quantized_model)
             if verbose:
                 print("--- Quantization complete ---")
         finally:

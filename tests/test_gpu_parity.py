@@ -362,6 +362,79 @@ def test_precision_map_and_perturbed_quantize():
         assert np.array_equal(_bits_of(s), s_o.astype(np.float16).view(np.uint16))
 
 
+def test_sibling_linears_share_a_launch():
+    """fuse_sibling_linears: q/k/v (and gate/up) read one input; grouped, the first call computes all of them and
+    the siblings return slices.  Results, state_dict and behaviour after copies / in-place input edits must not change."""
+    import copy
+    import io
+    import bitween_amd
+    torch.manual_seed(11)
+
+    model = _QkvBlock().half().cuda()
+    qm = bitween_amd.Bitween(model, bits=4, group_size=128).quantize(verbose=False)
+    x = torch.randn(3, 256, device="cuda", dtype=torch.float16)
+    with torch.no_grad():
+        before = [t.clone() for t in qm(x)]
+        sd_before = {k: v.clone() for k, v in qm.state_dict().items()}
+        assert bitween_amd.fuse_sibling_linears(qm) == 1
+        calls = []
+        real = bitween_amd.kernels.hip_loader.quantized_matmul_hip
+        bitween_amd.modules._hip.quantized_matmul_hip = lambda *a, **k: (calls.append(a[1].shape[0]), real(*a, **k))[1]
+        try:
+            after = qm(x)
+            assert calls == [256]                                   # one launch over the 128 + 64 + 64 rows
+            for a, b in zip(after, before):
+                assert torch.equal(a, b)
+            x2 = x.clone()
+            r1 = qm.q_proj(x2)
+            x2.mul_(2.0)                                            # same tensor object, new contents
+            r2 = qm.k_proj(x2)
+            assert torch.equal(r2, real(x2, qm.k_proj.qweight, qm.k_proj.scale, qm.k_proj.zero_point, qm.k_proj.bias, 4, 128))
+            assert calls[-2:] == [256, 256] and r1.shape == (3, 128)
+        finally:
+            bitween_amd.modules._hip.quantized_matmul_hip = real
+        # siblings fed different inputs (cross-attention style) stop being grouped after a few wasted launches
+        cross = copy.deepcopy(qm)
+        outs = []
+        for i in range(8):
+            xa, xb = torch.randn_like(x), torch.randn_like(x)
+            outs.append((cross.q_proj(xa), cross.k_proj(xb), xa, xb))
+        assert cross.q_proj.__dict__["_sibling_group"].wasted >= 4
+        qa, kb, xa, xb = outs[-1]
+        assert torch.equal(qa, real(xa, qm.q_proj.qweight, qm.q_proj.scale, qm.q_proj.zero_point, qm.q_proj.bias, 4, 128))
+        assert torch.equal(kb, real(xb, qm.k_proj.qweight, qm.k_proj.scale, qm.k_proj.zero_point, qm.k_proj.bias, 4, 128))
+        sd_after = qm.state_dict()
+        assert set(sd_after) == set(sd_before) and all(torch.equal(sd_after[k], sd_before[k]) for k in sd_before)
+        # copies and pickles keep working (fused when the views survive, per layer otherwise)
+        for clone in (copy.deepcopy(qm), torch.load(io.BytesIO(_saved(qm)), weights_only=False)):
+            for a, b in zip(clone(x), before):
+                assert torch.equal(a, b)
+        # gradients bypass the group
+        xg = x.clone().requires_grad_(True)
+    y = qm.q_proj(xg)
+    y.float().sum().backward()
+    assert xg.grad is not None and xg.grad.shape == x.shape
+
+
+class _QkvBlock(torch.nn.Module):
+    def __init__(self):
+        super().__init__()
+        self.q_proj = torch.nn.Linear(256, 128)
+        self.k_proj = torch.nn.Linear(256, 64)
+        self.v_proj = torch.nn.Linear(256, 64)
+        self.o_proj = torch.nn.Linear(128, 256)
+
+    def forward(self, x):
+        return self.q_proj(x), self.k_proj(x), self.v_proj(x)
+
+
+def _saved(model):
+    import io
+    buf = io.BytesIO()
+    torch.save(model, buf)
+    return buf.getvalue()
+
+
 def test_error_conventions_on_gpu():
     import bitween_amd
     w = torch.zeros(4, 100, device="cuda")
