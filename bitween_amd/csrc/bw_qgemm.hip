@@ -328,12 +328,15 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
     }
     // acc[i][j][r] = y[m0 + 16 i + nl][n0 + 16 j + 4 kq + r]
     if (partial) {
-        // float32 partial tile to this workgroup's block of the workspace (tile-shaped, so no bounds to check)
+        // float32 partial tile to this workgroup's block of the workspace (tile-shaped; rows past M are never
+        // read back, so they are not written either)
         float* blk = a.ws + (size_t)run * (BM * BN) + wave * (NT * 16) + 4 * kq;
 #pragma unroll
-        for (int j = 0; j < NT; j++)
+        for (int i = 0; i < MT; i++) {
+            if (m0 + 16 * i + nl >= a.M) continue;
 #pragma unroll
-            for (int i = 0; i < MT; i++) *reinterpret_cast<f4*>(blk + (16 * i + nl) * BN + 16 * j) = acc[i][j];
+            for (int j = 0; j < NT; j++) *reinterpret_cast<f4*>(blk + (16 * i + nl) * BN + 16 * j) = acc[i][j];
+        }
         return;
     }
 #pragma unroll
@@ -556,6 +559,15 @@ extern "C" int bw_qgemm(const void* x, int act_dtype, int64_t M, int64_t K, int6
 extern "C" int bw_qlinear(const void* x, int act_dtype, int64_t M, int64_t K, int64_t ldx, const int32_t* qweight,
                           const void* scale16, const void* zp16, const void* bias, int64_t N, int bits, int group,
                           void* y, int64_t ldy, void* stream) {
-    if (M >= 1 && M <= 16) return bw_qgemv(x, act_dtype, M, K, ldx, qweight, scale16, zp16, bias, N, bits, group, y, ldy, stream);
+    // up to 48 rows the HBM-bound kernel, 16 rows per launch (the later launches find the weights in L2),
+    // beats a mostly empty 128-row MFMA tile
+    if (M >= 1 && M <= 48 && act_dtype == BW_F16) {
+        for (int64_t m0 = 0; m0 < M; m0 += 16) {
+            const int st = bw_qgemv((const _Float16*)x + m0 * ldx, act_dtype, M - m0 < 16 ? M - m0 : 16, K, ldx, qweight, scale16,
+                                    zp16, bias, N, bits, group, (_Float16*)y + m0 * ldy, ldy, stream);
+            if (st != BW_OK) return st;
+        }
+        return BW_OK;
+    }
     return bw_qgemm(x, act_dtype, M, K, ldx, qweight, scale16, zp16, bias, N, bits, group, y, ldy, stream);
 }

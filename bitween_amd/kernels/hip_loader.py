@@ -188,8 +188,9 @@ def _matmul(entry, x, qweight, scale, zero_point, bias, bits, group_size):
     if bias is not None:
         bias_ptr = (bias if bias.is_contiguous() else bias.contiguous()).data_ptr()
     with _on_device(x.device) as index:
-        if entry != "bw_qgemv" and m > 16:
-            # prefill: give the library a split-K workspace when the shape wants one
+        if (entry == "bw_qgemm" and m > 16) or (entry == "bw_qlinear" and m > 48):
+            # prefill (bw_qlinear itself keeps M <= 48 on the decode kernel): give the library a split-K
+            # workspace when the shape wants one
             nbytes = lib.bw_qgemm_workspace_bytes(m, n, k, bits, group_size)
             ws = torch.empty(nbytes, dtype=torch.uint8, device=x.device) if nbytes else None
             st = lib.bw_qgemm_ws(x.data_ptr(), BW_F16, m, k, ldx, qweight.data_ptr(), scale.data_ptr(),

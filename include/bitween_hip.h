@@ -93,7 +93,8 @@ int bw_dequantize(const int32_t* qweight, const void* scale, int scale_dtype, co
  *   bias   [N] of act_dtype or NULL
  * bw_qgemv: decode path, 1 <= M <= 16, HBM-bound, no workspace.
  * bw_qgemm: prefill path, any M >= 1, MFMA-bound.
- * bw_qlinear: picks between them by M (what the Python forward calls). */
+ * bw_qlinear: picks between them by M (what the Python forward calls): the decode kernel, 16 rows per
+ *             launch, up to M = 48; the prefill kernel (without a workspace) beyond. */
 int bw_qgemv(const void* x, int act_dtype, int64_t M, int64_t K, int64_t ldx,
              const int32_t* qweight, const void* scale16, const void* zp16, const void* bias,
              int64_t N, int bits, int group, void* y, int64_t ldy, void* stream);
