@@ -19,6 +19,7 @@ _lib = None
 BW_F16, BW_BF16, BW_F32, BW_I32 = 0, 1, 2, 3
 _DTYPE_CODE = {torch.float16: BW_F16, torch.bfloat16: BW_BF16, torch.float32: BW_F32, torch.int32: BW_I32}
 
+ABI_VERSION = 2            # what bw_abi_version() of a matching library returns
 ENTRY_POINTS = ("bw_abi_version", "bw_strerror", "bw_quantize_pack", "bw_quantize_pack_add", "bw_dequantize", "bw_qgemv", "bw_qgemm",
                 "bw_qgemm_ws", "bw_qgemm_workspace_bytes", "bw_qlinear")
 
@@ -43,6 +44,9 @@ def load():
     lib = ctypes.CDLL(_LIB_PATH)
     vp, i64, i32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int
     lib.bw_abi_version.restype = i32
+    if lib.bw_abi_version() != ABI_VERSION:
+        raise BitweenHipError(f"{_LIB_PATH} has ABI version {lib.bw_abi_version()}, this package expects {ABI_VERSION}: "
+                              "rebuild it with `python -m bitween_amd.csrc.build`")
     lib.bw_strerror.restype = ctypes.c_char_p
     lib.bw_strerror.argtypes = [i32]
     lib.bw_quantize_pack.argtypes = [vp, i32, i32, i64, i64, i64, i32, i32, vp, vp, i32, vp, i32, vp]
