@@ -206,11 +206,10 @@ def extras_quantize(torch, hip, QuantizedLinear, layers):
 def extras_mixed_precision_model(torch, hip, QuantizedLinear, layers):
     """The linears of a 32-layer, hidden-4096, MLP-11008 decoder with the mixed recipe: attention 8-bit g128,
     gate/up/down 4-bit g128, down_proj of layers 0, 1, 30, 31 2-bit g32.  Reports the time to quantise all of
-    them (fp16 in) and the time of one decode token through all of them (M = 1, one HIP graph, nothing but the
+    them (13 GB of fp16 in) and the time of one decode token through all of them (M = 1, one HIP graph, nothing but the
     quantised linears: no attention, norms, embeddings or lm_head), next to fp16 hipBLASLt on the same shapes."""
     nlayers, low = 32, (0, 1, 30, 31)
     gen = torch.Generator(device="cuda").manual_seed(5)
-    src = {(k, n): (torch.randn(n, k, device="cuda", generator=gen) * 0.02).half() for _, k, n in LLAMA7B_LINEARS[3:]}
     plan = []
     for li in range(nlayers):
         for name, k, n in LLAMA7B_LINEARS:
@@ -220,14 +219,19 @@ def extras_mixed_precision_model(torch, hip, QuantizedLinear, layers):
                 plan.append((k, n, 2, 32))
             else:
                 plan.append((k, n, 4, 128))
-    # quantise: one launch per linear, same random source per shape (the values do not change the timing)
-    torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    e0.record()
-    packed = [hip.quantize_pack(src[(k, n)], b, g, torch.float32, torch.float16, torch.float16) for k, n, b, g in plan]
-    e1.record()
-    torch.cuda.synchronize()
-    quant_ms = e0.elapsed_time(e1)
+    # quantise: one launch per linear, every linear its own fp16 weights (13 GB in all: nothing is cache-resident).
+    # The first pass only warms torch's allocator (4.3 GB of fresh hipMalloc would otherwise be what is timed).
+    srcs = [torch.empty(n, k, device="cuda", dtype=torch.float16).normal_(0, 0.02, generator=gen) for k, n, _, _ in plan]
+    for timed in (False, True):
+        packed = None
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        packed = [hip.quantize_pack(w, b, g, torch.float32, torch.float16, torch.float16) for w, (k, n, b, g) in zip(srcs, plan)]
+        e1.record()
+        torch.cuda.synchronize()
+        quant_ms = e0.elapsed_time(e1)
+    del srcs
     weights = sum(k * n for k, n, _, _ in plan)
     xs = {k: torch.randn(1, k, device="cuda", dtype=torch.float16) for k in (4096, 11008)}
     gr = graph_of(torch, lambda: [hip.quantized_gemv_hip(xs[k], qw, s, z, None, b, g)
@@ -235,6 +239,33 @@ def extras_mixed_precision_model(torch, hip, QuantizedLinear, layers):
     tok_us = time_calls(torch, gr.replay, 20, 3)
     by = sum(decode_bytes(1, k, n, b, g) for k, n, b, g in plan)
     del gr
+    # the same token with q/k/v and gate/up sharing a launch (fuse_sibling_linears): 7 module calls, 4 launches per layer
+    import bitween_amd
+    names = [nm for nm, _, _ in LLAMA7B_LINEARS]
+    blocks = []
+    for li in range(nlayers):
+        blk = torch.nn.Module()
+        for j, nm in enumerate(names):
+            k, n, b, g = plan[li * 7 + j]
+            q = QuantizedLinear(k, n, bits=b, group_size=g, bias=False)
+            q._buffers["qweight"], q._buffers["scale"], q._buffers["zero_point"] = packed[li * 7 + j]
+            setattr(blk, nm, q)
+        bitween_amd.fuse_sibling_linears(blk)
+        blocks.append(blk)
+    del packed
+
+    def fused_token():
+        with torch.no_grad():
+            for blk in blocks:
+                xa, xo, xm, xd = xs[4096][:], xs[4096][:], xs[4096][:], xs[11008][:]
+                blk.q_proj(xa), blk.k_proj(xa), blk.v_proj(xa)
+                blk.o_proj(xo)
+                blk.gate_proj(xm), blk.up_proj(xm)
+                blk.down_proj(xd)
+
+    gr = graph_of(torch, fused_token)
+    fused_us = time_calls(torch, gr.replay, 20, 3)
+    del gr, blocks
     # fp16 hipBLASLt over the same shapes: one set of fp16 weights per layer would be 13 GB; rotate 4 layers' worth
     w16 = [[torch.randn(n, k, device="cuda", dtype=torch.float16) for _, k, n in LLAMA7B_LINEARS] for _ in range(4)]
     gr = graph_of(torch, lambda: [torch.matmul(xs[w.shape[1]], w.T) for li in range(nlayers) for w in w16[li % 4]])
@@ -243,6 +274,8 @@ def extras_mixed_precision_model(torch, hip, QuantizedLinear, layers):
             "quantize_Gweights_per_s": round(weights / quant_ms / 1e6, 1),
             "decode_token_us_linears_only": round(tok_us, 1), "decode_tokens_per_s_linears_only": round(1e6 / tok_us, 1),
             "decode_GBps": round(by / tok_us / 1e3, 1), "decode_bytes_per_token": by,
+            "decode_token_us_fused_siblings": round(fused_us, 1),
+            "decode_tokens_per_s_fused_siblings": round(1e6 / fused_us, 1),
             "hipblaslt_fp16_token_us_linears_only": round(blas_us, 1)}
 
 
