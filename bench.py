@@ -450,7 +450,7 @@ def main():
                      "frac": round(bytes_per_launch / (us_per_launch * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4),
                      # HBM bytes per launch from rocprofv3 FETCH_SIZE / WRITE_SIZE, scaled by the same counters on
                      # a plain copy (profiles/qgemv_w4g128_llama7b_decode_M1_hbm_traffic.txt); not measurable live
-                     "traffic": 15531000 if m == 1 else None, "kernel": "qgemv_w4g128_kernel" if m <= 2 else "qgemv_kernel<4,128>", "avg_launch_us": round(us_per_launch, 3),
+                     "traffic": 15531000 if m == 1 else None, "kernel": "qgemv_w4_kernel<128>" if m <= 2 else "qgemv_kernel<4,128>", "avg_launch_us": round(us_per_launch, 3),
                      "bytes_per_launch": round(bytes_per_launch)},
     }
 

@@ -217,36 +217,47 @@ __global__ __launch_bounds__((64 * GemvCfg<BITS, GROUP, MT>::MAX_WAVES)) void qg
     }
 }
 
-// ---- 4-bit, group 128, M <= 2: integer operands, zero point taken out of the inner loop ----------------
+// ---- 4-bit, M <= 2: integer operands, scale and zero point taken out of the inner loop -------------------
 //
 // A masked packed word is already a float16: bits 0-3 of a half are the subnormal q * 2^-24, bits 4-7 the
 // subnormal q * 2^-20, and the matrix core keeps subnormal inputs exactly.  So a word unpacks with one shift
-// and four ANDs, the products x * q are exact, and per group (= per chunk)
+// and four ANDs, the products x * q are exact, and per group
 //     sum_k x_k (q_k - z) = 2^24 * (E + O / 16) - z * S,     S = sum_k x_k,
 // with E and O the accumulators of the even and the odd nibbles.  S comes from the lanes that stage x (a
-// 16-lane reduction per chunk and row), so the inner loop holds no per-weight arithmetic at all; that
+// cross-lane reduction per group and row), so the inner loop holds no per-weight arithmetic at all; that
 // staging cost grows with M, which is why wider activation tiles stay on the kernel above.
+//
+// A chunk is 128 weights of each row.  With groups of 64 or 32 it spans 2 or 4 groups, but an MFMA adds up
+// all of a chunk's k.  The MFMA rows an M <= 2 activation tile leaves idle separate them: row m * NGC + g of
+// the staged tile holds x[m] with everything outside group g of the chunk zeroed, so output row m * NGC + g is
+// the partial sum of group g alone and gets that group's scale and zero point.
 // Results agree with the per-weight float16 dequantisation to float32 rounding: a one-hot x still returns
 // the reference's W16 column bit for bit.
 BW_DEV float half_of(uint32_t word, int hi) {
     return (float)__builtin_bit_cast(_Float16, (uint16_t)(hi ? word >> 16 : word));
 }
 
-BW_DEV float row16_sum(float v) {
-    // sum over the 16 lanes of a DPP row; every lane of the row ends up with the total
-    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true));
-    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, true));
-    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xF, 0xF, true));
-    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x140, 0xF, 0xF, true));
+// sum over aligned runs of LANES (4, 8 or 16) lanes; every lane of a run ends up with the run's total
+template <int LANES>
+BW_DEV float lanes_sum(float v) {
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true));   // quad_perm [1,0,3,2]
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, true));   // quad_perm [2,3,0,1]
+    if constexpr (LANES >= 8)
+        v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xF, 0xF, true));   // row_half_mirror
+    if constexpr (LANES >= 16)
+        v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x140, 0xF, 0xF, true));   // row_mirror
     return v;
 }
 
-template <int MT, int KB>
-__global__ __launch_bounds__(1024) void qgemv_w4g128_kernel(const GemvArgs a) {
-    static_assert(MT == 1 || MT == 2 || MT == 4, "rows of one MFMA row quad");
+template <int GROUP, int MT, int KB>
+__global__ __launch_bounds__(1024) void qgemv_w4_kernel(const GemvArgs a) {
+    constexpr int NGC = 128 / GROUP;                      // groups per chunk
+    constexpr int ROWS = MT * NGC;                        // MFMA rows in use: (m, group of the chunk)
+    static_assert(ROWS <= 4, "the outputs must fit the four rows the lanes with kq == 0 hold");
+    constexpr int GL = GROUP / 8;                         // staging lanes per group (8 halves each)
     constexpr int UPR = KB * 16;                          // 8-half units per activation row and round
     constexpr int XL = (MT * UPR + 63) / 64;              // unit loads per lane and round
-    constexpr int ROW_BYTES = KB * 256 + 16, X_BYTES = MT * ROW_BYTES;
+    constexpr int ROW_BYTES = KB * 256 + 16, X_BYTES = ROWS * ROW_BYTES;
     constexpr uint32_t kOob = 0x80000000u;
     extern __shared__ __attribute__((aligned(16))) char smem[];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nwaves = blockDim.x >> 6;
@@ -261,29 +272,39 @@ __global__ __launch_bounds__(1024) void qgemv_w4g128_kernel(const GemvArgs a) {
     const __amdgpu_buffer_rsrc_t rw = make_rsrc(a.qweight, a.w_bytes), rx = make_rsrc(a.x, a.x_bytes),
                                  rs = make_rsrc(a.scale, a.meta_bytes), rz = make_rsrc(a.zp, a.meta_bytes);
 
-    // scales / zero points of the 16 rows: thread e takes row (e / 32) % 16, column e % 32 + 32 * (e / 512)
+    // Scales / zero points of the 16 rows: entry e = tid + j * blockDim is row (e / 32) % 16, column
+    // e % 32 + 32 * (e / 512).  The first ME entries of a thread are requested ahead of x and the weights
+    // (loads return in order: a request made later only comes back after the whole weight batch); shapes
+    // with more entries than that finish in a loop behind them.
+    constexpr int ME = 128 / GROUP;
     const uint32_t meta_base = (uint32_t)n0 * a.groups * 2;
-    const int mr = (tid >> 5) & 15, mc = (tid & 31) + 32 * (tid >> 9);
-    uint32_t ms = 0, mz = 0;
-    if (mc < gcols) {
-        const uint32_t off = mc < a.groups ? meta_base + (mr * a.groups + mc) * 2 : kOob;
-        ms = __builtin_amdgcn_raw_buffer_load_b16(rs, off, 0, 0);
-        mz = __builtin_amdgcn_raw_buffer_load_b16(rz, off, 0, 0);
+    const int meta_entries = 16 * gcols;
+    auto meta_off = [&](int e) {
+        const int r = (e >> 5) & 15, c = (e & 31) + 32 * (e >> 9);
+        return c < a.groups ? meta_base + (r * a.groups + c) * 2 : kOob;
+    };
+    auto meta_slot = [&](int e) { return ((e >> 5) & 15) * GP + (e & 31) + 32 * (e >> 9); };
+    uint32_t ms[ME], mz[ME];
+#pragma unroll
+    for (int j = 0; j < ME; j++) {
+        ms[j] = mz[j] = 0;
+        if ((wave + j * nwaves) * 64 < meta_entries) {          // wave-uniform
+            const uint32_t off = meta_off(tid + j * (int)blockDim.x);
+            ms[j] = __builtin_amdgcn_raw_buffer_load_b16(rs, off, 0, 0);
+            mz[j] = __builtin_amdgcn_raw_buffer_load_b16(rz, off, 0, 0);
+        }
     }
 
     const uint32_t w_lane = (uint32_t)(n0 + nl) * a.row_bytes + kq * 16;
-    // where this lane's unit u = lane + 64 i of the round goes: row u / UPR, unit ku = u % UPR
+    // where this lane's unit u = lane + 64 i of the round goes: activation row u / UPR, unit ku = u % UPR
     uint32_t x_off[XL], x_dst[XL];
 #pragma unroll
     for (int i = 0; i < XL; i++) {
         const int u = lane + 64 * i, m = u / UPR, ku = u % UPR;
         x_off[i] = m < a.M ? (uint32_t)(m * a.ldx + ku * 8) * 2 : kOob;
-        x_dst[i] = m * ROW_BYTES + (ku >> 2) * 64 + (ku & 3) * 8;
+        x_dst[i] = m * NGC * ROW_BYTES + (ku >> 2) * 64 + (ku & 3) * 8;
     }
     u4 xr[XL], wr[KB];
-    // Requests of a round: the weights, then x.  Every workgroup of the grid reads the same few KB of x at
-    // the same time and those hot lines come back late; loads return in order, so weights queued behind
-    // them would be held up too.  The unpack below needs only the weights and runs while x is on its way.
     // x before the weights: loads return in order and the staging of x should overlap the weight stream
     auto issue = [&](int c0) {
 #pragma unroll
@@ -301,25 +322,30 @@ __global__ __launch_bounds__(1024) void qgemv_w4g128_kernel(const GemvArgs a) {
     int c0 = wave * KB;
     issue(c0);
 
-    if (mc < gcols) meta[mr * GP + mc] = ms | (mz << 16);
-    for (int e = tid + blockDim.x; e < 16 * gcols; e += blockDim.x) {   // more pairs than threads
-        const int r = (e >> 5) & 15, c = (e & 31) + 32 * (e >> 9);
-        const uint32_t off = c < a.groups ? meta_base + (r * a.groups + c) * 2 : kOob;
+#pragma unroll
+    for (int j = 0; j < ME; j++) {
+        const int e = tid + j * (int)blockDim.x;
+        if (e < meta_entries) meta[meta_slot(e)] = ms[j] | (mz[j] << 16);
+    }
+    for (int e = tid + ME * (int)blockDim.x; e < meta_entries; e += blockDim.x) {   // more entries than that
+        const uint32_t off = meta_off(e);
         const uint32_t s2 = __builtin_amdgcn_raw_buffer_load_b16(rs, off, 0, 0);
         const uint32_t z2 = __builtin_amdgcn_raw_buffer_load_b16(rz, off, 0, 0);
-        meta[r * GP + c] = s2 | (z2 << 16);
+        meta[meta_slot(e)] = s2 | (z2 << 16);
     }
     __syncthreads();
 
     float acc[MT];
 #pragma unroll
     for (int r = 0; r < MT; r++) acc[r] = 0.f;
-    const char* xrow = xs + (nl < MT ? nl : MT - 1) * ROW_BYTES + kq * 64;
+    const char* xrow = xs + (nl < ROWS ? nl : ROWS - 1) * ROW_BYTES + kq * 64;
     const uint32_t* mrow = meta + nl * GP;
+    const int my_group = ((lane & 15) * 8) / GROUP;       // group of the chunk this lane's staged unit lies in
     constexpr uint32_t kEven = 0x000F000Fu, kOdd = 0x00F000F0u;
     while (true) {
         // stage the round's activations: even-k quartets (x0,x4,x2,x6) and odd-k quartets (x1,x5,x3,x7) of
-        // every 8 values, in the order the masks below emit the nibbles; and -2^-24 * sum(x) per chunk
+        // every 8 values, in the order the masks below emit the nibbles, into the row of their group (zeros
+        // into the rows of the chunk's other groups); and -2^-24 * sum(x) per group
         float nsum[XL];
 #pragma unroll
         for (int i = 0; i < XL; i++) {
@@ -330,8 +356,13 @@ __global__ __launch_bounds__(1024) void qgemv_w4g128_kernel(const GemvArgs a) {
             od[0] = __builtin_amdgcn_perm(v[2], v[0], 0x07060302u);
             od[1] = __builtin_amdgcn_perm(v[3], v[1], 0x07060302u);
             if (MT * UPR >= 64 * (i + 1) || lane + 64 * i < MT * UPR) {
-                *reinterpret_cast<u2*>(xs + x_dst[i]) = ev;
-                *reinterpret_cast<u2*>(xs + x_dst[i] + 32) = od;
+#pragma unroll
+                for (int g = 0; g < NGC; g++) {
+                    const bool mine = NGC == 1 || g == my_group;
+                    char* dst = xs + x_dst[i] + g * ROW_BYTES;
+                    *reinterpret_cast<u2*>(dst) = mine ? ev : u2{0u, 0u};
+                    *reinterpret_cast<u2*>(dst + 32) = mine ? od : u2{0u, 0u};
+                }
             }
             float t = 0.f;
 #pragma unroll
@@ -340,10 +371,9 @@ __global__ __launch_bounds__(1024) void qgemv_w4g128_kernel(const GemvArgs a) {
                 t -= (float)p[0];
                 t -= (float)p[1];
             }
-            nsum[i] = row16_sum(t) * 0x1p-24f;
+            nsum[i] = lanes_sum<GL>(t) * 0x1p-24f;
         }
         __builtin_amdgcn_wave_barrier();
-        const uint32_t* mp = mrow + c0;
 #pragma unroll
         for (int b = 0; b < KB; b++) {
             const u4 w = wr[b];
@@ -362,15 +392,18 @@ __global__ __launch_bounds__(1024) void qgemv_w4g128_kernel(const GemvArgs a) {
             po = __builtin_amdgcn_mfma_f32_16x16x32_f16(xp[2], __builtin_bit_cast(h8, o0), po, 0, 0, 0);
             pe = __builtin_amdgcn_mfma_f32_16x16x32_f16(xp[1], __builtin_bit_cast(h8, e1), pe, 0, 0, 0);
             po = __builtin_amdgcn_mfma_f32_16x16x32_f16(xp[3], __builtin_bit_cast(h8, o1), po, 0, 0, 0);
-            const uint32_t sz = mp[b];
-            const float sf = half_of(sz, 0), zf = half_of(sz, 1);
 #pragma unroll
-            for (int r = 0; r < MT; r++) {
-                // unit (row r, chunk b) of the round was reduced in the DPP row that starts at lane u % 64 of load u / 64
-                const int u = r * UPR + 16 * b;
-                const float ns = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, nsum[u / 64]), u % 64));
-                const float t = __builtin_fmaf(po[r], 0.0625f, pe[r]);
-                acc[r] = __builtin_fmaf(sf, __builtin_fmaf(zf, ns, t), acc[r]);
+            for (int g = 0; g < NGC; g++) {
+                const uint32_t sz = mrow[(c0 + b) * NGC + g];
+                const float sf = half_of(sz, 0), zf = half_of(sz, 1);
+#pragma unroll
+                for (int m = 0; m < MT; m++) {
+                    // the sum of (row m, chunk b, group g) sits in the lanes that staged it: unit m * UPR + 16 b + g * GL
+                    const int u = m * UPR + 16 * b + g * GL, r = m * NGC + g;
+                    const float ns = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, nsum[u / 64]), u % 64));
+                    const float t = __builtin_fmaf(po[r], 0.0625f, pe[r]);
+                    acc[m] = __builtin_fmaf(sf, __builtin_fmaf(zf, ns, t), acc[m]);
+                }
             }
         }
         c0 += nwaves * KB;
@@ -379,7 +412,7 @@ __global__ __launch_bounds__(1024) void qgemv_w4g128_kernel(const GemvArgs a) {
         issue(c0);
     }
 
-    // acc[r] = 2^-24 * partial y[m = r][n = nl] in the lanes with kq == 0
+    // acc[m] = 2^-24 * partial y[m][n = nl] in the lanes with kq == 0
     if (kq == 0) {
 #pragma unroll
         for (int r = 0; r < MT; r++) red[(wave * MT + r) * 16 + nl] = acc[r];
@@ -400,16 +433,17 @@ __global__ __launch_bounds__(1024) void qgemv_w4g128_kernel(const GemvArgs a) {
     }
 }
 
-template <int MT, int KB>
-int launch_w4g128_kb(const GemvArgs& a, hipStream_t stream) {
+template <int GROUP, int MT, int KB>
+int launch_w4_kb(const GemvArgs& a, hipStream_t stream) {
     int nwaves = (a.nchunks + KB - 1) / KB;
     if (nwaves > 16) nwaves = 16;
     const int gcols = (a.groups + 31) & ~31;
-    const size_t lds = (size_t)((16 * (gcols + 1) * 4 + 15) & ~15) + (size_t)nwaves * (MT * (KB * 256 + 16) + MT * 64);
-    auto kern = qgemv_w4g128_kernel<MT, KB>;
+    const size_t lds = (size_t)((16 * (gcols + 1) * 4 + 15) & ~15) +
+                       (size_t)nwaves * (MT * (128 / GROUP) * (KB * 256 + 16) + MT * 64);
+    auto kern = qgemv_w4_kernel<GROUP, MT, KB>;
     static bool attr_set = false;                          // per instantiation; benign if raced
+    if (lds > 150 * 1024) return BW_EUNSUPPORTED;
     if (lds > 64 * 1024 && !attr_set) {
-        if (lds > 150 * 1024) return BW_EUNSUPPORTED;
         if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) != hipSuccess)
             return BW_ELAUNCH;
         attr_set = true;
@@ -418,14 +452,12 @@ int launch_w4g128_kb(const GemvArgs& a, hipStream_t stream) {
     return hipGetLastError() == hipSuccess ? BW_OK : BW_ELAUNCH;
 }
 
-template <int MT>
-int launch_w4g128(const GemvArgs& a, hipStream_t stream) {
-    static const int force_kb = getenv("BW_GEMV_KB") ? atoi(getenv("BW_GEMV_KB")) : 0;
-    int kb = (a.nchunks <= 32 && a.N <= 4096) ? 2 : 4;
-    if (force_kb) kb = force_kb;
-    if (kb >= 8) return launch_w4g128_kb<MT, 8>(a, stream);
-    if (kb >= 4) return launch_w4g128_kb<MT, 4>(a, stream);
-    return launch_w4g128_kb<MT, 2>(a, stream);
+// BW_EUNSUPPORTED = the scale / zero-point block does not fit LDS; the caller falls back
+template <int GROUP, int MT>
+int launch_w4(const GemvArgs& a, hipStream_t stream) {
+    // chunks a wave has in flight per round: 2 for the small square projections (more, shorter waves), else 4
+    if (a.nchunks <= 32 && a.N <= 4096) return launch_w4_kb<GROUP, MT, 2>(a, stream);
+    return launch_w4_kb<GROUP, MT, 4>(a, stream);
 }
 
 constexpr int kLdsBudget = 150 * 1024;
@@ -454,7 +486,6 @@ int launch_gemv_kb(const GemvArgs& a, hipStream_t stream) {
 template <int BITS, int GROUP, int MT>
 int launch_gemv_mt(const GemvArgs& a, hipStream_t stream) {
     using C = GemvCfg<BITS, GROUP, MT>;
-    static const int force_kb = getenv("BW_GEMV_KB") ? atoi(getenv("BW_GEMV_KB")) : 0;
     // Chunks per wave and round, from timing Llama-shaped layers on MI355X: short rows want many small
     // waves (more requests in flight early), wide activation tiles want small batches (LDS, registers);
     // never more than ~16 KB of staged activations per wave.
@@ -463,7 +494,6 @@ int launch_gemv_mt(const GemvArgs& a, hipStream_t stream) {
     if (MT >= 8) kb = a.nchunks <= 32 ? 1 : 2;
     else kb = (a.nchunks <= 32 && a.N < 8192) ? 2 : 4;
     if (kb > fit) kb = fit >= 4 ? 4 : (fit >= 2 ? 2 : 1);
-    if (force_kb) kb = force_kb;
     if (kb >= 8) return launch_gemv_kb<BITS, GROUP, MT, 8>(a, stream);
     if (kb >= 4) return launch_gemv_kb<BITS, GROUP, MT, 4>(a, stream);
     if (kb >= 2) return launch_gemv_kb<BITS, GROUP, MT, 2>(a, stream);
@@ -472,9 +502,14 @@ int launch_gemv_mt(const GemvArgs& a, hipStream_t stream) {
 
 template <int BITS, int GROUP>
 int launch_gemv(const GemvArgs& a, hipStream_t stream) {
-    if constexpr (BITS == 4 && GROUP == 128) {
-        if (a.M == 1) return launch_w4g128<1>(a, stream);
-        if (a.M == 2) return launch_w4g128<2>(a, stream);
+    if constexpr (BITS == 4) {
+        // rows of the MFMA tile in use = M * groups per chunk, at most 4.  With groups of 64 the doubled
+        // activation rows cost more than the cheaper unpack saves until the weights reach about 16 MiB.
+        const bool pays = GROUP != 64 || (int64_t)a.N * a.K > (int64_t)1 << 25;
+        if (a.M * (128 / GROUP) <= 4 && a.M <= 2 && pays) {
+            const int st = a.M == 1 ? launch_w4<GROUP, 1>(a, stream) : launch_w4<GROUP, (GROUP >= 64 ? 2 : 1)>(a, stream);
+            if (st != BW_EUNSUPPORTED) return st;
+        }
     }
     if (a.M == 1) return launch_gemv_mt<BITS, GROUP, 1>(a, stream);
     if (a.M <= 4) return launch_gemv_mt<BITS, GROUP, 4>(a, stream);

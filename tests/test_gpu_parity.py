@@ -452,7 +452,8 @@ def test_error_conventions_on_gpu():
 
 
 @pytest.mark.parametrize("bits,g,k,n", [(4, 128, 4096, 11008), (4, 128, 11008, 4096), (8, 128, 4096, 11008),
-                                        (4, 64, 4096, 11008), (2, 32, 4096, 11008), (4, 128, 4096, 4096)])
+                                        (4, 64, 4096, 11008), (2, 32, 4096, 11008), (4, 128, 4096, 4096),
+                                        (4, 32, 11008, 4096), (4, 64, 11008, 4096)])
 def test_full_size_properties(bits, g, k, n):
     """BASELINE-size layers, checked through size-independent properties:
       * a one-hot activation row returns a column of W16 bit-for-bit (the fused kernels reproduce the
@@ -478,6 +479,15 @@ def test_full_size_properties(bits, g, k, n):
         for i, c in enumerate(cols):
             assert torch.equal(y[i], w16[:, c])              # value compare: the accumulator turns -0 into +0
         assert (y[len(cols):] == 0).all()
+    # the same through the one- and two-row decode kernels (W4: the subnormal-operand kernel)
+    for i in range(0, len(cols) - 1, 2):
+        x = torch.zeros(2, k, device="cuda", dtype=torch.float16)
+        x[0, cols[i]] = 1.0
+        x[1, cols[i + 1]] = 1.0
+        y2 = hip.quantized_gemv_hip(x, q.qweight, q.scale, q.zero_point, None, bits, g)
+        y1 = hip.quantized_gemv_hip(x[1:], q.qweight, q.scale, q.zero_point, None, bits, g)
+        assert torch.equal(y2[0], w16[:, cols[i]]) and torch.equal(y2[1], w16[:, cols[i + 1]])
+        assert torch.equal(y1[0], w16[:, cols[i + 1]])
     # reconstruction bound
     w32 = hip.dequantize(q.qweight, q.scale, q.zero_point, g, bits, torch.float32)
     qmax = (1 << bits) - 1
