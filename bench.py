@@ -335,10 +335,79 @@ def extras_eager_call(torch, hip, QuantizedLinear, layers):
                 "torch_fp16_linear_forward_us": round(wall(lambda: lin(x)), 1)}
 
 
+def extras_llama7b_end_to_end(torch, hip, QuantizedLinear, layers):
+    """The reference's use end to end: a transformers Llama of Llama-2-7B shape (random weights, fp16, no network
+    for a checkpoint), Bitween(...).quantize(rtn=True, ignore_layers=[lm_head, embed_tokens], layer_config=the mixed
+    recipe), then a 512-token prompt and 256 greedy tokens at batch 1, eager PyTorch (no graph), next to the fp16
+    model in the same loop.  Attention, norms, rotary embedding, the KV cache and lm_head are transformers' own
+    kernels and Python; only the 224 linears are this library's."""
+    try:
+        from transformers import LlamaConfig, LlamaForCausalLM
+    except Exception as exc:                                   # noqa: BLE001
+        return {"skipped": "transformers not importable: %s" % exc}
+    import bitween_amd
+    cfg = LlamaConfig(hidden_size=4096, intermediate_size=11008, num_hidden_layers=32, num_attention_heads=32,
+                      num_key_value_heads=32, vocab_size=32000, max_position_embeddings=2048, tie_word_embeddings=False)
+    old = torch.get_default_dtype()
+    torch.set_default_dtype(torch.float16)
+    try:
+        with torch.device("cuda"):
+            model = LlamaForCausalLM(cfg)
+    finally:
+        torch.set_default_dtype(old)
+    model = model.half().cuda().eval()
+    recipe = {}
+    for i in range(32):
+        recipe["model.layers.%d.self_attn" % i] = (8, 128)
+        recipe["model.layers.%d.mlp" % i] = (4, 128)
+    for i in (0, 1, 30, 31):
+        recipe["model.layers.%d.mlp.down_proj" % i] = (2, 32)
+    ids = torch.randint(0, 32000, (1, 512), device="cuda", generator=torch.Generator(device="cuda").manual_seed(0))
+
+    def run(m, new_tokens=256):
+        with torch.no_grad():
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            out = m(input_ids=ids, use_cache=True)
+            past = out.past_key_values
+            tok = out.logits[:, -1].argmax(-1, keepdim=True)
+            torch.cuda.synchronize()
+            t1 = time.perf_counter()
+            for _ in range(new_tokens - 1):
+                out = m(input_ids=tok, past_key_values=past, use_cache=True)
+                past = out.past_key_values
+                tok = out.logits[:, -1].argmax(-1, keepdim=True)
+            torch.cuda.synchronize()
+            t2 = time.perf_counter()
+        return (t1 - t0) * 1e3, (new_tokens - 1) / (t2 - t1)
+
+    res = {}
+    run(model, 8)
+    pre, tps = run(model)
+    res["fp16_prefill512_ms"], res["fp16_decode_tokens_per_s"] = round(pre, 1), round(tps, 1)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    qmodel = bitween_amd.Bitween(model, bits=4, group_size=128).quantize(
+        rtn=True, ignore_layers=["lm_head", "embed_tokens"], layer_config=recipe, verbose=False)
+    torch.cuda.synchronize()
+    res["bitween_quantize_call_s"] = round(time.perf_counter() - t0, 2)      # includes the deep copy of the model
+    del model
+    res["quantized_linears"] = sum(isinstance(m, QuantizedLinear) for m in qmodel.modules())
+    run(qmodel, 8)
+    pre, tps = run(qmodel)
+    res["quantized_prefill512_ms"], res["quantized_decode_tokens_per_s"] = round(pre, 1), round(tps, 1)
+    bitween_amd.fuse_sibling_linears(qmodel)
+    run(qmodel, 8)
+    pre, tps = run(qmodel)
+    res["fused_siblings_prefill512_ms"], res["fused_siblings_decode_tokens_per_s"] = round(pre, 1), round(tps, 1)
+    res["note"] = "eager transformers loop: host-bound (hundreds of small launches per token), not a kernel figure"
+    return res
+
+
 EXTRAS = {"decode": extras_decode, "decode_infinity_cache_hot": extras_decode_hot,
           "decode_other_formats": extras_decode_other_formats, "hipblaslt_fp16_decode": extras_hipblaslt_decode,
           "prefill": extras_prefill, "quantize": extras_quantize, "mixed_precision_model": extras_mixed_precision_model, "eager_call": extras_eager_call,
-          "decode_fused_siblings": extras_decode_fused_siblings}
+          "llama7b_end_to_end": extras_llama7b_end_to_end, "decode_fused_siblings": extras_decode_fused_siblings}
 
 
 def main():
