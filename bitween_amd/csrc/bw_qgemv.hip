@@ -41,9 +41,7 @@ struct GemvCfg {
     // group's partial dot product scaled by s afterwards (4 FMAs per chunk instead of a multiply per
     // weight pair).  Smaller groups scale every weight, reproducing the reference's W16 bit for bit.
     static constexpr bool POST = GROUP % CHUNK_K == 0;
-    // 16 activation rows need 64 registers for the staged x alone: cap the workgroup at 8 waves there so
-    // that every wave may use 256 VGPRs
-    static constexpr int MAX_WAVES = MT > 8 ? 8 : 16;
+    static constexpr int MAX_WAVES = 16;
     static_assert(GROUP % VPI == 0, "a packed word must not straddle groups");
 };
 
@@ -468,7 +466,10 @@ int launch_gemv_kb(const GemvArgs& a, hipStream_t stream) {
     constexpr int BK = KB * C::CHUNK_K, X_BYTES = MT * (BK + 8) * 2;
     const size_t fixed = (size_t)((16 * (a.groups | 1) * 4 + 15) & ~15);
     int nwaves = (a.nchunks + KB - 1) / KB;
-    if (nwaves > C::MAX_WAVES) nwaves = C::MAX_WAVES;
+    // 16 activation rows: when the grid has more workgroups than the chip has CUs, 8-wave workgroups (two fit
+    // a CU) balance better than 16-wave ones; a grid of at most one workgroup per CU wants all 16 waves
+    const int max_waves = (MT > 8 && (a.N + 15) / 16 > 256) ? 8 : C::MAX_WAVES;
+    if (nwaves > max_waves) nwaves = max_waves;
     while (nwaves > 1 && fixed + (size_t)nwaves * (X_BYTES + MT * 64) > (size_t)kLdsBudget) nwaves--;
     const size_t lds = fixed + (size_t)nwaves * (X_BYTES + MT * 64);
     if (lds > (size_t)kLdsBudget) return BW_EUNSUPPORTED;
@@ -494,8 +495,9 @@ int launch_gemv_mt(const GemvArgs& a, hipStream_t stream) {
     if (MT >= 8) kb = a.nchunks <= 32 ? 1 : 2;
     else kb = (a.nchunks <= 32 && a.N < 8192) ? 2 : 4;
     if (kb > fit) kb = fit >= 4 ? 4 : (fit >= 2 ? 2 : 1);
-    if (kb >= 8) return launch_gemv_kb<BITS, GROUP, MT, 8>(a, stream);
-    if (kb >= 4) return launch_gemv_kb<BITS, GROUP, MT, 4>(a, stream);
+    if (MT > 8 && kb > 2) kb = 2;                         // 16-wave workgroups leave a wave 128 registers
+    if constexpr (MT <= 8)
+        if (kb >= 4) return launch_gemv_kb<BITS, GROUP, MT, 4>(a, stream);
     if (kb >= 2) return launch_gemv_kb<BITS, GROUP, MT, 2>(a, stream);
     return launch_gemv_kb<BITS, GROUP, MT, 1>(a, stream);
 }
