@@ -404,10 +404,37 @@ def extras_llama7b_end_to_end(torch, hip, QuantizedLinear, layers):
     return res
 
 
+def extras_backward(torch, hip, QuantizedLinear, layers):
+    """grad_input of QuantizedLinearFunction.backward, 4096 -> 14336 W4 g128: the fused kernel (bw_qdgrad), the
+    path it replaces (HIP dequantise to float16 + library GEMM) and that GEMM alone on resident fp16 weights."""
+    k, n = 4096, 14336
+    q = make_layer(torch, QuantizedLinear, k, n, 4, 128, seed=11)
+    w16 = hip.dequantize(q.qweight, q.scale, q.zero_point, 128, 4, torch.float16)
+    out = {}
+    for m in (128, 512, 2048):
+        go = torch.randn(m, n, device="cuda", dtype=torch.float16)
+
+        def ours():
+            w = hip.dequantize(q.qweight, q.scale, q.zero_point, 128, 4, torch.float16)
+            return go @ w
+
+        def fused():
+            return hip.quantized_input_grad(go, q.qweight, q.scale, q.zero_point, 4, 128)
+
+        t_fused = time_calls(torch, fused, 30, 5)
+        t_ours = time_calls(torch, ours, 30, 5)
+        t_deq = time_calls(torch, lambda: hip.dequantize(q.qweight, q.scale, q.zero_point, 128, 4, torch.float16), 30, 5)
+        t_gemm = time_calls(torch, lambda: go @ w16, 30, 5)
+        out["4096x14336_M%d" % m] = {"fused_dgrad_us": round(t_fused, 1), "fused_TFLOPs": round(2.0 * m * n * k / t_fused / 1e6, 1),
+                                     "dequantize_plus_gemm_us": round(t_ours, 1), "dequantize_us": round(t_deq, 1),
+                                     "fp16_gemm_us": round(t_gemm, 1)}
+    return out
+
+
 EXTRAS = {"decode": extras_decode, "decode_infinity_cache_hot": extras_decode_hot,
           "decode_other_formats": extras_decode_other_formats, "hipblaslt_fp16_decode": extras_hipblaslt_decode,
           "prefill": extras_prefill, "quantize": extras_quantize, "mixed_precision_model": extras_mixed_precision_model, "eager_call": extras_eager_call,
-          "llama7b_end_to_end": extras_llama7b_end_to_end, "decode_fused_siblings": extras_decode_fused_siblings}
+          "llama7b_end_to_end": extras_llama7b_end_to_end, "backward": extras_backward, "decode_fused_siblings": extras_decode_fused_siblings}
 
 
 def main():

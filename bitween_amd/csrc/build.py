@@ -10,7 +10,7 @@ import subprocess
 import sys
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-SOURCES = ["bw_quantize.hip", "bw_qgemv.hip", "bw_qgemm.hip"]
+SOURCES = ["bw_quantize.hip", "bw_qgemv.hip", "bw_qgemm.hip", "bw_qdgrad.hip"]
 LIB = os.path.join(HERE, "libbitween_hip.so")
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",

@@ -1,0 +1,281 @@
+// bw_qdgrad.hip - input gradient of the quantised linear layer, fused with the dequantisation:
+//
+//     grad_x[M][K] = grad_y[M][N] @ W16[N][K],      W16 = fp16(scale * (q - zp))
+//
+// (QuantizedLinearFunction.backward, bitween/modules.py:108-141: it unpacks, forms W32 = scale * (q - zp),
+// casts to grad_output's dtype and calls matmul; for float16 gradients that cast gives exactly W16.)
+//
+// The reduction runs over N, the dimension the packed words do NOT run along, so a weight tile has to be
+// transposed on its way to the matrix core.  A workgroup owns a 128 (m) x 128 (k) tile of grad_x and walks N
+// in steps of 32 rows:
+//   * 256 threads each take 16 consecutive k of one row n (one group: groups are >= 32 wide), dequantise them to
+//     the reference's W16 (magic-number unpack, exact q - z, one multiply by the scale) and scatter the 16
+//     halves into an LDS tile stored k-major (row k holds the 32 n of the step) - that is the transposition;
+//   * the 128 x 32 slice of grad_y goes to a second LDS tile as it is;
+//   * v_mfma_f32_16x16x32_f16 with A = rows of the k-major tile (8 consecutive n per lane) and B = rows of the
+//     grad_y tile: D[k][m], so a lane ends up with 4 consecutive k of one m.
+// LDS is double buffered, global loads of step s+1 are in flight during the MFMAs of step s, one barrier per step.
+// Small M * K leaves the chip idle, so N is cut into slices whose float32 partial tiles a second kernel adds up.
+#include <hip/hip_runtime.h>
+
+#include "bw_common.h"
+
+namespace {
+
+constexpr int DM = 128, DK = 128, DN = 32, DTHREADS = 256;
+constexpr int DPITCH = 80;                           // bytes per LDS row: 32 halves + 16 (rows stay 16-byte aligned)
+constexpr int A_BYTES = DM * DPITCH;                 // grad_y tile
+constexpr int B_BYTES = DK * DPITCH + (DK / 16) * 16;   // k-major weight tile; every 16-row block shifted 16 bytes
+constexpr int STAGE = A_BYTES + B_BYTES;
+
+struct DgradArgs {
+    const _Float16* go;
+    const char* qweight;
+    const _Float16* scale;
+    const _Float16* zp;
+    _Float16* gx;
+    float* ws;
+    int M, N, K, ldg, ldx, groups, row_bytes;
+    int tiles_k, splits, steps_per_split;
+};
+
+BW_DEV int b_row_offset(int k) { return k * DPITCH + (k >> 4) * 16; }
+
+template <int BITS> struct WLoad;
+template <> struct WLoad<4> { typedef u2 type; };
+template <> struct WLoad<8> { typedef u4 type; };
+template <> struct WLoad<2> { typedef uint32_t type; };
+
+// 16 values of one row -> 8 float16 pairs; pair p, half h is element kmap(p, h) of the 16
+template <int BITS>
+BW_DEV void dequant16(const typename WLoad<BITS>::type& w, const GroupConst<BITS>& gc, h2* out) {
+    if constexpr (BITS == 4) {
+        dequant_word4<true>(w[0], gc, out);
+        dequant_word4<true>(w[1], gc, out + 4);
+    } else if constexpr (BITS == 8) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) dequant_word8<true>(w[j], gc, out + 2 * j);
+    } else {
+        dequant_word2<true>(w, gc, out);
+    }
+}
+template <int BITS>
+BW_DEV constexpr int kmap(int p, int h) {
+    if constexpr (BITS == 4) return 8 * (p >> 2) + (p & 3) + 4 * h;
+    else if constexpr (BITS == 8) return 2 * p + h;
+    else return p + 8 * h;
+}
+
+template <int BITS, int GROUP>
+__global__ __launch_bounds__(DTHREADS) void qdgrad_kernel(const DgradArgs a) {
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    typedef typename WLoad<BITS>::type wload_t;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tile = blockIdx.x / a.splits, split = blockIdx.x % a.splits;
+    const int m0 = (tile / a.tiles_k) * DM, k0 = (tile % a.tiles_k) * DK;
+    const int nsteps = a.N / DN;
+    const int s_begin = split * a.steps_per_split;
+    const int s_end = min(s_begin + a.steps_per_split, nsteps);
+
+    // loader roles
+    const int wn = tid >> 3, wks = tid & 7;                           // weight: row of the step, 16-value segment
+    const int gm = tid >> 1, gpart = tid & 1;                         // grad_y: row of the tile, 32-byte half
+    const char* wp = a.qweight + (int64_t)wn * a.row_bytes + (int64_t)(k0 + wks * 16) * BITS / 8;
+    const int gcol = (k0 + wks * 16) / GROUP;
+    const _Float16* sp = a.scale + (int64_t)wn * a.groups + gcol;
+    const _Float16* zp = a.zp + (int64_t)wn * a.groups + gcol;
+    const bool g_ok = m0 + gm < a.M;
+    const _Float16* gp = a.go + (int64_t)(m0 + gm) * a.ldg + gpart * 16;
+
+    wload_t wreg;
+    _Float16 sreg, zreg;
+    u4 greg[2];
+    auto issue = [&](int step) {
+        const int64_t n0 = (int64_t)step * DN;
+        wreg = *reinterpret_cast<const wload_t*>(wp + n0 * a.row_bytes);
+        sreg = sp[n0 * a.groups];
+        zreg = zp[n0 * a.groups];
+        if (g_ok) {
+            greg[0] = *reinterpret_cast<const u4*>(gp + n0);
+            greg[1] = *reinterpret_cast<const u4*>(gp + n0 + 8);
+        } else {
+            greg[0] = greg[1] = u4{0u, 0u, 0u, 0u};
+        }
+    };
+
+    f4 acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) acc[i][j] = f4{0.f, 0.f, 0.f, 0.f};
+
+    const int wk = (wave & 1) * 64, wm = (wave >> 1) * 64;            // this wave's quarter of the tile
+    const int l16 = lane & 15, q = lane >> 4;
+
+    if (s_begin < s_end) issue(s_begin);
+    for (int step = s_begin; step < s_end; step++) {
+        char* As = smem + ((step - s_begin) & 1) * STAGE;
+        char* Bs = As + A_BYTES;
+        // weights: dequantise, scatter transposed
+        {
+            GroupConst<BITS> gc;
+            gc.set(sreg, zreg);
+            h2 w16[8];
+            dequant16<BITS>(wreg, gc, w16);
+#pragma unroll
+            for (int p = 0; p < 8; p++)
+#pragma unroll
+                for (int h = 0; h < 2; h++) {
+                    const int k = wks * 16 + kmap<BITS>(p, h);
+                    *reinterpret_cast<_Float16*>(Bs + b_row_offset(k) + wn * 2) = w16[p][h];
+                }
+            u4* dst = reinterpret_cast<u4*>(As + gm * DPITCH + gpart * 32);
+            dst[0] = greg[0];
+            dst[1] = greg[1];
+        }
+        if (step + 1 < s_end) issue(step + 1);
+        __syncthreads();
+        h8 af[4], bf[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) af[i] = *reinterpret_cast<const h8*>(Bs + b_row_offset(wk + 16 * i + l16) + q * 16);
+#pragma unroll
+        for (int j = 0; j < 4; j++) bf[j] = *reinterpret_cast<const h8*>(As + (wm + 16 * j + l16) * DPITCH + q * 16);
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+                acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[i], bf[j], acc[i][j], 0, 0, 0);
+    }
+
+    // acc[i][j][r] = grad_x[m0 + wm + 16 j + l16][k0 + wk + 16 i + 4 q + r]
+    if (a.splits > 1) {
+        float* dst = a.ws + (size_t)blockIdx.x * (DM * DK);
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+                *reinterpret_cast<f4*>(dst + (wm + 16 * j + l16) * DK + wk + 16 * i + 4 * q) = acc[i][j];
+    } else {
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const int m = m0 + wm + 16 * j + l16;
+            if (m >= a.M) continue;
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const f4 v = acc[i][j];
+                _Float16* dst = a.gx + (int64_t)m * a.ldx + k0 + wk + 16 * i + 4 * q;
+                *reinterpret_cast<u2*>(dst) = u2{as_u32(h2{(_Float16)v[0], (_Float16)v[1]}), as_u32(h2{(_Float16)v[2], (_Float16)v[3]})};
+            }
+        }
+    }
+}
+
+// grad_x tile = sum of its slices' partial tiles, rounded once
+__global__ __launch_bounds__(256) void qdgrad_reduce_kernel(const DgradArgs a) {
+    const int tile = blockIdx.y;
+    const int quad = (int)(blockIdx.x * blockDim.x + threadIdx.x);    // < DM * DK / 4
+    const int ml = quad / (DK / 4), kl = (quad % (DK / 4)) * 4;
+    const int m = (tile / a.tiles_k) * DM + ml, k = (tile % a.tiles_k) * DK + kl;
+    if (m >= a.M) return;
+    const float* src = a.ws + (size_t)tile * a.splits * (DM * DK) + ml * DK + kl;
+    f4 v = {0.f, 0.f, 0.f, 0.f};
+    for (int z = 0; z < a.splits; z++) {
+        const f4 t = *reinterpret_cast<const f4*>(src + (size_t)z * (DM * DK));
+#pragma unroll
+        for (int i = 0; i < 4; i++) v[i] += t[i];
+    }
+    *reinterpret_cast<u2*>(a.gx + (int64_t)m * a.ldx + k) =
+        u2{as_u32(h2{(_Float16)v[0], (_Float16)v[1]}), as_u32(h2{(_Float16)v[2], (_Float16)v[3]})};
+}
+
+struct DgradPlan {
+    int tiles_k, tiles, splits, steps_per_split;
+    size_t ws_bytes;
+};
+
+inline int dgrad_cus() {
+    static const int cus = [] {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess)
+            n = 0;
+        return n > 0 ? n : 256;
+    }();
+    return cus;
+}
+
+// Three workgroups fit a CU.  Fewer tiles than CUs: cut N so that every CU has one, never below 8 steps a slice.
+inline DgradPlan dgrad_plan(int64_t M, int64_t N, int64_t K, bool have_workspace) {
+    DgradPlan p;
+    p.tiles_k = (int)(K / DK);
+    p.tiles = p.tiles_k * (int)((M + DM - 1) / DM);
+    const int nsteps = (int)(N / DN);
+    p.splits = 1;
+    p.steps_per_split = nsteps;
+    p.ws_bytes = 0;
+    const int cus = dgrad_cus();
+    if (!have_workspace || p.tiles >= cus) return p;
+    int s = (cus + p.tiles - 1) / p.tiles;
+    if (s > nsteps / 8) s = nsteps / 8;
+    if (s > 32) s = 32;
+    if (s < 2) return p;
+    const int sps = (nsteps + s - 1) / s;
+    s = (nsteps + sps - 1) / sps;
+    if (s < 2) return p;
+    p.splits = s;
+    p.steps_per_split = sps;
+    p.ws_bytes = (size_t)p.tiles * s * DM * DK * sizeof(float);
+    return p;
+}
+
+inline bool dgrad_fast_shape(int64_t M, int64_t N, int64_t K, int64_t ldg, int64_t ldx, int bits, int group) {
+    return (group == 32 || group == 64 || group == 128) && K % DK == 0 && N % DN == 0 && ldg % 8 == 0 && ldx % 4 == 0 &&
+           M >= 1 && M < ((int64_t)1 << 24) && N * (K * bits / 8) < ((int64_t)1 << 40);
+}
+
+template <int BITS, int GROUP>
+int launch_dgrad(DgradArgs a, void* workspace, size_t workspace_bytes, hipStream_t stream) {
+    const DgradPlan p = dgrad_plan(a.M, a.N, a.K, workspace != nullptr);
+    if (p.ws_bytes > workspace_bytes) return BW_EWORKSPACE;
+    a.ws = (float*)workspace;
+    a.tiles_k = p.tiles_k;
+    a.splits = p.splits;
+    a.steps_per_split = p.steps_per_split;
+    hipLaunchKernelGGL((qdgrad_kernel<BITS, GROUP>), dim3((unsigned)(p.tiles * p.splits)), dim3(DTHREADS), 2 * STAGE, stream, a);
+    if (hipGetLastError() != hipSuccess) return BW_ELAUNCH;
+    if (p.splits > 1) {
+        hipLaunchKernelGGL(qdgrad_reduce_kernel, dim3(DM * DK / 4 / 256, (unsigned)p.tiles), dim3(256), 0, stream, a);
+        if (hipGetLastError() != hipSuccess) return BW_ELAUNCH;
+    }
+    return BW_OK;
+}
+
+}  // namespace
+
+extern "C" size_t bw_qdgrad_workspace_bytes(int64_t M, int64_t N, int64_t K, int bits, int group) {
+    if (!bw_shape_ok(N, K, bits, group) || !dgrad_fast_shape(M, N, K, N, K, bits, group)) return 0;
+    return dgrad_plan(M, N, K, true).ws_bytes;
+}
+
+extern "C" int bw_qdgrad(const void* grad_y, int act_dtype, int64_t M, int64_t N, int64_t ldg, const int32_t* qweight,
+                         const void* scale16, const void* zp16, int64_t K, int bits, int group, void* grad_x,
+                         int64_t ldx, void* workspace, size_t workspace_bytes, void* stream) {
+    if (!grad_y || !qweight || !scale16 || !zp16 || !grad_x) return BW_EINVAL;
+    if (!bw_shape_ok(N, K, bits, group) || M < 1 || ldg < N || ldx < K) return BW_EINVAL;
+    if (act_dtype != BW_F16) return BW_EUNSUPPORTED;
+    if (!dgrad_fast_shape(M, N, K, ldg, ldx, bits, group)) return BW_EUNSUPPORTED;
+    if (!bw_aligned(grad_y, 16) || !bw_aligned(grad_x, 8) || !bw_aligned(qweight, 16)) return BW_EALIGN;
+    if (workspace && !bw_aligned(workspace, 16)) return BW_EALIGN;
+    DgradArgs a;
+    a.go = (const _Float16*)grad_y; a.qweight = (const char*)qweight; a.scale = (const _Float16*)scale16;
+    a.zp = (const _Float16*)zp16; a.gx = (_Float16*)grad_x; a.ws = nullptr;
+    a.M = (int)M; a.N = (int)N; a.K = (int)K; a.ldg = (int)ldg; a.ldx = (int)ldx;
+    a.groups = (int)(K / group); a.row_bytes = (int)(K * bits / 8);
+    hipStream_t st = (hipStream_t)stream;
+#define BW_CASE(B, G) \
+    if (bits == B && group == G) return launch_dgrad<B, G>(a, workspace, workspace_bytes, st);
+    BW_CASE(4, 128) BW_CASE(4, 64) BW_CASE(4, 32)
+    BW_CASE(8, 128) BW_CASE(8, 64) BW_CASE(8, 32)
+    BW_CASE(2, 128) BW_CASE(2, 64) BW_CASE(2, 32)
+#undef BW_CASE
+    return BW_EUNSUPPORTED;
+}

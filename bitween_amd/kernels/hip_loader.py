@@ -19,9 +19,9 @@ _lib = None
 BW_F16, BW_BF16, BW_F32, BW_I32 = 0, 1, 2, 3
 _DTYPE_CODE = {torch.float16: BW_F16, torch.bfloat16: BW_BF16, torch.float32: BW_F32, torch.int32: BW_I32}
 
-ABI_VERSION = 2            # what bw_abi_version() of a matching library returns
+ABI_VERSION = 3            # what bw_abi_version() of a matching library returns
 ENTRY_POINTS = ("bw_abi_version", "bw_strerror", "bw_quantize_pack", "bw_quantize_pack_add", "bw_dequantize", "bw_qgemv", "bw_qgemm",
-                "bw_qgemm_ws", "bw_qgemm_workspace_bytes", "bw_qlinear")
+                "bw_qgemm_ws", "bw_qgemm_workspace_bytes", "bw_qlinear", "bw_qdgrad", "bw_qdgrad_workspace_bytes")
 
 
 class BitweenHipError(RuntimeError):
@@ -58,6 +58,10 @@ def load():
     lib.bw_qgemm_ws.argtypes = mm[:-1] + [vp, ctypes.c_size_t, vp]
     lib.bw_qgemm_workspace_bytes.argtypes = [i64, i64, i64, i32, i32]
     lib.bw_qgemm_workspace_bytes.restype = ctypes.c_size_t
+    lib.bw_qdgrad_workspace_bytes.argtypes = [i64, i64, i64, i32, i32]
+    lib.bw_qdgrad_workspace_bytes.restype = ctypes.c_size_t
+    lib.bw_qdgrad.argtypes = [vp, i32, i64, i64, i64, vp, vp, vp, i64, i32, i32, vp, i64, vp, ctypes.c_size_t, vp]
+    lib.bw_qdgrad.restype = i32
     for name in ("bw_quantize_pack", "bw_quantize_pack_add", "bw_dequantize", "bw_qgemv", "bw_qgemm", "bw_qgemm_ws", "bw_qlinear"):
         getattr(lib, name).restype = i32
     for name in ("bw_qgemv", "bw_qgemm", "bw_qlinear"):
@@ -207,6 +211,36 @@ def _matmul(entry, x, qweight, scale, zero_point, bias, bits, group_size):
     if st:
         _check(st, entry)
     return y
+
+
+def quantized_input_grad(grad_y, qweight, scale, zero_point, bits, group_size):
+    """grad_x[M,K] = grad_y[M,N] @ W16[N,K] with the dequantisation fused in (bw_qdgrad); None when the library
+    has no fused kernel for this shape / dtype - the caller then dequantises and calls the library GEMM."""
+    if grad_y.dtype is not torch.float16 or not grad_y.is_cuda or grad_y.dim() != 2:
+        return None
+    if qweight.dtype is not torch.int32 or scale.dtype is not torch.float16 or zero_point.dtype is not torch.float16:
+        return None
+    m, n = grad_y.shape
+    k = qweight.shape[1] * (32 // bits)
+    if m == 0 or qweight.shape[0] != n:
+        return None
+    if grad_y.stride(1) != 1 or grad_y.stride(0) % 8 or grad_y.data_ptr() % 16:
+        grad_y = grad_y.contiguous()
+        if grad_y.stride(0) % 8:
+            return None
+    qweight, scale, zero_point = qweight.contiguous(), scale.contiguous(), zero_point.contiguous()
+    lib = load()
+    grad_x = torch.empty((m, k), dtype=torch.float16, device=grad_y.device)
+    with _on_device(grad_y.device) as index:
+        nbytes = lib.bw_qdgrad_workspace_bytes(m, n, k, bits, group_size)
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=grad_y.device) if nbytes else None
+        st = lib.bw_qdgrad(grad_y.data_ptr(), BW_F16, m, n, grad_y.stride(0), qweight.data_ptr(), scale.data_ptr(),
+                           zero_point.data_ptr(), k, bits, group_size, grad_x.data_ptr(), k,
+                           None if ws is None else ws.data_ptr(), nbytes, _raw_stream(index))
+    if st == -2:                                           # BW_EUNSUPPORTED: shape outside the fused kernel
+        return None
+    _check(st, "bw_qdgrad")
+    return grad_x
 
 
 def quantized_matmul_hip(x, qweight, scale, zero_point, bias, bits, group_size):

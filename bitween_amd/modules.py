@@ -33,6 +33,12 @@ class QuantizedLinearFunction(torch.autograd.Function):
         x, qweight, scale, zero_point, bias = ctx.saved_tensors
         grad_input = None
         if ctx.needs_input_grad[0]:
+            # float16 gradients on kernel-sized shapes: one fused kernel, the weights are never materialised
+            if grad_output.dtype is torch.float16 and grad_output.is_cuda:
+                go2 = grad_output.reshape(-1, grad_output.shape[-1])
+                gx = _hip.quantized_input_grad(go2, qweight, scale, zero_point, ctx.bits, ctx.group_size)
+                if gx is not None:
+                    return gx.view(*grad_output.shape[:-1], gx.shape[-1]), None, None, None, None, None, None
             # W = scale * (q - zp) in float32, cast to grad_output.dtype: the float32 product is exact,
             # so dequantising straight to that dtype gives the same bits.
             gdt = grad_output.dtype if grad_output.dtype in (torch.float16, torch.bfloat16, torch.float32) else torch.float32

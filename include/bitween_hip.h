@@ -120,6 +120,23 @@ int bw_qlinear(const void* x, int act_dtype, int64_t M, int64_t K, int64_t ldx,
                const int32_t* qweight, const void* scale16, const void* zp16, const void* bias,
                int64_t N, int bits, int group, void* y, int64_t ldy, void* stream);
 
+/* Input gradient, fused with the dequantisation:  grad_x[M][K] = grad_y[M][N] @ W16[N][K]
+ * replaces QuantizedLinearFunction.backward (bitween/modules.py:108-141), which unpacks the weights, forms
+ * scale * (q - zp), casts it to grad_output's dtype and calls matmul; for float16 gradients that cast gives the
+ * same W16 as the forward.  Products accumulate in float32, grad_x is rounded once.
+ *   grad_y [M][ldg], grad_x [M][ldx] of act_dtype (BW_F16 only)
+ * Built for K % 128 == 0, N % 32 == 0, group 32 | 64 | 128, ldg % 8 == 0, ldx % 4 == 0; other shapes and dtypes
+ * return BW_EUNSUPPORTED (the Python backward then dequantises with bw_dequantize and calls the library GEMM).
+ * When M * K is small the reduction over N is cut into slices whose float32 partial sums go through a
+ * caller-provided workspace of bw_qdgrad_workspace_bytes(...) bytes (16-byte aligned; 0 = none needed);
+ * workspace == NULL runs unsliced. */
+size_t bw_qdgrad_workspace_bytes(int64_t M, int64_t N, int64_t K, int bits, int group);
+
+int bw_qdgrad(const void* grad_y, int act_dtype, int64_t M, int64_t N, int64_t ldg,
+              const int32_t* qweight, const void* scale16, const void* zp16,
+              int64_t K, int bits, int group, void* grad_x, int64_t ldx,
+              void* workspace, size_t workspace_bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,137 @@
+"""bw_qdgrad (grad_x = grad_y @ W16, dequantisation fused) through the C ABI against the oracle's
+qlinear_backward (bitween/modules.py:108-141 of the reference).
+
+Bars: max |g - ref| <= 1e-2 * max |ref| and mean |g - ref| < 1e-2 * mean |ref| (the forward's tolerance,
+main.py:471-477: the reference states none for the backward); elementwise one float16 rounding of the result plus
+float32 accumulation slack; a one-hot grad_y row returns a ROW of W16 bit for bit."""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+from gpu_util import quantized_layer, to_gpu
+from oracle import rtn_oracle as orc
+
+pytestmark = pytest.mark.gpu
+
+COMBOS = [(b, g) for b in (2, 4, 8) for g in (32, 64, 128)]
+
+
+def _call(lib, go, d, m, n, k, bits, g, use_ws=True, ldg=None):
+    ldg = n if ldg is None else ldg
+    need = lib.bw_qdgrad_workspace_bytes(m, n, k, bits, g) if use_ws else 0
+    ws = torch.empty(max(need, 16), dtype=torch.uint8, device="cuda")
+    gx = torch.full((m, k), float("nan"), dtype=torch.float16, device="cuda")
+    st = lib.bw_qdgrad(go.data_ptr(), 0, m, n, ldg, d[0].data_ptr(), d[1].data_ptr(), d[2].data_ptr(), k, bits, g,
+                       gx.data_ptr(), k, ws.data_ptr() if need else None, need,
+                       ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    torch.cuda.synchronize()
+    return st, gx, need
+
+
+def _check(gx, go16, qw, s16, z16, bits, g):
+    ref = orc.qlinear_backward(go16, qw, s16, z16, bits, g)                  # float64
+    got = gx.double().cpu().numpy()
+    assert np.isfinite(got).all()
+    w16 = np.abs(orc.dequantize_f16(qw, s16, z16, g, bits).astype(np.float64))
+    mag = np.abs(go16.astype(np.float64)) @ w16
+    bound = 2.0 ** -10 * np.abs(ref) + 2e-6 * mag + 1e-7
+    assert (np.abs(got - ref) <= bound).all(), float((np.abs(got - ref) / bound).max())
+    assert np.abs(got - ref).max() <= 1e-2 * np.abs(ref).max()
+    assert np.abs(got - ref).mean() < 1e-2 * np.abs(ref).mean()
+
+
+@pytest.mark.parametrize("bits,g", COMBOS)
+def test_dgrad_vs_oracle(bits, g):
+    from bitween_amd.kernels import hip_loader
+    lib = hip_loader.load()
+    for (n, k) in ((256, 384), (1024, 128), (96, 768)):
+        _, qw, s16, z16, _ = quantized_layer(n, k, bits, g, seed=n + k + bits + g, outliers=True, bias=False)
+        d = [to_gpu(a) for a in (qw, s16, z16)]
+        rng = np.random.default_rng(n * 7 + k)
+        for m in (1, 17, 128, 200):
+            go16 = rng.standard_normal((m, n)).astype(np.float16)
+            for use_ws in (True, False):
+                st, gx, need = _call(lib, to_gpu(go16), d, m, n, k, bits, g, use_ws)
+                assert st == 0
+                _check(gx, go16, qw, s16, z16, bits, g)
+
+
+@pytest.mark.parametrize("bits,g,n,k", [(4, 128, 11008, 4096), (8, 128, 4096, 4096), (2, 32, 4096, 11008), (4, 64, 14336, 4096)])
+def test_dgrad_full_size_one_hot_rows_and_split(bits, g, n, k):
+    """Full-size layers: the reduction over N is cut into slices (workspace) at small M; a one-hot grad_y row
+    returns a row of the reference's W16 exactly; random rows meet the oracle on a sample of columns."""
+    from bitween_amd.kernels import hip_loader
+    hip = hip_loader
+    lib = hip.load()
+    gen = torch.Generator(device="cuda").manual_seed(bits * 17 + g)
+    w = (torch.randn(n, k, device="cuda", generator=gen) * 0.02).half()
+    qw, sc, zp = hip.quantize_pack(w, bits, g, math_dtype=torch.float32, scale_dtype=torch.float16, zp_dtype=torch.float16)
+    w16 = hip.dequantize(qw, sc, zp, g, bits, torch.float16)
+    d = [qw, sc, zp]
+    rows = [0, 1, 31, 32, n // 2 + 5, n - 1]
+    go = torch.zeros(len(rows), n, device="cuda", dtype=torch.float16)
+    for i, r in enumerate(rows):
+        go[i, r] = 1.0
+    st, gx, need = _call(lib, go, d, len(rows), n, k, bits, g)
+    assert st == 0 and need > 0, "small M on a full-size layer is meant to split"
+    for i, r in enumerate(rows):
+        assert torch.equal(gx[i], w16[r])
+    for m in (64, 300):
+        go = torch.randn(m, n, device="cuda", dtype=torch.float16, generator=gen)
+        st, gx, _ = _call(lib, go, d, m, n, k, bits, g)
+        assert st == 0
+        ref = go.float() @ w16.float()
+        err = (gx.float() - ref).abs()
+        assert (err <= 2.0 ** -9 * ref.abs() + 2e-5 * (go.float().abs() @ w16.float().abs()) + 1e-6).all()
+
+
+def test_dgrad_refusals_and_padding():
+    from bitween_amd.kernels import hip_loader
+    lib = hip_loader.load()
+    n, k, bits, g = 64, 256, 4, 64
+    _, qw, s16, z16, _ = quantized_layer(n, k, bits, g, seed=3, bias=False)
+    d = [to_gpu(a) for a in (qw, s16, z16)]
+    go16 = np.random.default_rng(0).standard_normal((5, n)).astype(np.float16)
+    # padded grad_y rows: the padding is never read
+    buf = torch.full((5, n + 8), float("nan"), dtype=torch.float16, device="cuda")
+    buf[:, :n] = to_gpu(go16)
+    st, gx, _ = _call(lib, buf, d, 5, n, k, bits, g, ldg=n + 8)
+    assert st == 0
+    _check(gx, go16, qw, s16, z16, bits, g)
+    # shapes outside the fused kernel are refused, nothing is launched
+    assert lib.bw_qdgrad_workspace_bytes(5, 40, 256, 4, 64) == 0
+    go = to_gpu(go16)
+    gx = torch.full((5, k), 7.0, dtype=torch.float16, device="cuda")
+    st = lib.bw_qdgrad(go.data_ptr(), 0, 5, n, n, d[0].data_ptr(), d[1].data_ptr(), d[2].data_ptr(), k, bits, g,
+                       gx.data_ptr(), k, None, 0, None)
+    assert st == 0
+    assert lib.bw_qdgrad(go.data_ptr(), 1, 5, n, n, d[0].data_ptr(), d[1].data_ptr(), d[2].data_ptr(), k, bits, g,
+                         gx.data_ptr(), k, None, 0, None) == -2          # bfloat16: BW_EUNSUPPORTED
+    assert lib.bw_qdgrad(go.data_ptr(), 0, 5, n, n, d[0].data_ptr(), d[1].data_ptr(), d[2].data_ptr(), k, 3, g,
+                         gx.data_ptr(), k, None, 0, None) == -1          # BW_EINVAL
+    assert lib.bw_qdgrad(None, 0, 5, n, n, d[0].data_ptr(), d[1].data_ptr(), d[2].data_ptr(), k, bits, g,
+                         gx.data_ptr(), k, None, 0, None) == -1
+
+
+def test_module_backward_uses_fused_kernel_and_falls_back():
+    """autograd through QuantizedLinear: float16 gradients take bw_qdgrad; float32 gradients and odd shapes take
+    the dequantise + library GEMM path; both meet the oracle."""
+    import bitween_amd
+    torch.manual_seed(4)
+    for (k, n, gdt) in ((256, 512, torch.float16), (256, 512, torch.float32), (96, 40, torch.float16)):
+        lin = torch.nn.Linear(k, n, bias=True, device="cuda", dtype=torch.float16)
+        q = bitween_amd.QuantizedLinear.from_float(lin, 4, 32)
+        x = torch.randn(3, 7, k, device="cuda", dtype=torch.float16, requires_grad=True)
+        y = q(x)
+        go = torch.randn(3, 7, n, device="cuda", dtype=torch.float16)
+        if gdt is torch.float32:
+            (y.float() * go.float()).sum().backward()
+        else:
+            y.backward(go)
+        ref = orc.qlinear_backward(go.reshape(21, n).cpu().numpy(), q.qweight.cpu().numpy(), q.scale.cpu().numpy(),
+                                   q.zero_point.cpu().numpy(), 4, 32)
+        got = x.grad.reshape(21, k).double().cpu().numpy()
+        assert x.grad.dtype == torch.float16
+        assert np.abs(got - ref).max() <= 1e-2 * np.abs(ref).max()
