@@ -14,7 +14,8 @@
 //   * the 128 x 32 slice of grad_y goes to a second LDS tile as it is;
 //   * v_mfma_f32_16x16x32_f16 with A = rows of the k-major tile (8 consecutive n per lane) and B = rows of the
 //     grad_y tile: D[k][m], so a lane ends up with 4 consecutive k of one m.
-// LDS is double buffered, global loads of step s+1 are in flight during the MFMAs of step s, one barrier per step.
+// LDS is double buffered and filled one step ahead, in the shadow of the current step's MFMAs; global loads run
+// four steps ahead; one barrier per step.
 // Small M * K leaves the chip idle, so N is cut into slices whose float32 partial tiles a second kernel adds up.
 #include <hip/hip_runtime.h>
 
@@ -22,11 +23,16 @@
 
 namespace {
 
-constexpr int DM = 128, DK = 128, DN = 32, DTHREADS = 256;
+constexpr int DK = 128, DN = 32, DTHREADS = 256;
 constexpr int DPITCH = 80;                           // bytes per LDS row: 32 halves + 16 (rows stay 16-byte aligned)
-constexpr int A_BYTES = DM * DPITCH;                 // grad_y tile
 constexpr int B_BYTES = DK * DPITCH + (DK / 16) * 16;   // k-major weight tile; every 16-row block shifted 16 bytes
-constexpr int STAGE = A_BYTES + B_BYTES;
+// MT = 16-row m tiles per wave (the workgroup's 2 x 2 waves cover 32 MT rows of m).  MT = 8 was measured too:
+// 128 accumulators leave one wave per SIMD and it only wins on one shape, so 4 is what is built.
+template <int MT> struct DgradTile {
+    static constexpr int DM = 32 * MT;
+    static constexpr int A_BYTES = DM * DPITCH;      // grad_y tile
+    static constexpr int STAGE = A_BYTES + B_BYTES;
+};
 
 struct DgradArgs {
     const _Float16* go;
@@ -38,6 +44,10 @@ struct DgradArgs {
     int M, N, K, ldg, ldx, groups, row_bytes;
     int tiles_k, splits, steps_per_split;
 };
+
+BW_DEV uint32_t dpp_xor8(uint32_t v) {               // value of lane ^ 8 (rotate a 16-lane row by 8)
+    return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x128, 0xF, 0xF, true);
+}
 
 BW_DEV int b_row_offset(int k) { return k * DPITCH + (k >> 4) * 16; }
 
@@ -66,8 +76,11 @@ BW_DEV constexpr int kmap(int p, int h) {
     else return p + 8 * h;
 }
 
-template <int BITS, int GROUP>
+template <int BITS, int GROUP, int MT>
 __global__ __launch_bounds__(DTHREADS) void qdgrad_kernel(const DgradArgs a) {
+    constexpr int DM = DgradTile<MT>::DM, A_BYTES = DgradTile<MT>::A_BYTES, STAGE = DgradTile<MT>::STAGE;
+    constexpr int GR = DM / 128;                                      // grad_y rows a thread stages
+    constexpr int PD = 4;                                             // steps of global loads in flight
     extern __shared__ __attribute__((aligned(16))) char smem[];
     typedef typename WLoad<BITS>::type wload_t;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -84,67 +97,99 @@ __global__ __launch_bounds__(DTHREADS) void qdgrad_kernel(const DgradArgs a) {
     const int gcol = (k0 + wks * 16) / GROUP;
     const _Float16* sp = a.scale + (int64_t)wn * a.groups + gcol;
     const _Float16* zp = a.zp + (int64_t)wn * a.groups + gcol;
-    const bool g_ok = m0 + gm < a.M;
-    const _Float16* gp = a.go + (int64_t)(m0 + gm) * a.ldg + gpart * 16;
+    // rows past M repeat the last row: every output row depends on its own grad_y row only, and rows >= M are
+    // never stored
+    const _Float16* gp[GR];
+#pragma unroll
+    for (int r = 0; r < GR; r++) gp[r] = a.go + (int64_t)min(m0 + gm + 128 * r, a.M - 1) * a.ldg + gpart * 16;
+    // Two lanes 8 apart hold the same 16 k of rows n and n + 1.  They swap half of their values so that each
+    // writes whole dwords (n, n + 1) of the k-major tile: the even row's lane takes the first 8 of the 16
+    // values (pairs 0-3), the odd row's lane the rest.
+    const bool odd = wn & 1;
+    const uint32_t sel_lo = odd ? 0x01000504u : 0x05040100u, sel_hi = odd ? 0x03020706u : 0x07060302u;
+    const int b_dst = wks * (16 * DPITCH + 16) + (odd ? kmap<BITS>(4, 0) * DPITCH : 0) + (wn & ~1) * 2;
 
-    wload_t wreg;
-    _Float16 sreg, zreg;
-    u4 greg[2];
-    auto issue = [&](int step) {
-        const int64_t n0 = (int64_t)step * DN;
-        wreg = *reinterpret_cast<const wload_t*>(wp + n0 * a.row_bytes);
-        sreg = sp[n0 * a.groups];
-        zreg = zp[n0 * a.groups];
-        if (g_ok) {
-            greg[0] = *reinterpret_cast<const u4*>(gp + n0);
-            greg[1] = *reinterpret_cast<const u4*>(gp + n0 + 8);
-        } else {
-            greg[0] = greg[1] = u4{0u, 0u, 0u, 0u};
+    // PD steps of loads are in flight (a step's MFMAs take a fraction of a memory round trip).  Requests are
+    // unconditional - past the slice's end they repeat its last step - so the wait counts stay exact.
+    wload_t wreg[PD];
+    _Float16 sreg[PD], zreg[PD];
+    u4 greg[PD][2 * GR];
+    auto issue = [&](int step, int slot) {
+        const int64_t n0 = (int64_t)min(step, s_end - 1) * DN;
+        wreg[slot] = *reinterpret_cast<const wload_t*>(wp + n0 * a.row_bytes);
+        sreg[slot] = sp[n0 * a.groups];
+        zreg[slot] = zp[n0 * a.groups];
+#pragma unroll
+        for (int r = 0; r < GR; r++) {
+            greg[slot][2 * r] = *reinterpret_cast<const u4*>(gp[r] + n0);
+            greg[slot][2 * r + 1] = *reinterpret_cast<const u4*>(gp[r] + n0 + 8);
         }
     };
 
-    f4 acc[4][4];
+    f4 acc[4][MT];
 #pragma unroll
     for (int i = 0; i < 4; i++)
 #pragma unroll
-        for (int j = 0; j < 4; j++) acc[i][j] = f4{0.f, 0.f, 0.f, 0.f};
+        for (int j = 0; j < MT; j++) acc[i][j] = f4{0.f, 0.f, 0.f, 0.f};
 
-    const int wk = (wave & 1) * 64, wm = (wave >> 1) * 64;            // this wave's quarter of the tile
+    const int wk = (wave & 1) * 64, wm = (wave >> 1) * (16 * MT);     // this wave's quarter of the tile
     const int l16 = lane & 15, q = lane >> 4;
 
-    if (s_begin < s_end) issue(s_begin);
-    for (int step = s_begin; step < s_end; step++) {
-        char* As = smem + ((step - s_begin) & 1) * STAGE;
+    // slot -> LDS stage: dequantise the 16 weights and scatter them transposed; copy the grad_y rows
+    auto fill = [&](int slot, int stage, bool live) {
+        char* As = smem + stage * STAGE;
         char* Bs = As + A_BYTES;
-        // weights: dequantise, scatter transposed
-        {
-            GroupConst<BITS> gc;
-            gc.set(sreg, zreg);
-            h2 w16[8];
-            dequant16<BITS>(wreg, gc, w16);
+        GroupConst<BITS> gc;
+        gc.set(live ? sreg[slot] : (_Float16)0.f, zreg[slot]);        // past the slice's end: weights of zero
+        h2 w16[8];
+        dequant16<BITS>(wreg[slot], gc, w16);
 #pragma unroll
-            for (int p = 0; p < 8; p++)
-#pragma unroll
-                for (int h = 0; h < 2; h++) {
-                    const int k = wks * 16 + kmap<BITS>(p, h);
-                    *reinterpret_cast<_Float16*>(Bs + b_row_offset(k) + wn * 2) = w16[p][h];
-                }
-            u4* dst = reinterpret_cast<u4*>(As + gm * DPITCH + gpart * 32);
-            dst[0] = greg[0];
-            dst[1] = greg[1];
+        for (int i = 0; i < 4; i++) {
+            const uint32_t lo4 = as_u32(w16[i]), hi4 = as_u32(w16[4 + i]);
+            const uint32_t keep = odd ? hi4 : lo4, recv = dpp_xor8(odd ? lo4 : hi4);
+            *reinterpret_cast<uint32_t*>(Bs + b_dst + kmap<BITS>(i, 0) * DPITCH) = __builtin_amdgcn_perm(recv, keep, sel_lo);
+            *reinterpret_cast<uint32_t*>(Bs + b_dst + kmap<BITS>(i, 1) * DPITCH) = __builtin_amdgcn_perm(recv, keep, sel_hi);
         }
-        if (step + 1 < s_end) issue(step + 1);
+#pragma unroll
+        for (int r = 0; r < GR; r++) {
+            u4* dst = reinterpret_cast<u4*>(As + (gm + 128 * r) * DPITCH + gpart * 32);
+            dst[0] = greg[slot][2 * r];
+            dst[1] = greg[slot][2 * r + 1];
+        }
+    };
+
+    // Step s: read the fragments of stage s & 1, then - in the shadow of the step's MFMAs - fill the other
+    // stage with step s + 1 and request step s + 1 + PD.  One barrier per step: everybody has read the
+    // fragments of stage s & 1 before the next step overwrites it, and has written step s + 1 before it is read.
+    if (s_begin < s_end) {
+#pragma unroll
+        for (int d = 0; d < PD; d++) issue(s_begin + d, d);
+        fill(0, 0, true);
+        issue(s_begin + PD, 0);
         __syncthreads();
-        h8 af[4], bf[4];
+    }
+    // whole passes of PD steps, no early exit (the steps past the end multiply by zero weights): the loop body
+    // is one straight block, which keeps the compiler's count of outstanding loads exact
+    for (int base = s_begin; base < s_end; base += PD) {
 #pragma unroll
-        for (int i = 0; i < 4; i++) af[i] = *reinterpret_cast<const h8*>(Bs + b_row_offset(wk + 16 * i + l16) + q * 16);
+        for (int d = 0; d < PD; d++) {
+            const int step = base + d;
+            const char* As = smem + (d & 1) * STAGE;                  // PD is even: stages alternate across passes too
+            const char* Bs = As + A_BYTES;
+            h8 af[4], bf[MT];
 #pragma unroll
-        for (int j = 0; j < 4; j++) bf[j] = *reinterpret_cast<const h8*>(As + (wm + 16 * j + l16) * DPITCH + q * 16);
+            for (int i = 0; i < 4; i++) af[i] = *reinterpret_cast<const h8*>(Bs + b_row_offset(wk + 16 * i + l16) + q * 16);
 #pragma unroll
-        for (int i = 0; i < 4; i++)
+            for (int j = 0; j < MT; j++) bf[j] = *reinterpret_cast<const h8*>(As + (wm + 16 * j + l16) * DPITCH + q * 16);
+            fill((d + 1) % PD, (d + 1) & 1, step + 1 < s_end);
+            issue(step + 1 + PD, (d + 1) % PD);
 #pragma unroll
-            for (int j = 0; j < 4; j++)
-                acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[i], bf[j], acc[i][j], 0, 0, 0);
+            for (int j = 0; j < MT; j++)
+#pragma unroll
+                for (int i = 0; i < 4; i++)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[i], bf[j], acc[i][j], 0, 0, 0);
+            __syncthreads();
+        }
     }
 
     // acc[i][j][r] = grad_x[m0 + wm + 16 j + l16][k0 + wk + 16 i + 4 q + r]
@@ -153,11 +198,11 @@ __global__ __launch_bounds__(DTHREADS) void qdgrad_kernel(const DgradArgs a) {
 #pragma unroll
         for (int i = 0; i < 4; i++)
 #pragma unroll
-            for (int j = 0; j < 4; j++)
+            for (int j = 0; j < MT; j++)
                 *reinterpret_cast<f4*>(dst + (wm + 16 * j + l16) * DK + wk + 16 * i + 4 * q) = acc[i][j];
     } else {
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
+        for (int j = 0; j < MT; j++) {
             const int m = m0 + wm + 16 * j + l16;
             if (m >= a.M) continue;
 #pragma unroll
@@ -171,6 +216,7 @@ __global__ __launch_bounds__(DTHREADS) void qdgrad_kernel(const DgradArgs a) {
 }
 
 // grad_x tile = sum of its slices' partial tiles, rounded once
+template <int DM>
 __global__ __launch_bounds__(256) void qdgrad_reduce_kernel(const DgradArgs a) {
     const int tile = blockIdx.y;
     const int quad = (int)(blockIdx.x * blockDim.x + threadIdx.x);    // < DM * DK / 4
@@ -189,7 +235,7 @@ __global__ __launch_bounds__(256) void qdgrad_reduce_kernel(const DgradArgs a) {
 }
 
 struct DgradPlan {
-    int tiles_k, tiles, splits, steps_per_split;
+    int mt, tiles_k, tiles, splits, steps_per_split;
     size_t ws_bytes;
 };
 
@@ -203,19 +249,26 @@ inline int dgrad_cus() {
     return cus;
 }
 
-// Three workgroups fit a CU.  Fewer tiles than CUs: cut N so that every CU has one, never below 8 steps a slice.
+// Two workgroups fit a CU and hide each other's barriers.  With fewer tiles than that N is cut into slices: to two
+// workgroups per CU when a slice keeps at least 24 steps, else to one per CU with at least 8 (short slices pay
+// their prologue and the partial tiles' traffic).
 inline DgradPlan dgrad_plan(int64_t M, int64_t N, int64_t K, bool have_workspace) {
     DgradPlan p;
+    p.mt = 4;
+    const int DM = 32 * p.mt;
     p.tiles_k = (int)(K / DK);
     p.tiles = p.tiles_k * (int)((M + DM - 1) / DM);
     const int nsteps = (int)(N / DN);
     p.splits = 1;
     p.steps_per_split = nsteps;
     p.ws_bytes = 0;
+    if (!have_workspace) return p;
     const int cus = dgrad_cus();
-    if (!have_workspace || p.tiles >= cus) return p;
-    int s = (cus + p.tiles - 1) / p.tiles;
-    if (s > nsteps / 8) s = nsteps / 8;
+    int s = (2 * cus + p.tiles - 1) / p.tiles;
+    if (s < 2 || nsteps / s < 24) {
+        s = (cus + p.tiles - 1) / p.tiles;
+        if (s > nsteps / 8) s = nsteps / 8;
+    }
     if (s > 32) s = 32;
     if (s < 2) return p;
     const int sps = (nsteps + s - 1) / s;
@@ -232,6 +285,25 @@ inline bool dgrad_fast_shape(int64_t M, int64_t N, int64_t K, int64_t ldg, int64
            M >= 1 && M < ((int64_t)1 << 24) && N * (K * bits / 8) < ((int64_t)1 << 40);
 }
 
+template <int BITS, int GROUP, int MT>
+int launch_dgrad_mt(const DgradArgs& a, const DgradPlan& p, hipStream_t stream) {
+    constexpr int DM = DgradTile<MT>::DM;
+    auto kern = qdgrad_kernel<BITS, GROUP, MT>;
+    static bool attr_set = false;                          // per instantiation; benign if raced
+    if (2 * DgradTile<MT>::STAGE > 64 * 1024 && !attr_set) {
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) != hipSuccess)
+            return BW_ELAUNCH;
+        attr_set = true;
+    }
+    hipLaunchKernelGGL(kern, dim3((unsigned)(p.tiles * p.splits)), dim3(DTHREADS), 2 * DgradTile<MT>::STAGE, stream, a);
+    if (hipGetLastError() != hipSuccess) return BW_ELAUNCH;
+    if (p.splits > 1) {
+        hipLaunchKernelGGL(qdgrad_reduce_kernel<DM>, dim3(DM * DK / 4 / 256, (unsigned)p.tiles), dim3(256), 0, stream, a);
+        if (hipGetLastError() != hipSuccess) return BW_ELAUNCH;
+    }
+    return BW_OK;
+}
+
 template <int BITS, int GROUP>
 int launch_dgrad(DgradArgs a, void* workspace, size_t workspace_bytes, hipStream_t stream) {
     const DgradPlan p = dgrad_plan(a.M, a.N, a.K, workspace != nullptr);
@@ -240,13 +312,7 @@ int launch_dgrad(DgradArgs a, void* workspace, size_t workspace_bytes, hipStream
     a.tiles_k = p.tiles_k;
     a.splits = p.splits;
     a.steps_per_split = p.steps_per_split;
-    hipLaunchKernelGGL((qdgrad_kernel<BITS, GROUP>), dim3((unsigned)(p.tiles * p.splits)), dim3(DTHREADS), 2 * STAGE, stream, a);
-    if (hipGetLastError() != hipSuccess) return BW_ELAUNCH;
-    if (p.splits > 1) {
-        hipLaunchKernelGGL(qdgrad_reduce_kernel, dim3(DM * DK / 4 / 256, (unsigned)p.tiles), dim3(256), 0, stream, a);
-        if (hipGetLastError() != hipSuccess) return BW_ELAUNCH;
-    }
-    return BW_OK;
+    return launch_dgrad_mt<BITS, GROUP, 4>(a, p, stream);
 }
 
 }  // namespace

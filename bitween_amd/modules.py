@@ -12,6 +12,9 @@ import torch.nn as nn
 from .kernels import hip_loader as _hip
 
 
+FUSED_DGRAD_MAX_ROWS = 512       # measured on MI355X, Llama-shaped layers: fused wins up to here (3x at 128 rows)
+
+
 class QuantizedLinearFunction(torch.autograd.Function):
     """apply(x, qweight, scale, zero_point, bias, bits, group_size) -> float16 [..., N]
     (bitween/modules.py:62-106).  backward returns grad_input only
@@ -33,9 +36,11 @@ class QuantizedLinearFunction(torch.autograd.Function):
         x, qweight, scale, zero_point, bias = ctx.saved_tensors
         grad_input = None
         if ctx.needs_input_grad[0]:
-            # float16 gradients on kernel-sized shapes: one fused kernel, the weights are never materialised
-            if grad_output.dtype is torch.float16 and grad_output.is_cuda:
-                go2 = grad_output.reshape(-1, grad_output.shape[-1])
+            # float16 gradients, up to FUSED_DGRAD_MAX_ROWS rows: one fused kernel, the weights are never
+            # materialised.  Beyond that the library GEMM on dequantised weights is faster (the fused kernel
+            # re-dequantises the weights for every 128 rows of grad_output).
+            go2 = grad_output.reshape(-1, grad_output.shape[-1])
+            if grad_output.dtype is torch.float16 and grad_output.is_cuda and go2.shape[0] <= FUSED_DGRAD_MAX_ROWS:
                 gx = _hip.quantized_input_grad(go2, qweight, scale, zero_point, ctx.bits, ctx.group_size)
                 if gx is not None:
                     return gx.view(*grad_output.shape[:-1], gx.shape[-1]), None, None, None, None, None, None
