@@ -282,7 +282,7 @@ def extras_mixed_precision_model(torch, hip, QuantizedLinear, layers):
 def extras_decode_fused_siblings(torch, hip, QuantizedLinear, layers):
     """The headline step again with q/k/v and gate/up grouped by fuse_sibling_linears: the model still calls seven
     modules per layer, four launches run (a launch costs ~2.5 us before its first byte arrives).  Not the headline:
-    the caller has to opt in.  Run last: it re-points the layers' buffers at concatenated copies."""
+    the caller has to opt in.  Runs after every section that uses `layers`: it re-points their buffers at concatenated copies."""
     import bitween_amd
     names = [n for n, _, _ in LLAMA7B_LINEARS]
     blocks = []
@@ -434,7 +434,9 @@ def extras_backward(torch, hip, QuantizedLinear, layers):
 EXTRAS = {"decode": extras_decode, "decode_infinity_cache_hot": extras_decode_hot,
           "decode_other_formats": extras_decode_other_formats, "hipblaslt_fp16_decode": extras_hipblaslt_decode,
           "prefill": extras_prefill, "quantize": extras_quantize, "mixed_precision_model": extras_mixed_precision_model, "eager_call": extras_eager_call,
-          "llama7b_end_to_end": extras_llama7b_end_to_end, "backward": extras_backward, "decode_fused_siblings": extras_decode_fused_siblings}
+          "decode_fused_siblings": extras_decode_fused_siblings,
+          # the heavy sections last: the GEMMs and the 7B model leave the board warm, which shows in the decode timings
+          "backward": extras_backward, "llama7b_end_to_end": extras_llama7b_end_to_end}
 
 
 def main():

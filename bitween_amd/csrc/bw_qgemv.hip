@@ -103,23 +103,12 @@ __global__ __launch_bounds__((64 * GemvCfg<BITS, GROUP, MT>::MAX_WAVES)) void qg
                                  rs = make_rsrc(a.scale, a.meta_bytes), rz = make_rsrc(a.zp, a.meta_bytes);
 
     // ---- request everything of the first round, small things first (loads return in order) ----
-    // scales / zero points: thread t fetches pair index t, t + blockDim, ... of the 16 x groups block.  The first
-    // ME of them are requested ahead of x and the weights: a request made after those only returns behind the
-    // whole weight batch, and small groups at few bits have several pairs per thread (128 KB / (GROUP * BITS)
-    // when a wave holds KB chunks).  A wave skips requests that lie past the block (they would still cost a trip).
-    constexpr int ME = (512 / (GROUP * BITS)) > 8 ? 8 : ((512 / (GROUP * BITS)) < 1 ? 1 : (512 / (GROUP * BITS)));
+    // scales / zero points: thread t fetches pair index t (and t + blockDim, ...) of the 16 x groups block
     const uint32_t meta_base = (uint32_t)n0 * groups * 2;
-    const int meta_entries = 16 * groups;
-    uint16_t ms[ME], mz[ME];
-#pragma unroll
-    for (int j = 0; j < ME; j++) {
-        ms[j] = mz[j] = 0;
-        if ((wave + j * nwaves) * 64 < meta_entries) {              // wave-uniform
-            const int e = tid + j * (int)blockDim.x;
-            const uint32_t off = e < meta_entries ? meta_base + e * 2 : kOob;
-            ms[j] = __builtin_amdgcn_raw_buffer_load_b16(rs, off, 0, 0);
-            mz[j] = __builtin_amdgcn_raw_buffer_load_b16(rz, off, 0, 0);
-        }
+    uint16_t ms = 0, mz = 0;
+    if (tid < 16 * groups) {
+        ms = __builtin_amdgcn_raw_buffer_load_b16(rs, meta_base + tid * 2, 0, 0);
+        mz = __builtin_amdgcn_raw_buffer_load_b16(rz, meta_base + tid * 2, 0, 0);
     }
     u4 xr[XL * UW];
     u4 wr[KB];
@@ -143,15 +132,11 @@ __global__ __launch_bounds__((64 * GemvCfg<BITS, GROUP, MT>::MAX_WAVES)) void qg
     issue(c0);
 
     // ---- scales / zero points to LDS, once per workgroup ----
-#pragma unroll
-    for (int j = 0; j < ME; j++) {
-        const int e = tid + j * (int)blockDim.x;
-        if (e < meta_entries) {
-            const int r = e / groups, c = e - r * groups;
-            meta[r * GP + c] = (uint32_t)ms[j] | ((uint32_t)mz[j] << 16);
-        }
+    if (tid < 16 * groups) {
+        const int r = tid / groups, c = tid - r * groups;
+        meta[r * GP + c] = (uint32_t)ms | ((uint32_t)mz << 16);
     }
-    for (int e = tid + ME * blockDim.x; e < meta_entries; e += blockDim.x) {   // more pairs than that
+    for (int e = tid + blockDim.x; e < 16 * groups; e += blockDim.x) {   // more pairs than threads
         const int r = e / groups, c = e - r * groups;
         const uint32_t s2 = __builtin_amdgcn_raw_buffer_load_b16(rs, meta_base + e * 2, 0, 0);
         const uint32_t z2 = __builtin_amdgcn_raw_buffer_load_b16(rz, meta_base + e * 2, 0, 0);
