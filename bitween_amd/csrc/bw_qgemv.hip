@@ -458,6 +458,251 @@ int launch_w4(const GemvArgs& a, hipStream_t stream) {
     return launch_w4_kb<GROUP, MT, 4>(a, stream);
 }
 
+// ---- 2-bit, M <= 2: the same integer-operand scheme ---------------------------------------------------------
+//
+// A masked 2-bit field at bits 2c..2c+1 (c = 0..3) of a half is the subnormal q * 4^c * 2^-24; the fields at bits
+// 8-15 are brought down by one shift.  A word of 16 weights unpacks with 1 shift + 8 ANDs into four operand
+// classes; class c accumulates in its own register quad and  sum x q = 2^24 (P0 + P1/4 + P2/16 + P3/64).
+// A chunk is 256 weights of a row: 2, 4 or 8 groups.  Row m * NGC + g of the MFMA tile carries group g of
+// activation row m: a lane reads its A operand from the staged x only where its 32-value slice lies in that
+// group and from a row of zeros elsewhere, so output row m * NGC + g is the group's partial sum.
+template <int LANES>
+BW_DEV float lanes_sum_small(float v) {                  // aligned runs of 2, 4 or 8 lanes
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true));
+    if constexpr (LANES >= 4)
+        v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, true));
+    if constexpr (LANES >= 8)
+        v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xF, 0xF, true));
+    return v;
+}
+
+template <int GROUP, int MT, int KB>
+__global__ __launch_bounds__(1024) void qgemv_w2_kernel(const GemvArgs a) {
+    constexpr int NGC = 256 / GROUP;                      // groups per chunk
+    constexpr int ROWS = MT * NGC;                        // MFMA rows in use: (m, group of the chunk)
+    static_assert(ROWS <= 16, "one MFMA tile of rows");
+    constexpr int SPG = GROUP / 32;                       // 32-value slices (half a lane load) per group
+    constexpr int UPR = KB * 16;                          // 16-value units per activation row and round
+    constexpr int XL = (MT * UPR + 63) / 64;              // unit loads per lane and round
+    constexpr int ROW_BYTES = KB * 512 + 16;
+    constexpr int X_BYTES = (MT + 1) * ROW_BYTES;         // the staged rows and one row of zeros
+    constexpr int NS_BYTES = MT * KB * NGC * 4;
+    constexpr int WAVE_BYTES = (X_BYTES + NS_BYTES + 15) & ~15;
+    constexpr uint32_t kOob = 0x80000000u;
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nwaves = blockDim.x >> 6;
+    const int nl = lane & 15, kq = lane >> 4;
+    const int n0 = blockIdx.x * 16;
+    // LDS: [(scale, zero point) pairs, 16 rows x GP][wave 0: x rows, zero row, group sums] ... [partial sums]
+    const int gcols = (a.groups + 31) & ~31, GP = gcols + 1;
+    uint32_t* meta = reinterpret_cast<uint32_t*>(smem);
+    char* after_meta = smem + ((16 * GP * 4 + 15) & ~15);
+    char* xs = after_meta + wave * WAVE_BYTES;
+    float* nsb = reinterpret_cast<float*>(xs + X_BYTES);
+    float* red = reinterpret_cast<float*>(after_meta + nwaves * WAVE_BYTES);
+    const __amdgpu_buffer_rsrc_t rw = make_rsrc(a.qweight, a.w_bytes), rx = make_rsrc(a.x, a.x_bytes),
+                                 rs = make_rsrc(a.scale, a.meta_bytes), rz = make_rsrc(a.zp, a.meta_bytes);
+
+    constexpr int ME = GROUP == 32 ? 4 : (GROUP == 64 ? 2 : 1);
+    const uint32_t meta_base = (uint32_t)n0 * a.groups * 2;
+    const int meta_entries = 16 * gcols;
+    auto meta_off = [&](int e) {
+        const int r = (e >> 5) & 15, c = (e & 31) + 32 * (e >> 9);
+        return c < a.groups ? meta_base + (r * a.groups + c) * 2 : kOob;
+    };
+    auto meta_slot = [&](int e) { return ((e >> 5) & 15) * GP + (e & 31) + 32 * (e >> 9); };
+    uint32_t ms[ME], mz[ME];
+#pragma unroll
+    for (int j = 0; j < ME; j++) {
+        ms[j] = mz[j] = 0;
+        if ((wave + j * nwaves) * 64 < meta_entries) {          // wave-uniform
+            const uint32_t off = meta_off(tid + j * (int)blockDim.x);
+            ms[j] = __builtin_amdgcn_raw_buffer_load_b16(rs, off, 0, 0);
+            mz[j] = __builtin_amdgcn_raw_buffer_load_b16(rz, off, 0, 0);
+        }
+    }
+
+    const uint32_t w_lane = (uint32_t)(n0 + nl) * a.row_bytes + kq * 16;
+    // unit u = lane + 64 i of the round: activation row u / UPR, chunk b, 16-value unit w of the chunk; unit w is
+    // word j = w % 4 of the 64-value slice kq_x = w / 4.  Class c of the unit goes to operand (p = j / 2, c) of
+    // the lanes with kq == kq_x, second half if j is odd.
+    uint32_t x_off[XL], x_dst[XL], ns_dst[XL];
+#pragma unroll
+    for (int i = 0; i < XL; i++) {
+        const int u = lane + 64 * i, m = u / UPR, rest = u % UPR, b = rest >> 4, w = rest & 15;
+        x_off[i] = m < a.M ? (uint32_t)(m * a.ldx + b * 256 + w * 16) * 2 : kOob;
+        x_dst[i] = m * ROW_BYTES + b * 512 + ((w >> 1) & 1) * 256 + (w >> 2) * 16 + (w & 1) * 8;
+        ns_dst[i] = (m * KB + b) * NGC + (w * 16) / GROUP;
+    }
+    u4 xr[XL][2], wr[KB];
+    auto issue = [&](int c0) {
+#pragma unroll
+        for (int i = 0; i < XL; i++) {
+            const int rest = (lane + 64 * i) % UPR;
+            const uint32_t xo = (x_off[i] != kOob && c0 * 256 + rest * 16 < a.K) ? x_off[i] + c0 * 512 : kOob;
+            xr[i][0] = __builtin_amdgcn_raw_buffer_load_b128(rx, xo, 0, 0);
+            xr[i][1] = __builtin_amdgcn_raw_buffer_load_b128(rx, xo == kOob ? kOob : xo + 16, 0, 0);
+        }
+        asm volatile("" ::: "memory");
+        const uint32_t off = c0 * 64 < a.row_bytes ? w_lane + c0 * 64 : kOob;
+#pragma unroll
+        for (int b = 0; b < KB; b++) wr[b] = __builtin_amdgcn_raw_buffer_load_b128(rw, off + b * 64, 0, 0);
+        asm volatile("" ::: "memory");
+    };
+    int c0 = wave * KB;
+    issue(c0);
+
+#pragma unroll
+    for (int j = 0; j < ME; j++) {
+        const int e = tid + j * (int)blockDim.x;
+        if (e < meta_entries) meta[meta_slot(e)] = ms[j] | (mz[j] << 16);
+    }
+    for (int e = tid + ME * (int)blockDim.x; e < meta_entries; e += blockDim.x) {
+        const uint32_t off = meta_off(e);
+        const uint32_t s2 = __builtin_amdgcn_raw_buffer_load_b16(rs, off, 0, 0);
+        const uint32_t z2 = __builtin_amdgcn_raw_buffer_load_b16(rz, off, 0, 0);
+        meta[meta_slot(e)] = s2 | (z2 << 16);
+    }
+    // the row of zeros behind the staged rows
+    for (int o = lane * 4; o < ROW_BYTES; o += 256) *reinterpret_cast<uint32_t*>(xs + MT * ROW_BYTES + o) = 0u;
+    __syncthreads();
+
+    // this lane's MFMA row: activation row and group of the chunk; its two 32-value slices (p = 0, 1) are live
+    // where they lie in that group
+    const int row_m = nl / NGC < MT ? nl / NGC : MT - 1, row_g = nl % NGC;
+    const char* xbase[2];
+#pragma unroll
+    for (int p = 0; p < 2; p++) {
+        const bool live = nl < ROWS && (2 * kq + p) / SPG == row_g;
+        xbase[p] = xs + (live ? row_m : MT) * ROW_BYTES + p * 256 + kq * 16;
+    }
+    // the four output rows this lane holds: rows 4 kq + r
+    int out_m[4], out_g[4];
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+        const int row = 4 * kq + r;
+        out_m[r] = row / NGC < MT ? row / NGC : MT - 1;
+        out_g[r] = row % NGC;
+    }
+    f4 acc = {0.f, 0.f, 0.f, 0.f};
+    const uint32_t* mrow = meta + nl * GP;
+    while (true) {
+        // stage the round's activations: per 16 values the pairs (x_f, x_f+8), f = 0..7, which is the order in which
+        // the masks below emit the fields of a word; class c takes pairs c and c + 4.  And -2^-24 sum(x) per group.
+#pragma unroll
+        for (int i = 0; i < XL; i++) {
+            uint32_t in[8], o[8];
+#pragma unroll
+            for (int j = 0; j < 4; j++) { in[j] = xr[i][0][j]; in[4 + j] = xr[i][1][j]; }
+            permute_unit<2>(in, o);
+            const bool mine = MT * UPR >= 64 * (i + 1) || lane + 64 * i < MT * UPR;
+            if (mine) {
+#pragma unroll
+                for (int c = 0; c < 4; c++) *reinterpret_cast<u2*>(xs + x_dst[i] + c * 64) = u2{o[c], o[c + 4]};
+            }
+            float t = 0.f;
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                const h2 pr = __builtin_bit_cast(h2, in[j]);
+                t -= (float)pr[0];
+                t -= (float)pr[1];
+            }
+            t = lanes_sum_small<GROUP / 16>(t) * 0x1p-24f;
+            if (mine && (lane & (GROUP / 16 - 1)) == 0) nsb[ns_dst[i]] = t;
+        }
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int b = 0; b < KB; b++) {
+            const u4 w = wr[b];
+            f4 pc[4];
+#pragma unroll
+            for (int c = 0; c < 4; c++) pc[c] = f4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int p = 0; p < 2; p++) {
+                const uint32_t wa = w[2 * p], sa = wa >> 8, wb = w[2 * p + 1], sb = wb >> 8;
+#pragma unroll
+                for (int c = 0; c < 4; c++) {
+                    const uint32_t mask = 0x00030003u << (2 * c);
+                    const u4 bop = {wa & mask, sa & mask, wb & mask, sb & mask};
+                    const h8 xa = *reinterpret_cast<const h8*>(xbase[p] + b * 512 + c * 64);
+                    pc[c] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa, __builtin_bit_cast(h8, bop), pc[c], 0, 0, 0);
+                }
+            }
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                const uint32_t sz = mrow[min((c0 + b) * NGC + out_g[r], gcols - 1)];   // chunks past K: zero weights and x
+                const float sf = half_of(sz, 0), zf = half_of(sz, 1);
+                const float ns = nsb[(out_m[r] * KB + b) * NGC + out_g[r]];
+                float t = __builtin_fmaf(pc[3][r], 0.25f, pc[2][r]);
+                t = __builtin_fmaf(t, 0.25f, pc[1][r]);
+                t = __builtin_fmaf(t, 0.25f, pc[0][r]);
+                acc[r] = __builtin_fmaf(sf, __builtin_fmaf(zf, ns, t), acc[r]);
+            }
+        }
+        c0 += nwaves * KB;
+        if (c0 >= a.nchunks) break;                       // wave-uniform
+        __builtin_amdgcn_wave_barrier();
+        issue(c0);
+    }
+
+    // acc[r] = 2^-24 * partial of row 4 kq + r = (m, g); add the groups of each m, one value per (m, n) and wave
+    if constexpr (NGC >= 4) {
+        float v = (acc[0] + acc[1]) + (acc[2] + acc[3]);
+        if constexpr (NGC == 8) v += __shfl_xor(v, 16);
+        const int m = (4 * kq) / NGC;
+        if (m < MT && (NGC == 4 || (kq & 1) == 0)) red[(wave * MT + m) * 16 + nl] = v;
+    } else {
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            const int m = 2 * kq + h;
+            if (m < MT) red[(wave * MT + m) * 16 + nl] = acc[2 * h] + acc[2 * h + 1];
+        }
+    }
+    __syncthreads();
+    for (int m = wave; m < MT; m += nwaves) {
+        float v = 0.f;
+        for (int w = kq; w < nwaves; w += 4) v += red[(w * MT + m) * 16 + nl];
+        v += __shfl_xor(v, 16);
+        v += __shfl_xor(v, 32);
+        const int n = n0 + nl;
+        if (kq == 0 && m < a.M && n < a.N) {
+            v *= 0x1p24f;
+            if (a.bias) v += (float)a.bias[n];
+            a.y[(int64_t)m * a.ldy + n] = (_Float16)v;
+        }
+    }
+}
+
+template <int GROUP, int MT, int KB>
+int launch_w2_kb(const GemvArgs& a, hipStream_t stream) {
+    constexpr int NGC = 256 / GROUP;
+    constexpr int WAVE_BYTES = ((MT + 1) * (KB * 512 + 16) + MT * KB * NGC * 4 + 15) & ~15;
+    const int gcols = (a.groups + 31) & ~31;
+    const size_t fixed = (size_t)((16 * (gcols + 1) * 4 + 15) & ~15);
+    int nwaves = (a.nchunks + KB - 1) / KB;
+    if (nwaves > 16) nwaves = 16;
+    while (nwaves > 1 && fixed + (size_t)nwaves * (WAVE_BYTES + MT * 64) > (size_t)150 * 1024) nwaves--;
+    const size_t lds = fixed + (size_t)nwaves * (WAVE_BYTES + MT * 64);
+    if (lds > (size_t)150 * 1024) return BW_EUNSUPPORTED;
+    auto kern = qgemv_w2_kernel<GROUP, MT, KB>;
+    static bool attr_set = false;                          // per instantiation; benign if raced
+    if (lds > 64 * 1024 && !attr_set) {
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) != hipSuccess)
+            return BW_ELAUNCH;
+        attr_set = true;
+    }
+    hipLaunchKernelGGL(kern, dim3((unsigned)((a.N + 15) / 16)), dim3(nwaves * 64), lds, stream, a);
+    return hipGetLastError() == hipSuccess ? BW_OK : BW_ELAUNCH;
+}
+
+template <int GROUP, int MT>
+int launch_w2(const GemvArgs& a, hipStream_t stream) {
+    // chunks a wave has in flight per round: rows are short at 2 bits (K = 4096 is 16 chunks), so 2, and 1 where
+    // groups of 32 make the scale block as large as half the weights
+    if (GROUP == 32 && a.nchunks <= 16) return launch_w2_kb<GROUP, MT, 1>(a, stream);
+    return launch_w2_kb<GROUP, MT, 2>(a, stream);
+}
+
 constexpr int kLdsBudget = 150 * 1024;
 
 template <int BITS, int GROUP, int MT, int KB>
@@ -510,6 +755,12 @@ int launch_gemv(const GemvArgs& a, hipStream_t stream) {
         const bool pays = GROUP != 64 || (int64_t)a.N * a.K > (int64_t)1 << 25;
         if (a.M * (128 / GROUP) <= 4 && a.M <= 2 && pays) {
             const int st = a.M == 1 ? launch_w4<GROUP, 1>(a, stream) : launch_w4<GROUP, (GROUP >= 64 ? 2 : 1)>(a, stream);
+            if (st != BW_EUNSUPPORTED) return st;
+        }
+    }
+    if constexpr (BITS == 2) {
+        if (a.M <= 2) {
+            const int st = a.M == 1 ? launch_w2<GROUP, 1>(a, stream) : launch_w2<GROUP, 2>(a, stream);
             if (st != BW_EUNSUPPORTED) return st;
         }
     }
