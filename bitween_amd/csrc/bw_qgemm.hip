@@ -561,7 +561,7 @@ extern "C" int bw_qlinear(const void* x, int act_dtype, int64_t M, int64_t K, in
                           void* y, int64_t ldy, void* stream) {
     // up to 48 rows the HBM-bound kernel, 16 rows per launch (the later launches find the weights in L2),
     // beats a mostly empty 128-row MFMA tile
-    if (M >= 1 && M <= 48 && act_dtype == BW_F16) {
+    if (M >= 1 && M <= 48 && (act_dtype == BW_F16 || act_dtype == BW_BF16)) {
         for (int64_t m0 = 0; m0 < M; m0 += 16) {
             const int st = bw_qgemv((const _Float16*)x + m0 * ldx, act_dtype, M - m0 < 16 ? M - m0 : 16, K, ldx, qweight, scale16,
                                     zp16, bias, N, bits, group, (_Float16*)y + m0 * ldy, ldy, stream);

@@ -74,7 +74,14 @@ struct GemvArgs {
     uint32_t x_bytes, w_bytes, meta_bytes;   // extents for the buffer range checks
     int M, N, K, ldx, ldy;
     int groups, nchunks, row_bytes;
+    int x_bf16;                              // x holds bfloat16: every value is rounded to float16 as it is staged
 };
+
+// two bfloat16 -> two float16, round to nearest even (what torch's .to(float16) does)
+BW_DEV uint32_t bf16x2_to_f16x2(uint32_t w) {
+    const float lo = __builtin_bit_cast(float, w << 16), hi = __builtin_bit_cast(float, w & 0xFFFF0000u);
+    return as_u32(h2{(_Float16)lo, (_Float16)hi});
+}
 
 BW_DEV __amdgpu_buffer_rsrc_t make_rsrc(const void* p, uint32_t bytes) {
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), (short)0, (int)bytes, 0x00020000);
@@ -156,6 +163,10 @@ __global__ __launch_bounds__((64 * GemvCfg<BITS, GROUP, MT>::MAX_WAVES)) void qg
                 uint32_t in[4 * UW], o[4 * UW];
 #pragma unroll
                 for (int j = 0; j < UW; j++) { in[4 * j] = xr[i * UW + j][0]; in[4 * j + 1] = xr[i * UW + j][1]; in[4 * j + 2] = xr[i * UW + j][2]; in[4 * j + 3] = xr[i * UW + j][3]; }
+                if (a.x_bf16) {
+#pragma unroll
+                    for (int j = 0; j < 4 * UW; j++) in[j] = bf16x2_to_f16x2(in[j]);
+                }
                 permute_unit<BITS>(in, o);
                 u4* dst = reinterpret_cast<u4*>(xs + m * PITCH + ku * C::UNIT);
 #pragma unroll
@@ -347,7 +358,11 @@ __global__ __launch_bounds__(1024) void qgemv_w4_kernel(const GemvArgs a) {
         float nsum[XL];
 #pragma unroll
         for (int i = 0; i < XL; i++) {
-            const u4 v = xr[i];
+            u4 v = xr[i];
+            if (a.x_bf16) {
+#pragma unroll
+                for (int j = 0; j < 4; j++) v[j] = bf16x2_to_f16x2(v[j]);
+            }
             u2 ev, od;
             ev[0] = __builtin_amdgcn_perm(v[2], v[0], 0x05040100u);
             ev[1] = __builtin_amdgcn_perm(v[3], v[1], 0x05040100u);
@@ -594,6 +609,10 @@ __global__ __launch_bounds__(1024) void qgemv_w2_kernel(const GemvArgs a) {
             uint32_t in[8], o[8];
 #pragma unroll
             for (int j = 0; j < 4; j++) { in[j] = xr[i][0][j]; in[4 + j] = xr[i][1][j]; }
+            if (a.x_bf16) {
+#pragma unroll
+                for (int j = 0; j < 8; j++) in[j] = bf16x2_to_f16x2(in[j]);
+            }
             permute_unit<2>(in, o);
             const bool mine = MT * UPR >= 64 * (i + 1) || lane + 64 * i < MT * UPR;
             if (mine) {
@@ -789,7 +808,7 @@ extern "C" int bw_qgemv(const void* x, int act_dtype, int64_t M, int64_t K, int6
                         void* y, int64_t ldy, void* stream) {
     if (!x || !qweight || !scale16 || !zp16 || !y) return BW_EINVAL;
     if (!bw_shape_ok(N, K, bits, group) || M < 1 || M > 16 || ldx < K || ldy < N) return BW_EINVAL;
-    if (act_dtype != BW_F16) return BW_EUNSUPPORTED;
+    if (act_dtype != BW_F16 && act_dtype != BW_BF16) return BW_EUNSUPPORTED;
     if (!bw_fast_shape(M, N, K, ldx, bits, group) || !bw_aligned(x, 16) || (ldx * 2) % 16 || !bw_aligned(qweight, 16))
         return bw_qgemm_generic(x, act_dtype, M, K, ldx, qweight, scale16, zp16, bias, N, bits, group, y, ldy, stream);
     GemvArgs a;
@@ -797,6 +816,7 @@ extern "C" int bw_qgemv(const void* x, int act_dtype, int64_t M, int64_t K, int6
     a.M = (int)M; a.N = (int)N; a.K = (int)K; a.ldx = (int)ldx; a.ldy = (int)ldy;
     a.groups = (int)(K / group);
     a.row_bytes = (int)(K * bits / 8);
+    a.x_bf16 = act_dtype == BW_BF16;
     a.nchunks = (a.row_bytes + 63) / 64;
     a.x_bytes = (uint32_t)(((M - 1) * ldx + K) * 2);
     a.w_bytes = (uint32_t)(N * a.row_bytes);

@@ -167,10 +167,19 @@ def _matmul(entry, x, qweight, scale, zero_point, bias, bits, group_size):
         raise ValueError("x must be [M, K]")
     if qweight.dtype is not torch.int32 or scale.dtype is not torch.float16 or zero_point.dtype is not torch.float16:
         raise TypeError("qweight must be int32 and scale / zero_point float16 (the QuantizedLinear buffers)")
-    if x.dtype is not torch.float16:
-        raise TypeError("x must be float16")
+    m = x.shape[0]
+    act = BW_F16
+    if x.dtype is torch.bfloat16:
+        # the decode kernels round bfloat16 to float16 as they stage x (the reference's x.to(float16),
+        # bitween/modules.py:74, without the extra kernel); the prefill kernel wants float16 in memory
+        if entry == "bw_qgemv" or (entry == "bw_qlinear" and m <= 48):
+            act = BW_BF16
+        else:
+            x = x.to(torch.float16)
+    elif x.dtype is not torch.float16:
+        raise TypeError("x must be float16 or bfloat16")
     if bias is not None and bias.dtype is not torch.float16:
-        raise TypeError("bias must have the dtype of x")
+        raise TypeError("bias must be float16")
     ldx = x.stride(0)
     if x.stride(1) != 1 or (ldx * 2) % 16 or x.data_ptr() % 16:
         x = x.contiguous().clone()
@@ -206,8 +215,12 @@ def _matmul(entry, x, qweight, scale, zero_point, bias, bits, group_size):
                                  None if ws is None else ws.data_ptr(), nbytes, _raw_stream(index))
             entry = "bw_qgemm_ws"
         else:
-            st = _ENTRY[entry](x.data_ptr(), BW_F16, m, k, ldx, qweight.data_ptr(), scale.data_ptr(),
+            st = _ENTRY[entry](x.data_ptr(), act, m, k, ldx, qweight.data_ptr(), scale.data_ptr(),
                                zero_point.data_ptr(), bias_ptr, n, bits, group_size, y.data_ptr(), n, _raw_stream(index))
+            if st == -2 and act == BW_BF16:                # a shape only the generic kernel takes: float16 in memory
+                x = x.to(torch.float16)
+                st = _ENTRY[entry](x.data_ptr(), BW_F16, m, k, x.stride(0), qweight.data_ptr(), scale.data_ptr(),
+                                   zero_point.data_ptr(), bias_ptr, n, bits, group_size, y.data_ptr(), n, _raw_stream(index))
     if st:
         _check(st, entry)
     return y

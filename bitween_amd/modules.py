@@ -89,7 +89,7 @@ class QuantizedLinear(nn.Module):
         # nothing to differentiate (the buffers never require grad): same arithmetic without the autograd node
         shape = x.shape
         x2 = x.reshape(-1, shape[-1])
-        if x2.dtype is not torch.float16:
+        if x2.dtype is not torch.float16 and x2.dtype is not torch.bfloat16:    # bfloat16 is converted by the kernel
             x2 = x2.to(torch.float16)
         y = _hip.quantized_matmul_hip(x2, self.qweight, self.scale, self.zero_point, self.bias, self.bits, self.group_size)
         return y.view(*shape[:-1], self.out_features)
@@ -184,7 +184,7 @@ class _SiblingGroup:
             self.wasted = self.wasted + 1 if self._served == 1 else 0
             shape = x.shape
             x2 = x.reshape(-1, shape[-1])
-            if x2.dtype is not torch.float16:
+            if x2.dtype is not torch.float16 and x2.dtype is not torch.bfloat16:
                 x2 = x2.to(torch.float16)
             y = _hip.quantized_matmul_hip(x2, self.qweight, self.scale, self.zero_point, self.bias, self.bits, self.group_size)
             self._y = y.view(*shape[:-1], y.shape[-1])

@@ -87,10 +87,13 @@ int bw_dequantize(const int32_t* qweight, const void* scale, int scale_dtype, co
  * reference dequantizes; products accumulate in float32; y is rounded once
  * (the reference rounds before and after the bias add; within its 1e-2
  * tolerance, main.py:471-477).
- *   x      [M][ldx] of act_dtype (BW_F16; BW_BF16 where noted), y [M][ldy] same dtype
+ *   x      [M][ldx] of act_dtype: BW_F16, or BW_BF16 for bw_qgemv and for bw_qlinear up to 48 rows - the
+ *          kernel then rounds every value to float16 as it reads it, which is the reference's
+ *          x.to(float16) (bitween/modules.py:74) without a separate pass; other entry points return
+ *          BW_EUNSUPPORTED for BW_BF16.  y [M][ldy] is float16 in every case, as in the reference.
  *   scale16, zp16  float16 [N][K/group] (the module buffers); zp16 must hold
  *                  integers in [0, 2^bits), as every quantizer here produces
- *   bias   [N] of act_dtype or NULL
+ *   bias   [N] float16 or NULL
  * bw_qgemv: decode path, 1 <= M <= 16, HBM-bound, no workspace.
  * bw_qgemm: prefill path, any M >= 1, MFMA-bound.
  * bw_qlinear: picks between them by M (what the Python forward calls): the decode kernel, 16 rows per

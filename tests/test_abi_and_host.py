@@ -46,8 +46,9 @@ def test_entry_points_reject_bad_arguments_before_touching_the_gpu():
     # M out of range for the decode kernel
     assert lib.bw_qgemv(one, 0, 17, 128, 128, one, one, one, None, 16, 4, 32, one, 16, None) == -1
     assert lib.bw_qgemv(one, 0, 0, 128, 128, one, one, one, None, 16, 4, 32, one, 16, None) == -1
-    # bf16 activations are not built
-    assert lib.bw_qgemv(one, 1, 1, 128, 128, one, one, one, None, 16, 4, 32, one, 16, None) == -2
+    # float32 activations are not built (bfloat16 is, for the decode kernels only)
+    assert lib.bw_qgemv(one, 2, 1, 128, 128, one, one, one, None, 16, 4, 32, one, 16, None) == -2
+    assert lib.bw_qgemm(one, 1, 128, 128, 128, one, one, one, None, 16, 4, 32, one, 16, None) == -2
     # split-K prefill: same checks as bw_qgemm, before the workspace is looked at
     assert lib.bw_qgemm_ws(None, 0, 128, 128, 128, one, one, one, None, 16, 4, 32, one, 16, None, 0, None) == -1
     assert lib.bw_qgemm_ws(one, 0, 128, 128, 64, one, one, one, None, 16, 4, 32, one, 16, None, 0, None) == -1

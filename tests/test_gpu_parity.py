@@ -512,3 +512,32 @@ def test_full_size_properties(bits, g, k, n):
     x = torch.randn(256, k, device="cuda", dtype=torch.float16, generator=g_t)
     y = q(x)
     check_matmul(y[:, rows], x.cpu().numpy(), qw_o, s16, z16, None, bits, g)
+
+
+@pytest.mark.parametrize("bits,g", COMBOS)
+def test_bfloat16_activations_are_rounded_to_float16_in_the_kernel(bits, g):
+    """x.to(float16) of the reference's forward (bitween/modules.py:74) fused into the decode kernels: a bfloat16 x
+    gives bit for bit what its float16 rounding gives, for every decode kernel variant, through bw_qlinear's 16-row
+    slices and (cast on the host side) through the prefill kernel; tiny and huge values included."""
+    hip = _hip()
+    k, n = 1024, 272
+    _, qw, s16, z16, b16 = quantized_layer(n, k, bits, g, seed=bits * 31 + g, outliers=True)
+    d = [to_gpu(a) for a in (qw, s16, z16, b16)]
+    gen = torch.Generator(device="cuda").manual_seed(bits + g)
+    for m in (1, 2, 3, 8, 16, 17, 48, 64):
+        xb = torch.randn(m, k, device="cuda", generator=gen).to(torch.bfloat16)
+        xb[0, 0] = 3.0e-6          # below the float16 normal range: rounds to a subnormal
+        xb[0, 1] = 1.0e-9          # rounds to zero
+        xb[0, 2] = 60000.0
+        xh = xb.to(torch.float16)
+        y_b = hip.quantized_matmul_hip(xb, d[0], d[1], d[2], d[3], bits, g)
+        y_h = hip.quantized_matmul_hip(xh, d[0], d[1], d[2], d[3], bits, g)
+        assert y_b.dtype == torch.float16 and torch.equal(y_b, y_h)
+        if m <= 16:
+            assert torch.equal(hip.quantized_gemv_hip(xb, d[0], d[1], d[2], d[3], bits, g), y_h)
+    check_matmul(y_b, xh.cpu().numpy(), qw, s16, z16, b16, bits, g)
+    import bitween_amd
+    q = bitween_amd.QuantizedLinear(k, n, bits=bits, group_size=g, bias=True).cuda()
+    q.qweight.copy_(d[0]); q.scale.copy_(d[1]); q.zero_point.copy_(d[2]); q.bias.copy_(d[3])
+    xb = torch.randn(2, 3, k, device="cuda", generator=gen).to(torch.bfloat16)
+    assert torch.equal(q(xb), q(xb.to(torch.float16)))
