@@ -167,7 +167,8 @@ def extras_hipblaslt_decode(torch, hip, QuantizedLinear, layers):
 
 
 def extras_prefill(torch, hip, QuantizedLinear, layers):
-    """Prefill on the Llama-3-8B MLP shapes, W4 g128, next to fp16 hipBLASLt on the dequantised weights."""
+    """Prefill on the Llama-3-8B MLP shapes, W4 g128, next to fp16 hipBLASLt on the dequantised weights.  `us` is
+    the kernel on float16 x; `bf16_x_us` the forward on bfloat16 x (cast + split-K workspace + kernel)."""
     bits, g, out = 4, 128, {}
     for k, n in ((4096, 14336), (14336, 4096)):
         q = make_layer(torch, QuantizedLinear, k, n, bits, g, seed=7)
@@ -176,8 +177,12 @@ def extras_prefill(torch, hip, QuantizedLinear, layers):
             x = torch.randn(mm, k, device="cuda", dtype=torch.float16)
             us_q = time_calls(torch, lambda: hip.quantized_gemm_hip(x, q.qweight, q.scale, q.zero_point, None, bits, g), 20, 5)
             us_b = time_calls(torch, lambda: torch.matmul(x, w16.T), 20, 5)
+            # the configuration names bfloat16 activations: the reference's forward casts them to float16
+            # (bitween/modules.py:74) and so does this one, in a pass of its own ahead of the prefill kernel
+            xb = x.to(torch.bfloat16)
+            us_qb = time_calls(torch, lambda: hip.quantized_matmul_hip(xb, q.qweight, q.scale, q.zero_point, None, bits, g), 20, 5)
             fl = 2.0 * mm * n * k
-            out[f"{k}x{n}_M{mm}"] = {"us": round(us_q, 1), "TFLOPs": round(fl / us_q / 1e6, 1),
+            out[f"{k}x{n}_M{mm}"] = {"us": round(us_q, 1), "bf16_x_us": round(us_qb, 1), "TFLOPs": round(fl / us_q / 1e6, 1),
                                      "pct_mfma_f16_peak": round(100 * fl / us_q / 1e6 / MFMA_F16_PEAK_TFLOPS, 1),
                                      "hipblaslt_fp16_us": round(us_b, 1), "hipblaslt_fp16_TFLOPs": round(fl / us_b / 1e6, 1),
                                      "frac_of_hipblaslt": round(us_b / us_q, 3)}
