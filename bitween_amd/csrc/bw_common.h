@@ -171,3 +171,15 @@ static inline bool bw_shape_ok(int64_t N, int64_t K, int bits, int group) {
            N < (int64_t)1 << 31 && K < (int64_t)1 << 31;
 }
 static inline bool bw_aligned(const void* p, size_t a) { return ((uintptr_t)p & (a - 1)) == 0; }
+
+// A kernel that wants more than 64 KiB of dynamic LDS has to be told so once per device.  `done` is the caller's
+// static bit mask of devices already served for that kernel (a race sets the attribute twice, which is harmless).
+static inline bool bw_allow_big_lds(const void* kernel, uint64_t& done) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return false;
+    const uint64_t bit = 1ull << (dev & 63);
+    if (done & bit) return true;
+    if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) != hipSuccess) return false;
+    done |= bit;
+    return true;
+}

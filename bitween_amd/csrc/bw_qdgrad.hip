@@ -289,12 +289,8 @@ template <int BITS, int GROUP, int MT>
 int launch_dgrad_mt(const DgradArgs& a, const DgradPlan& p, hipStream_t stream) {
     constexpr int DM = DgradTile<MT>::DM;
     auto kern = qdgrad_kernel<BITS, GROUP, MT>;
-    static bool attr_set = false;                          // per instantiation; benign if raced
-    if (2 * DgradTile<MT>::STAGE > 64 * 1024 && !attr_set) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) != hipSuccess)
-            return BW_ELAUNCH;
-        attr_set = true;
-    }
+    static uint64_t big_lds_devices = 0;                   // per instantiation
+    if (2 * DgradTile<MT>::STAGE > 64 * 1024 && !bw_allow_big_lds(reinterpret_cast<const void*>(kern), big_lds_devices)) return BW_ELAUNCH;
     hipLaunchKernelGGL(kern, dim3((unsigned)(p.tiles * p.splits)), dim3(DTHREADS), 2 * DgradTile<MT>::STAGE, stream, a);
     if (hipGetLastError() != hipSuccess) return BW_ELAUNCH;
     if (p.splits > 1) {

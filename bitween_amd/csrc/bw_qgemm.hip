@@ -446,12 +446,8 @@ int launch_gemm(GemmArgs a, void* workspace, size_t workspace_bytes, hipStream_t
     using C = GemmCfg<BITS, GROUP>;
     const size_t lds = 2 * (size_t)C::STAGE_BYTES;
     auto kern = qgemm_kernel<BITS, GROUP>;
-    static bool attr_set = false;
-    if (lds > 64 * 1024 && !attr_set) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) != hipSuccess)
-            return BW_ELAUNCH;
-        attr_set = true;
-    }
+    static uint64_t big_lds_devices = 0;                   // per instantiation
+    if (lds > 64 * 1024 && !bw_allow_big_lds(reinterpret_cast<const void*>(kern), big_lds_devices)) return BW_ELAUNCH;
     const GemmPlan p = gemm_plan(a.M, a.N, a.nchunks, workspace != nullptr);
     if (p.ws_bytes > workspace_bytes) return BW_EWORKSPACE;
     a.ws = (float*)workspace;

@@ -454,13 +454,9 @@ int launch_w4_kb(const GemvArgs& a, hipStream_t stream) {
     const size_t lds = (size_t)((16 * (gcols + 1) * 4 + 15) & ~15) +
                        (size_t)nwaves * (MT * (128 / GROUP) * (KB * 256 + 16) + MT * 64);
     auto kern = qgemv_w4_kernel<GROUP, MT, KB>;
-    static bool attr_set = false;                          // per instantiation; benign if raced
+    static uint64_t big_lds_devices = 0;                   // per instantiation
     if (lds > 150 * 1024) return BW_EUNSUPPORTED;
-    if (lds > 64 * 1024 && !attr_set) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) != hipSuccess)
-            return BW_ELAUNCH;
-        attr_set = true;
-    }
+    if (lds > 64 * 1024 && !bw_allow_big_lds(reinterpret_cast<const void*>(kern), big_lds_devices)) return BW_ELAUNCH;
     hipLaunchKernelGGL(kern, dim3((unsigned)((a.N + 15) / 16)), dim3(nwaves * 64), lds, stream, a);
     return hipGetLastError() == hipSuccess ? BW_OK : BW_ELAUNCH;
 }
@@ -704,12 +700,8 @@ int launch_w2_kb(const GemvArgs& a, hipStream_t stream) {
     const size_t lds = fixed + (size_t)nwaves * (WAVE_BYTES + MT * 64);
     if (lds > (size_t)150 * 1024) return BW_EUNSUPPORTED;
     auto kern = qgemv_w2_kernel<GROUP, MT, KB>;
-    static bool attr_set = false;                          // per instantiation; benign if raced
-    if (lds > 64 * 1024 && !attr_set) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) != hipSuccess)
-            return BW_ELAUNCH;
-        attr_set = true;
-    }
+    static uint64_t big_lds_devices = 0;                   // per instantiation
+    if (lds > 64 * 1024 && !bw_allow_big_lds(reinterpret_cast<const void*>(kern), big_lds_devices)) return BW_ELAUNCH;
     hipLaunchKernelGGL(kern, dim3((unsigned)((a.N + 15) / 16)), dim3(nwaves * 64), lds, stream, a);
     return hipGetLastError() == hipSuccess ? BW_OK : BW_ELAUNCH;
 }
@@ -738,12 +730,8 @@ int launch_gemv_kb(const GemvArgs& a, hipStream_t stream) {
     const size_t lds = fixed + (size_t)nwaves * (X_BYTES + MT * 64);
     if (lds > (size_t)kLdsBudget) return BW_EUNSUPPORTED;
     auto kern = qgemv_kernel<BITS, GROUP, MT, KB>;
-    static bool attr_set = false;                          // per instantiation; benign if raced
-    if (lds > 64 * 1024 && !attr_set) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) != hipSuccess)
-            return BW_ELAUNCH;
-        attr_set = true;
-    }
+    static uint64_t big_lds_devices = 0;                   // per instantiation
+    if (lds > 64 * 1024 && !bw_allow_big_lds(reinterpret_cast<const void*>(kern), big_lds_devices)) return BW_ELAUNCH;
     hipLaunchKernelGGL(kern, dim3((unsigned)((a.N + 15) / 16)), dim3(nwaves * 64), lds, stream, a);
     return hipGetLastError() == hipSuccess ? BW_OK : BW_ELAUNCH;
 }
