@@ -23,6 +23,11 @@ How each function is pinned (see tests/test_oracle_pins.py):
   dequantize_f16              closed form RNE_f16(s16*(q-z)); product exact
   dequantize_rtn_f32          single binary32 multiply
   qlinear_forward             float64 dot of the fp16 operands, tolerance 1e-2
+  qlinear_backward            float64 product with the same W16 (the float32
+                              weight cast to float16 equals dequantize_f16:
+                              the product is exact); brute-force loops on a
+                              tiny case, one-hot rows, adjointness with the
+                              forward
 """
 import numpy as np
 

@@ -192,3 +192,34 @@ def test_error_conventions():
         orc.quantize_rtn(w, 4, 32)                   # bitween/functional.py:12-17
     with pytest.raises(AssertionError):
         orc.quantize_rtn(np.zeros((2, 96), np.float32), 3, 32)   # bitween/functional.py:6
+
+
+def test_backward_is_the_adjoint_of_the_forward_and_matches_brute_force():
+    """qlinear_backward (bitween/modules.py:108-141): grad_x[m][k] = sum_n grad_y[m][n] * W16[n][k].  Pinned by
+    plain loops over a tiny layer (an index or transposition slip fails), by one-hot rows returning rows of W16,
+    and by <grad_y, x W^T> == <grad_y W, x> in float64."""
+    rng = np.random.default_rng(12)
+    n, k, bits, g = 6, 64, 4, 32
+    w = (rng.standard_normal((n, k)) * 0.05).astype(np.float32)
+    qw, s, z, _ = orc.quantize_rtn(w, bits, g)
+    s16, z16 = orc.store_module_buffers(s, z)
+    w16 = orc.dequantize_f16(qw, s16, z16, g, bits)
+    # the float32 dequantised weight cast to float16 is the same W16 (what backward multiplies with)
+    assert np.array_equal(orc.dequantize_rtn_f32(qw, s16, z16, g, bits).astype(np.float16).view(np.uint16), w16.view(np.uint16))
+    go = rng.standard_normal((3, n)).astype(np.float16)
+    got = orc.qlinear_backward(go, qw, s16, z16, bits, g)
+    want = np.zeros((3, k))
+    for m in range(3):
+        for kk in range(k):
+            acc = 0.0
+            for nn in range(n):
+                acc += float(go[m, nn]) * float(w16[nn, kk])
+            want[m, kk] = acc
+    assert got.shape == (3, k) and np.allclose(got, want, rtol=1e-12, atol=1e-15)
+    eye = np.eye(n, dtype=np.float16)
+    assert np.array_equal(orc.qlinear_backward(eye, qw, s16, z16, bits, g), w16.astype(np.float64))
+    x = rng.standard_normal((3, k)).astype(np.float16)
+    _, y64 = orc.qlinear_forward(x, qw, s16, z16, None, bits, g)
+    lhs = (go.astype(np.float64) * y64).sum()
+    rhs = (got * x.astype(np.float64)).sum()
+    assert abs(lhs - rhs) <= 1e-9 * max(1.0, abs(lhs))
