@@ -436,7 +436,42 @@ def extras_backward(torch, hip, QuantizedLinear, layers):
     return out
 
 
-EXTRAS = {"decode": extras_decode, "decode_infinity_cache_hot": extras_decode_hot,
+def extras_opt125m_fc1(torch, hip, QuantizedLinear, layers):
+    """The one configuration that also runs on the CPU path: an OPT-125m fc1 (768 -> 3072), W4 g128, quantize + pack,
+    then the forward at M = 1 and 16 - on the GPU (graph replay, weights cache-resident at this size) and through the
+    C restatement of the reference arithmetic on this host's cores."""
+    import numpy as np
+    from oracle import c_oracle, rtn_oracle as orc
+    k, n, bits, g = 768, 3072, 4, 128
+    gen = torch.Generator(device="cuda").manual_seed(0)
+    w = (torch.randn(n, k, device="cuda", generator=gen) * 0.02).half()
+    out = {}
+    us_q = time_calls(torch, lambda: hip.quantize_pack(w, bits, g, math_dtype=torch.float32, scale_dtype=torch.float16,
+                                                      zp_dtype=torch.float16), 50, 10)
+    qw, sc, zp = hip.quantize_pack(w, bits, g, math_dtype=torch.float32, scale_dtype=torch.float16, zp_dtype=torch.float16)
+    w_np = w.float().cpu().numpy()
+    t0 = time.perf_counter()
+    for _ in range(10):
+        qw_c, s_c, z_c = c_oracle.quantize_rtn_f32(w_np, bits, g)
+    cpu_q_ms = (time.perf_counter() - t0) / 10 * 1e3
+    s16, z16 = orc.store_module_buffers(s_c, z_c)
+    out["quantize_pack"] = {"gpu_us": round(us_q, 2), "cpu_ms": round(cpu_q_ms, 3),
+                            "bit_identical": bool(np.array_equal(qw.cpu().numpy(), qw_c))}
+    for m in (1, 16):
+        x = torch.randn(m, k, device="cuda", dtype=torch.float16, generator=gen)
+        gr = graph_of(torch, lambda: [hip.quantized_matmul_hip(x, qw, sc, zp, None, bits, g) for _ in range(64)])
+        us = time_calls(torch, gr.replay, 20, 3) / 64
+        x_np = x.cpu().numpy()
+        c_oracle.qlinear_forward(x_np, qw_c, s16, z16, None, bits, g)
+        t0 = time.perf_counter()
+        for _ in range(20):
+            c_oracle.qlinear_forward(x_np, qw_c, s16, z16, None, bits, g)
+        cpu_ms = (time.perf_counter() - t0) / 20 * 1e3
+        out["forward_M%d" % m] = {"gpu_us": round(us, 2), "cpu_ms": round(cpu_ms, 3)}
+    return out
+
+
+EXTRAS = {"opt125m_fc1": extras_opt125m_fc1, "decode": extras_decode, "decode_infinity_cache_hot": extras_decode_hot,
           "decode_other_formats": extras_decode_other_formats, "hipblaslt_fp16_decode": extras_hipblaslt_decode,
           "prefill": extras_prefill, "quantize": extras_quantize, "mixed_precision_model": extras_mixed_precision_model, "eager_call": extras_eager_call,
           "decode_fused_siblings": extras_decode_fused_siblings,
