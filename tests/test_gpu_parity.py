@@ -541,3 +541,17 @@ def test_bfloat16_activations_are_rounded_to_float16_in_the_kernel(bits, g):
     q.qweight.copy_(d[0]); q.scale.copy_(d[1]); q.zero_point.copy_(d[2]); q.bias.copy_(d[3])
     xb = torch.randn(2, 3, k, device="cuda", generator=gen).to(torch.bfloat16)
     assert torch.equal(q(xb), q(xb.to(torch.float16)))
+
+
+def test_bfloat16_activations_on_a_shape_only_the_generic_kernel_takes():
+    """Group size 48 is outside the fast layouts: the C ABI answers BW_EUNSUPPORTED for bfloat16 there and the
+    Python forward casts to float16 and calls again."""
+    import bitween_amd
+    torch.manual_seed(3)
+    lin = torch.nn.Linear(96, 40, bias=True, device="cuda", dtype=torch.float16)
+    q = bitween_amd.QuantizedLinear.from_float(lin, 4, 48)
+    xb = torch.randn(5, 96, device="cuda").to(torch.bfloat16)
+    y = q(xb)
+    assert y.dtype == torch.float16 and torch.equal(y, q(xb.to(torch.float16)))
+    check_matmul(y, xb.to(torch.float16).cpu().numpy(), q.qweight.cpu().numpy(), q.scale.cpu().numpy(),
+                 q.zero_point.cpu().numpy(), q.bias.cpu().numpy(), 4, 48)
