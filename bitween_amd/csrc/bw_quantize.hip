@@ -204,43 +204,133 @@ __global__ __launch_bounds__(256) void quantize_pack_generic_kernel(const void* 
     qweight[idx] = (int32_t)word;
 }
 
-// out[n][k] = scale * (q - zp): float32 product, rounded once to the output type.
-template <int BITS, int ODT>
+// out[n][k] = scale * (q - zp): float32 product, rounded once to the output type.  A thread owns one packed word
+// (32 / BITS weights); grid.x runs along the row, grid.y over rows.  VEC: the row pitch and base of `out` allow
+// 16-byte stores (8-byte for the 8 bytes an 8-bit word becomes in a 16-bit type).
+template <int BITS, int ODT, bool VEC>
 __global__ __launch_bounds__(256) void dequantize_kernel(const uint32_t* __restrict__ qweight, const void* __restrict__ scale,
                                                          int scale_dtype, const void* __restrict__ zp, int zp_dtype,
                                                          int64_t N, int K, int group, void* __restrict__ out, int64_t ldo) {
     constexpr int VPI = 32 / BITS;
     const int words = K / VPI, groups = K / group;
-    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (idx >= N * (int64_t)words) return;
-    const int64_t row = idx / words;
-    const int wcol = (int)(idx - row * words);
-    const uint32_t w = qweight[idx];
-    float r[VPI];
-    int gprev = -1;
-    float s = 0.f, z = 0.f;
-#pragma unroll
-    for (int i = 0; i < VPI; i++) {
-        const int g = (wcol * VPI + i) / group;
-        if (g != gprev) {
+    const int wcol = (int)(blockIdx.x * blockDim.x + threadIdx.x);
+    if (wcol >= words) return;
+    for (int64_t row = blockIdx.y; row < N; row += gridDim.y) {
+        const uint32_t w = qweight[row * words + wcol];
+        float r[VPI];
+        auto load_sz = [&](int g, float& s, float& z) {
             const int64_t gi = row * groups + g;
             s = scale_dtype == BW_F32 ? ((const float*)scale)[gi] : (float)((const _Float16*)scale)[gi];
             z = zp_dtype == BW_I32 ? (float)((const int32_t*)zp)[gi] : (float)((const _Float16*)zp)[gi];
-            gprev = g;
+        };
+        const int g_first = (wcol * VPI) / group, g_last = (wcol * VPI + VPI - 1) / group;
+        float s = 0.f, z = 0.f;
+        load_sz(g_first, s, z);
+#pragma unroll
+        for (int i = 0; i < VPI; i++) {
+            if (g_first != g_last && i > 0 && (wcol * VPI + i) % group == 0) load_sz((wcol * VPI + i) / group, s, z);   // rare: groups narrower than a word
+            const float q = (float)((w >> (i * BITS)) & ((1u << BITS) - 1));
+            r[i] = __fmul_rn(s, __fsub_rn(q, z));                                  // functional.py:70, modules.py:55
+            // keep the product a value of its own: folded into a mixed-precision multiply-add with a +0 addend
+            // (what the compiler makes of multiply + narrowing conversion) 0 * -3 would lose its sign
+            asm volatile("" : "+v"(r[i]));
         }
-        const float q = (float)((w >> (i * BITS)) & ((1u << BITS) - 1));
-        r[i] = __fmul_rn(s, __fsub_rn(q, z));                                      // functional.py:70, modules.py:55
+        const int64_t o = row * ldo + (int64_t)wcol * VPI;
+        if constexpr (ODT == BW_F32) {
+            float* p = (float*)out + o;
+            if constexpr (VEC) {
+#pragma unroll
+                for (int i = 0; i < VPI; i += 4) *reinterpret_cast<f4*>(p + i) = f4{r[i], r[i + 1], r[i + 2], r[i + 3]};
+            } else {
+#pragma unroll
+                for (int i = 0; i < VPI; i++) p[i] = r[i];
+            }
+        } else {
+            uint16_t h[VPI];
+#pragma unroll
+            for (int i = 0; i < VPI; i++) h[i] = ODT == BW_F16 ? __builtin_bit_cast(uint16_t, (_Float16)r[i]) : f32_to_bf16(r[i]);
+            uint16_t* p = (uint16_t*)out + o;
+            if constexpr (VEC) {
+                uint32_t d[VPI / 2];
+#pragma unroll
+                for (int i = 0; i < VPI / 2; i++) d[i] = (uint32_t)h[2 * i] | ((uint32_t)h[2 * i + 1] << 16);
+                if constexpr (VPI == 4) {
+                    *reinterpret_cast<u2*>(p) = u2{d[0], d[1]};
+                } else {
+#pragma unroll
+                    for (int i = 0; i < VPI / 2; i += 4) *reinterpret_cast<u4*>(p + 2 * i) = u4{d[i], d[i + 1], d[i + 2], d[i + 3]};
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < VPI; i++) p[i] = h[i];
+            }
+        }
     }
-    const int64_t o = row * ldo + (int64_t)wcol * VPI;
-    if constexpr (ODT == BW_F32) {
-        float* p = (float*)out + o;
+}
+
+// The same for the usual layouts, four words per thread, 256 words apart so that every load and store instruction of
+// a wave stays contiguous.  All four words and their (scale, zero point) are requested before the first is used: with
+// one 4-byte load per thread the kernel waits a memory round trip per 16 bytes it writes.  The group is a power of
+// two and at least a word wide, so a shift finds it; scale / zero point float16 (the module buffers) or float32 /
+// int32 (what quantize_rtn returns) are told apart once per thread, not per value.
+template <int BITS, int ODT>
+__global__ __launch_bounds__(256) void dequantize_x4_kernel(const uint32_t* __restrict__ qweight, const void* __restrict__ scale,
+                                                            const void* __restrict__ zp, int module_buffers, int64_t N, int K,
+                                                            int group_shift, void* __restrict__ out, int64_t ldo) {
+    constexpr int VPI = 32 / BITS;
+    const int words = K / VPI, groups = K >> group_shift;
+    const int w0 = (int)(blockIdx.x * 1024 + threadIdx.x);
+    for (int64_t row = blockIdx.y; row < N; row += gridDim.y) {
+        uint32_t w[4];
+        float s[4], z[4];
 #pragma unroll
-        for (int i = 0; i < VPI; i++) p[i] = r[i];
-    } else {
-        uint16_t* p = (uint16_t*)out + o;
+        for (int j = 0; j < 4; j++) {
+            const int wc = w0 + 256 * j;
+            if (wc < words) {
+                w[j] = qweight[row * words + wc];
+                const int64_t gi = row * groups + ((wc * VPI) >> group_shift);
+                if (module_buffers) {
+                    s[j] = (float)((const _Float16*)scale)[gi];
+                    z[j] = (float)((const _Float16*)zp)[gi];
+                } else {
+                    s[j] = ((const float*)scale)[gi];
+                    z[j] = (float)((const int32_t*)zp)[gi];
+                }
+            }
+        }
 #pragma unroll
-        for (int i = 0; i < VPI; i++)
-            p[i] = ODT == BW_F16 ? __builtin_bit_cast(uint16_t, (_Float16)r[i]) : f32_to_bf16(r[i]);
+        for (int j = 0; j < 4; j++) {
+            const int wc = w0 + 256 * j;
+            if (wc >= words) break;
+            float r[VPI];
+#pragma unroll
+            for (int i = 0; i < VPI; i++) {
+                const float q = (float)((w[j] >> (i * BITS)) & ((1u << BITS) - 1));
+                r[i] = __fmul_rn(s[j], __fsub_rn(q, z[j]));                        // functional.py:70, modules.py:55
+                asm volatile("" : "+v"(r[i]));                                     // see dequantize_kernel
+            }
+            const int64_t o = row * ldo + (int64_t)wc * VPI;
+            if constexpr (ODT == BW_F32) {
+                float* p = (float*)out + o;
+#pragma unroll
+                for (int i = 0; i < VPI; i += 4) *reinterpret_cast<f4*>(p + i) = f4{r[i], r[i + 1], r[i + 2], r[i + 3]};
+            } else {
+                uint32_t d[VPI / 2];
+#pragma unroll
+                for (int i = 0; i < VPI / 2; i++) {
+                    const uint16_t lo = ODT == BW_F16 ? __builtin_bit_cast(uint16_t, (_Float16)r[2 * i]) : f32_to_bf16(r[2 * i]);
+                    const uint16_t hi = ODT == BW_F16 ? __builtin_bit_cast(uint16_t, (_Float16)r[2 * i + 1]) : f32_to_bf16(r[2 * i + 1]);
+                    d[i] = (uint32_t)lo | ((uint32_t)hi << 16);
+                }
+                uint16_t* p = (uint16_t*)out + o;
+                if constexpr (VPI == 4) {
+                    *reinterpret_cast<u2*>(p) = u2{d[0], d[1]};
+                } else {
+#pragma unroll
+                    for (int i = 0; i < VPI / 2; i += 4) *reinterpret_cast<u4*>(p + 2 * i) = u4{d[i], d[i + 1], d[i + 2], d[i + 3]};
+                }
+            }
+        }
     }
 }
 
@@ -335,13 +425,35 @@ extern "C" int bw_dequantize(const int32_t* qweight, const void* scale, int scal
     if (zp_dtype != BW_I32 && zp_dtype != BW_F16) return BW_EINVAL;
     if (out_dtype != BW_F32 && out_dtype != BW_F16 && out_dtype != BW_BF16) return BW_EINVAL;
     const int vpi = 32 / bits;
-    const int64_t total = N * (K / vpi);
-    dim3 grid((unsigned)((total + 255) / 256)), block(256);
+    const int64_t words = K / vpi;
+    const size_t esz = out_dtype == BW_F32 ? 4 : 2;
+    const bool vec = bw_aligned(w_out, 16) && (ldo * esz) % 16 == 0;
     hipStream_t st = (hipStream_t)stream;
+    const bool module_buffers = scale_dtype == BW_F16 && zp_dtype == BW_F16, returned = scale_dtype == BW_F32 && zp_dtype == BW_I32;
+    if (vec && (module_buffers || returned) && words >= 512 && (group & (group - 1)) == 0 && group >= vpi) {
+        int shift = 0;
+        while ((1 << shift) < group) shift++;
+        const int bsz = 256;
+        dim3 g4((unsigned)((words + 1023) / 1024), (unsigned)(N < 65535 ? N : 65535));
+#define BW_D4(B, OD)                                                                                                    \
+    if (bits == B && out_dtype == OD) {                                                                                 \
+        hipLaunchKernelGGL((dequantize_x4_kernel<B, OD>), g4, dim3(bsz), 0, st, (const uint32_t*)qweight, scale, zp,    \
+                           (int)module_buffers, N, (int)K, shift, w_out, ldo);                                          \
+        return hipGetLastError() == hipSuccess ? BW_OK : BW_ELAUNCH;                                                    \
+    }
+        BW_D4(2, BW_F32) BW_D4(4, BW_F32) BW_D4(8, BW_F32) BW_D4(2, BW_F16) BW_D4(4, BW_F16) BW_D4(8, BW_F16)
+        BW_D4(2, BW_BF16) BW_D4(4, BW_BF16) BW_D4(8, BW_BF16)
+#undef BW_D4
+    }
+    dim3 grid((unsigned)((words + 255) / 256), (unsigned)(N < 65535 ? N : 65535)), block(256);
 #define BW_D(B, OD)                                                                                                     \
     if (bits == B && out_dtype == OD) {                                                                                 \
-        hipLaunchKernelGGL((dequantize_kernel<B, OD>), grid, block, 0, st, (const uint32_t*)qweight, scale, scale_dtype, zp, \
-                           zp_dtype, N, (int)K, group, w_out, ldo);                                                     \
+        if (vec)                                                                                                        \
+            hipLaunchKernelGGL((dequantize_kernel<B, OD, true>), grid, block, 0, st, (const uint32_t*)qweight, scale,   \
+                               scale_dtype, zp, zp_dtype, N, (int)K, group, w_out, ldo);                                \
+        else                                                                                                            \
+            hipLaunchKernelGGL((dequantize_kernel<B, OD, false>), grid, block, 0, st, (const uint32_t*)qweight, scale,  \
+                               scale_dtype, zp, zp_dtype, N, (int)K, group, w_out, ldo);                                \
         return hipGetLastError() == hipSuccess ? BW_OK : BW_ELAUNCH;                                                    \
     }
     BW_D(2, BW_F32) BW_D(4, BW_F32) BW_D(8, BW_F32) BW_D(2, BW_F16) BW_D(4, BW_F16) BW_D(8, BW_F16)
