@@ -455,7 +455,7 @@ def test_error_conventions_on_gpu():
                                         (4, 64, 4096, 11008), (2, 32, 4096, 11008), (4, 128, 4096, 4096),
                                         (4, 32, 11008, 4096), (4, 64, 11008, 4096)])
 def test_full_size_properties(bits, g, k, n):
-    """BASELINE-size layers, checked through size-independent properties:
+    """Full-size layers (Llama-2-7B shapes), checked through size-independent properties:
       * a one-hot activation row returns a column of W16 bit-for-bit (the fused kernels reproduce the
         reference's dequantised weights exactly), for the decode and the prefill kernel;
       * quantise -> dequantise stays within half a step of the input for unclamped elements;
