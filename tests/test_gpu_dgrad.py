@@ -46,7 +46,7 @@ def _check(gx, go16, qw, s16, z16, bits, g):
 def test_dgrad_vs_oracle(bits, g):
     from bitween_amd.kernels import hip_loader
     lib = hip_loader.load()
-    for (n, k) in ((256, 384), (1024, 128), (96, 768)):
+    for (n, k) in ((256, 384), (1024, 128), (96, 768), (32, 128)):
         _, qw, s16, z16, _ = quantized_layer(n, k, bits, g, seed=n + k + bits + g, outliers=True, bias=False)
         d = [to_gpu(a) for a in (qw, s16, z16)]
         rng = np.random.default_rng(n * 7 + k)
