@@ -15,7 +15,7 @@
 //   * v_mfma_f32_16x16x32_f16 with A = rows of the k-major tile (8 consecutive n per lane) and B = rows of the
 //     grad_y tile: D[k][m], so a lane ends up with 4 consecutive k of one m.
 // LDS is double buffered and filled one step ahead, in the shadow of the current step's MFMAs; global loads run
-// four steps ahead; one barrier per step.
+// two steps ahead; one barrier per step.  Three workgroups share a CU and cover each other's barriers.
 // Small M * K leaves the chip idle, so N is cut into slices whose float32 partial tiles a second kernel adds up.
 #include <hip/hip_runtime.h>
 
@@ -77,10 +77,10 @@ BW_DEV constexpr int kmap(int p, int h) {
 }
 
 template <int BITS, int GROUP, int MT>
-__global__ __launch_bounds__(DTHREADS) void qdgrad_kernel(const DgradArgs a) {
+__global__ __launch_bounds__(DTHREADS, 3) void qdgrad_kernel(const DgradArgs a) {   // three workgroups per CU: <= 168 registers
     constexpr int DM = DgradTile<MT>::DM, A_BYTES = DgradTile<MT>::A_BYTES, STAGE = DgradTile<MT>::STAGE;
     constexpr int GR = DM / 128;                                      // grad_y rows a thread stages
-    constexpr int PD = 4;                                             // steps of global loads in flight
+    constexpr int PD = 2;                                             // steps of global loads in flight (even)
     extern __shared__ __attribute__((aligned(16))) char smem[];
     typedef typename WLoad<BITS>::type wload_t;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -249,9 +249,9 @@ inline int dgrad_cus() {
     return cus;
 }
 
-// Two workgroups fit a CU and hide each other's barriers.  With fewer tiles than that N is cut into slices: to two
-// workgroups per CU when a slice keeps at least 24 steps, else to one per CU with at least 8 (short slices pay
-// their prologue and the partial tiles' traffic).
+// Three workgroups fit a CU and hide each other's barriers.  With fewer tiles than two per CU N is cut into slices:
+// to two workgroups per CU (three measured slower: more partial-tile traffic) when a slice keeps at least 24 steps,
+// else to one per CU with at least 8 (short slices pay their prologue and the partial tiles' traffic).
 inline DgradPlan dgrad_plan(int64_t M, int64_t N, int64_t K, bool have_workspace) {
     DgradPlan p;
     p.mt = 4;
