@@ -26,8 +26,9 @@ namespace {
 constexpr int DK = 128, DN = 32, DTHREADS = 256;
 constexpr int DPITCH = 80;                           // bytes per LDS row: 32 halves + 16 (rows stay 16-byte aligned)
 constexpr int B_BYTES = DK * DPITCH + (DK / 16) * 16;   // k-major weight tile; every 16-row block shifted 16 bytes
-// MT = 16-row m tiles per wave (the workgroup's 2 x 2 waves cover 32 MT rows of m).  MT = 8 was measured too:
-// 128 accumulators leave one wave per SIMD and it only wins on one shape, so 4 is what is built.
+// MT = 16-row m tiles per wave (the workgroup's 2 x 2 waves cover 32 MT rows of m).  MT = 4 (161 registers, three
+// workgroups per CU) up to 512 rows of grad_y; MT = 8 (251 registers, two per CU, a quarter fewer LDS reads per MFMA)
+// beyond: 15-20 % faster there, slower below.
 template <int MT> struct DgradTile {
     static constexpr int DM = 32 * MT;
     static constexpr int A_BYTES = DM * DPITCH;      // grad_y tile
@@ -77,7 +78,7 @@ BW_DEV constexpr int kmap(int p, int h) {
 }
 
 template <int BITS, int GROUP, int MT>
-__global__ __launch_bounds__(DTHREADS, 3) void qdgrad_kernel(const DgradArgs a) {   // three workgroups per CU: <= 168 registers
+__global__ __launch_bounds__(DTHREADS, MT == 4 ? 3 : 2) void qdgrad_kernel(const DgradArgs a) {   // workgroups per CU: 3 (<= 168 registers) or 2
     constexpr int DM = DgradTile<MT>::DM, A_BYTES = DgradTile<MT>::A_BYTES, STAGE = DgradTile<MT>::STAGE;
     constexpr int GR = DM / 128;                                      // grad_y rows a thread stages
     constexpr int PD = 2;                                             // steps of global loads in flight (even)
@@ -254,7 +255,7 @@ inline int dgrad_cus() {
 // else to one per CU with at least 8 (short slices pay their prologue and the partial tiles' traffic).
 inline DgradPlan dgrad_plan(int64_t M, int64_t N, int64_t K, bool have_workspace) {
     DgradPlan p;
-    p.mt = 4;
+    p.mt = M > 512 ? 8 : 4;
     const int DM = 32 * p.mt;
     p.tiles_k = (int)(K / DK);
     p.tiles = p.tiles_k * (int)((M + DM - 1) / DM);
@@ -308,7 +309,7 @@ int launch_dgrad(DgradArgs a, void* workspace, size_t workspace_bytes, hipStream
     a.tiles_k = p.tiles_k;
     a.splits = p.splits;
     a.steps_per_split = p.steps_per_split;
-    return launch_dgrad_mt<BITS, GROUP, 4>(a, p, stream);
+    return p.mt == 8 ? launch_dgrad_mt<BITS, GROUP, 8>(a, p, stream) : launch_dgrad_mt<BITS, GROUP, 4>(a, p, stream);
 }
 
 }  // namespace

@@ -50,7 +50,7 @@ def test_dgrad_vs_oracle(bits, g):
         _, qw, s16, z16, _ = quantized_layer(n, k, bits, g, seed=n + k + bits + g, outliers=True, bias=False)
         d = [to_gpu(a) for a in (qw, s16, z16)]
         rng = np.random.default_rng(n * 7 + k)
-        for m in (1, 17, 128, 200):
+        for m in (1, 17, 128, 200, 513):
             go16 = rng.standard_normal((m, n)).astype(np.float16)
             for use_ws in (True, False):
                 st, gx, need = _call(lib, to_gpu(go16), d, m, n, k, bits, g, use_ws)
@@ -78,7 +78,7 @@ def test_dgrad_full_size_one_hot_rows_and_split(bits, g, n, k):
     assert st == 0 and need > 0, "small M on a full-size layer is meant to split"
     for i, r in enumerate(rows):
         assert torch.equal(gx[i], w16[r])
-    for m in (64, 300):
+    for m in (64, 300, 700):                                  # 700: the 256-row tile variant, last tile ragged
         go = torch.randn(m, n, device="cuda", dtype=torch.float16, generator=gen)
         st, gx, _ = _call(lib, go, d, m, n, k, bits, g)
         assert st == 0
