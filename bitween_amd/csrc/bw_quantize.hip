@@ -79,11 +79,11 @@ BW_DEV float quant_exact(float w, float s, float zf) {
 // the shape allows); the lpg = group / VPT threads of a group (a power of two <= 64, aligned inside the
 // wave) agree on min and max with cross-lane shuffles.
 //
-// float32 math takes a short cut that cannot change a result: q1 = fma(w - q0 s, r, q0) with q0 = w r and
-// r = 1/s refined once is within one ulp of the correctly rounded w / s, and for |q1| < 1024 the sum
-// t = q1 + zf is then within 2^-12 of what the exact quotient gives.  Unless t lies within 2^-11 of a
-// half-integer, round(t) is therefore the reference's value; the rare elements that do (and anything
-// large, infinite or NaN) are redone with the true IEEE divide.
+// float32 math takes a short cut that cannot change a result: with r = 1/s refined once (relative error
+// <= 2^-23) t = fma(w, r, zf) differs from the reference's fl(fl(w / s) + zf) by less than 3.5e-4 as long as
+// |w / s| < 1024 (1024 * 2^-23 for r, plus the roundings of the quotient and of the two sums near 1300).  Unless t
+// lies within 2^-11 = 4.9e-4 of a half-integer, round(t) is therefore the reference's value; beyond 1024 both clamp
+// to the same end of the range.  Values near a tie (and infinities, NaN) are redone with the true IEEE divide.
 template <int BITS, int WDT, int MATH, int WPT>
 __global__ __launch_bounds__(256) void quantize_pack_kernel(const void* __restrict__ w, const void* __restrict__ delta,
                                                             int64_t N, int K, int64_t ldw, int64_t ldd,
@@ -123,11 +123,10 @@ __global__ __launch_bounds__(256) void quantize_pack_kernel(const void* __restri
             const float r = __builtin_fmaf(__builtin_fmaf(-s, r0, 1.0f), r0, r0);
 #pragma unroll
             for (int i = 0; i < VPT; i++) {
-                const float q0 = __fmul_rn(v[i], r);
-                const float q1 = __builtin_fmaf(__builtin_fmaf(-q0, s, v[i]), r, q0);
-                const float sum = __fadd_rn(q1, zf);
+                const float sum = __builtin_fmaf(v[i], r, zf);
                 t[i] = rintf(sum);
-                // far from a tie (a huge |q1| has no fraction and clamps the same either way; NaN fails the test)
+                // far from a tie (a huge |sum| has no fraction and clamps the same either way; NaN fails the test)?
+                // else redo with the true divide: one value in a thousand, so a wave rarely enters any one of these
                 if (!(fabsf(__fsub_rn(sum, t[i])) < 0.5f - 0x1p-11f)) t[i] = quant_exact<MATH>(v[i], s, zf);
             }
         } else {
@@ -142,7 +141,7 @@ __global__ __launch_bounds__(256) void quantize_pack_kernel(const void* __restri
             float half[2] = {0.f, 0.f};
 #pragma unroll
             for (int i = 0; i < VPI; i++)
-                half[i / FPH] = __builtin_fmaf(fminf(fmaxf(t[j * VPI + i], 0.f), QMAX), (float)(1 << ((i % FPH) * BITS)), half[i / FPH]);
+                half[i / FPH] = __builtin_fmaf(__builtin_amdgcn_fmed3f(t[j * VPI + i], 0.f, QMAX), (float)(1 << ((i % FPH) * BITS)), half[i / FPH]);
             word[j] = (uint32_t)half[0] | ((uint32_t)half[1] << 16);
         }
         if (live) {
