@@ -135,3 +135,35 @@ def test_module_backward_uses_fused_kernel_and_falls_back():
         got = x.grad.reshape(21, k).double().cpu().numpy()
         assert x.grad.dtype == torch.float16
         assert np.abs(got - ref).max() <= 1e-2 * np.abs(ref).max()
+
+
+def _sweep():
+    rng = np.random.default_rng(77)
+    out = []
+    for i in range(24):
+        bits = int(rng.choice([2, 4, 8]))
+        g = int(rng.choice([32, 64, 128]))
+        k = 128 * int(rng.integers(1, 7))
+        n = 32 * int(rng.integers(1, 13))
+        m = int(rng.choice([1, 2, 15, 16, 33, 127, 128, 129, 255, 300, 513, 600]))
+        pad = int(rng.choice([0, 8, 40]))
+        out.append((i, bits, g, k, n, m, pad))
+    return out
+
+
+@pytest.mark.parametrize("case", _sweep(), ids=lambda c: "b%d_g%d_K%d_N%d_M%d_pad%d" % c[1:])
+def test_dgrad_seeded_sweep(case):
+    """Random supported shapes (K % 128 == 0, N % 32 == 0), both tile variants, ragged last m tile, padded grad_y
+    rows, sliced and unsliced reduction."""
+    from bitween_amd.kernels import hip_loader
+    lib = hip_loader.load()
+    i, bits, g, k, n, m, pad = case
+    _, qw, s16, z16, _ = quantized_layer(n, k, bits, g, seed=500 + i, outliers=True, bias=False)
+    d = [to_gpu(a) for a in (qw, s16, z16)]
+    go16 = np.random.default_rng(i).standard_normal((m, n)).astype(np.float16)
+    buf = torch.full((m, n + pad), float("nan"), dtype=torch.float16, device="cuda")
+    buf[:, :n] = to_gpu(go16)
+    for use_ws in (True, False):
+        st, gx, _ = _call(lib, buf, d, m, n, k, bits, g, use_ws, ldg=n + pad)
+        assert st == 0
+        _check(gx, go16, qw, s16, z16, bits, g)
