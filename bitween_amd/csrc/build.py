@@ -20,9 +20,7 @@ FLAGS = [
 ]
 
 
-def build(verbose=False):
-    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
-    cmd = [hipcc] + FLAGS + ["-o", LIB] + [os.path.join(HERE, s) for s in SOURCES]
+def _run(cmd, verbose):
     if verbose:
         print(" ".join(cmd))
     proc = subprocess.run(cmd, capture_output=True, text=True)
@@ -32,6 +30,20 @@ def build(verbose=False):
         raise RuntimeError(f"hipcc failed ({proc.returncode}):\n{err}")
     if verbose and err.strip():
         print(err, file=sys.stderr)
+
+
+def build(verbose=False):
+    """Compile every source to an object file (in parallel, one hipcc per file), then link the shared library."""
+    from concurrent.futures import ThreadPoolExecutor
+    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+    objdir = os.path.join(HERE, "build")
+    os.makedirs(objdir, exist_ok=True)
+    compile_flags = [f for f in FLAGS if f != "-shared"] + ["-c"]
+    objs = [os.path.join(objdir, s.replace(".hip", ".o")) for s in SOURCES]
+    jobs = [[hipcc] + compile_flags + ["-o", o, os.path.join(HERE, s)] for s, o in zip(SOURCES, objs)]
+    with ThreadPoolExecutor(max_workers=min(len(jobs), os.cpu_count() or 1)) as pool:
+        list(pool.map(lambda cmd: _run(cmd, verbose), jobs))
+    _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs, verbose)
     return LIB
 
 
