@@ -52,6 +52,10 @@ class QuantizedLinearFunction(torch.autograd.Function):
         return grad_input, None, None, None, None, None, None
 
 
+class BitweenShapeError(RuntimeError):
+    pass
+
+
 class QuantizedLinear(nn.Module):
     """Linear layer holding 2/4/8-bit group-quantised weights."""
 
@@ -114,14 +118,19 @@ class QuantizedLinear(nn.Module):
             weight = weight.to("cuda")
         qweight, scale, zero_point = _hip.quantize_pack(weight, bits, group_size, math_dtype=torch.float32,
                                                         scale_dtype=torch.float16, zp_dtype=torch.float16)
-        q_layer = cls(float_layer.in_features, float_layer.out_features, bits, group_size,
-                      bias=float_layer.bias is not None, dtype=torch.float16)
-        q_layer = q_layer.to(device)
-        q_layer.qweight.copy_(qweight)
-        q_layer.scale.copy_(scale)
-        q_layer.zero_point.copy_(zero_point)
+        # the constructor's zero buffers are built on the meta device (no memory, no host-to-device copy) and
+        # replaced by the kernel's outputs, which already have the buffers' shapes and dtypes
+        with torch.device("meta"):
+            q_layer = cls(float_layer.in_features, float_layer.out_features, bits, group_size,
+                          bias=float_layer.bias is not None, dtype=torch.float16)
+        new = {"qweight": qweight, "scale": scale, "zero_point": zero_point}
         if float_layer.bias is not None:
-            q_layer.bias.data.copy_(float_layer.bias.data)
+            new["bias"] = float_layer.bias.data.to(device="cuda", dtype=torch.float16, copy=True)
+        for name, value in new.items():
+            if value.shape != q_layer._buffers[name].shape or value.dtype != q_layer._buffers[name].dtype:
+                raise BitweenShapeError(f"{name}: kernel produced {tuple(value.shape)} {value.dtype}, the module "
+                                        f"declares {tuple(q_layer._buffers[name].shape)} {q_layer._buffers[name].dtype}")
+            q_layer._buffers[name] = value if device.type == "cuda" else value.to(device)
         return q_layer
 
     def __repr__(self):

@@ -84,8 +84,11 @@ class Bitween:
         if batch_size is not None:
             self.batch_size = batch_size
         try:
-            quantized_model = copy.deepcopy(self.model)
-            targets = [(name, module) for name, module in quantized_model.named_modules() if isinstance(module, nn.Linear)]
+            # The reference deep-copies the model and then replaces the copies of the linear layers
+            # (quantizer.py:69-80).  Same result without ever copying the weights that are about to be replaced:
+            # quantise from the original layers and hand deepcopy the replacements through its memo.
+            memo = {}
+            targets = [(name, module) for name, module in self.model.named_modules() if isinstance(module, nn.Linear)]
             for name, module in targets:
                 if name in self.ignore_layers:
                     if verbose:
@@ -94,7 +97,8 @@ class Bitween:
                 if verbose:
                     print(f"  - Quantizing layer: {name}")
                 bits, group_size = _precision_for(name, layer_config or {}, (self.bits, self.group_size))
-                _set_module(quantized_model, name, QuantizedLinear.from_float(module, bits, group_size))
+                memo[id(module)] = QuantizedLinear.from_float(module, bits, group_size)
+            quantized_model = copy.deepcopy(self.model, memo)
             if fuse_siblings:
                 fuse_sibling_linears(quantized_model)
             if verbose:
