@@ -226,6 +226,54 @@ def _matmul(entry, x, qweight, scale, zero_point, bias, bits, group_size):
     return y
 
 
+def make_decode_plan(qweight, scale, zero_point, bias, bits, group_size):
+    """Validate a layer's buffers once for decode_with_plan: returns a tuple holding the tensors (so that the
+    caller can tell by identity whether they are still the ones validated), their device addresses and the
+    layer's sizes - or None when the buffers do not qualify and the general path has to look at them."""
+    if not qweight.is_cuda or qweight.dtype is not torch.int32 or scale.dtype is not torch.float16 or \
+            zero_point.dtype is not torch.float16 or (bias is not None and bias.dtype is not torch.float16):
+        return None
+    if not (qweight.is_contiguous() and scale.is_contiguous() and zero_point.is_contiguous()) or \
+            (bias is not None and not bias.is_contiguous()):
+        return None
+    n, words = qweight.shape
+    k = words * (32 // bits)
+    if k % group_size or scale.shape != (n, k // group_size) or zero_point.shape != scale.shape or \
+            (bias is not None and bias.shape != (n,)):
+        return None
+    load()
+    index = qweight.device.index if qweight.device.index is not None else torch.cuda.current_device()
+    return (qweight, scale, zero_point, bias, qweight.data_ptr(), scale.data_ptr(), zero_point.data_ptr(),
+            None if bias is None else bias.data_ptr(), n, k, bits, group_size, index)
+
+
+def decode_with_plan(plan, x, m):
+    """bw_qlinear for up to 48 rows with buffers validated by make_decode_plan: only x is looked at.  Returns None
+    when x does not qualify (layout, device, dtype) - the caller then takes quantized_matmul_hip."""
+    dt = x.dtype
+    if dt is torch.float16:
+        act = BW_F16
+    elif dt is torch.bfloat16:
+        act = BW_BF16
+    else:
+        return None
+    ldx = x.stride(0)
+    xp = x.data_ptr()
+    index = plan[12]
+    if not x.is_cuda or x.stride(1) != 1 or (ldx * 2) % 16 or xp % 16 or x.shape[1] != plan[9] or \
+            torch.cuda.current_device() != index:
+        return None
+    n = plan[8]
+    y = torch.empty((m, n), dtype=torch.float16, device=x.device)
+    st = _ENTRY["bw_qlinear"](xp, act, m, plan[9], ldx, plan[4], plan[5], plan[6], plan[7], n, plan[10], plan[11],
+                              y.data_ptr(), n, _raw_stream(index))
+    if st:
+        if st == -2:
+            return None
+        _check(st, "bw_qlinear")
+    return y
+
+
 def quantized_input_grad(grad_y, qweight, scale, zero_point, bits, group_size):
     """grad_x[M,K] = grad_y[M,N] @ W16[N,K] with the dequantisation fused in (bw_qdgrad); None when the library
     has no fused kernel for this shape / dtype - the caller then dequantises and calls the library GEMM."""

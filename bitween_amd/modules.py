@@ -93,10 +93,30 @@ class QuantizedLinear(nn.Module):
         # nothing to differentiate (the buffers never require grad): same arithmetic without the autograd node
         shape = x.shape
         x2 = x.reshape(-1, shape[-1])
+        m = x2.shape[0]
+        if 0 < m <= 48:
+            # decode: the buffers were validated once; they are looked at again only when one of them has been
+            # replaced (module.to(), load with assign, sibling fusion) or moved
+            plan = self.__dict__.get("_decode_plan")
+            b = self._buffers
+            if plan is None or plan[0] is not b["qweight"] or plan[1] is not b["scale"] or \
+                    plan[2] is not b["zero_point"] or plan[3] is not b.get("bias") or plan[4] != plan[0].data_ptr():
+                plan = _hip.make_decode_plan(b["qweight"], b["scale"], b["zero_point"], b.get("bias"), self.bits,
+                                             self.group_size) if b["qweight"].is_cuda else None
+                self.__dict__["_decode_plan"] = plan
+            if plan is not None:
+                y = _hip.decode_with_plan(plan, x2, m)
+                if y is not None:
+                    return y.view(*shape[:-1], self.out_features)
         if x2.dtype is not torch.float16 and x2.dtype is not torch.bfloat16:    # bfloat16 is converted by the kernel
             x2 = x2.to(torch.float16)
         y = _hip.quantized_matmul_hip(x2, self.qweight, self.scale, self.zero_point, self.bias, self.bits, self.group_size)
         return y.view(*shape[:-1], self.out_features)
+
+    def __getstate__(self):                                # the validated-buffers cache holds device addresses
+        state = self.__dict__.copy()
+        state.pop("_decode_plan", None)
+        return state
 
     @classmethod
     def from_float(cls, float_layer: nn.Linear, bits=8, group_size=32):

@@ -555,3 +555,47 @@ def test_bfloat16_activations_on_a_shape_only_the_generic_kernel_takes():
     assert y.dtype == torch.float16 and torch.equal(y, q(xb.to(torch.float16)))
     check_matmul(y, xb.to(torch.float16).cpu().numpy(), q.qweight.cpu().numpy(), q.scale.cpu().numpy(),
                  q.zero_point.cpu().numpy(), q.bias.cpu().numpy(), 4, 48)
+
+
+def test_validated_buffer_cache_follows_replaced_buffers():
+    """The decode path validates a layer's buffers once and afterwards only checks that they are still the same
+    tensors at the same address.  Every way of changing them must be seen: in-place load, a replaced buffer, a
+    deep copy, a pickle round trip, a move off the GPU and back."""
+    import copy
+    import io
+    import bitween_amd
+    torch.manual_seed(11)
+    k, n = 256, 96
+    lin_a = torch.nn.Linear(k, n, bias=True, device="cuda", dtype=torch.float16)
+    lin_b = torch.nn.Linear(k, n, bias=True, device="cuda", dtype=torch.float16)
+    qa = bitween_amd.QuantizedLinear.from_float(lin_a, 4, 64)
+    qb = bitween_amd.QuantizedLinear.from_float(lin_b, 4, 64)
+    x = torch.randn(3, k, device="cuda", dtype=torch.float16)
+    hip = _hip()
+
+    def direct(q):
+        return hip.quantized_matmul_hip(x, q.qweight, q.scale, q.zero_point, q.bias, q.bits, q.group_size)
+
+    ya, yb = direct(qa), direct(qb)
+    assert not torch.equal(ya, yb)
+    assert torch.equal(qa(x), ya) and "_decode_plan" in qa.__dict__
+    qa.load_state_dict(qb.state_dict())                       # in place: same tensors, new contents
+    assert torch.equal(qa(x), yb)
+    qa.qweight = qa.qweight.clone()                           # a replaced buffer
+    qa.scale = torch.zeros_like(qa.scale)
+    assert torch.equal(qa(x), direct(qa)) and (qa(x) == qa.bias).all()
+    qc = copy.deepcopy(qb)
+    assert "_decode_plan" not in qc.__dict__ and torch.equal(qc(x), yb)
+    buf = io.BytesIO()
+    torch.save(qb, buf)
+    buf.seek(0)
+    qd = torch.load(buf, weights_only=False)                  # our own file
+    assert torch.equal(qd(x), yb)
+    qe = qb.to("cpu").to("cuda")                              # new tensors at new addresses
+    assert torch.equal(qe(x), yb)
+    lin_c = torch.nn.Linear(k, n, bias=False, device="cuda", dtype=torch.float16)
+    qf = bitween_amd.QuantizedLinear.from_float(lin_c, 8, 32)
+    assert torch.equal(qf(x), direct(qf))
+    assert torch.equal(qf(x.to(torch.bfloat16)), qf(x.to(torch.bfloat16).to(torch.float16)))
+    xs = torch.randn(3, 2 * k, device="cuda", dtype=torch.float16)[:, ::2]     # strided x falls back to the general path
+    assert torch.equal(qf(xs), qf(xs.contiguous()))
