@@ -6,16 +6,18 @@
 // casts to grad_output's dtype and calls matmul; for float16 gradients that cast gives exactly W16.)
 //
 // The reduction runs over N, the dimension the packed words do NOT run along, so a weight tile has to be
-// transposed on its way to the matrix core.  A workgroup owns a 128 (m) x 128 (k) tile of grad_x and walks N
-// in steps of 32 rows:
-//   * 256 threads each take 16 consecutive k of one row n (one group: groups are >= 32 wide), dequantise them to
-//     the reference's W16 (magic-number unpack, exact q - z, one multiply by the scale) and scatter the 16
-//     halves into an LDS tile stored k-major (row k holds the 32 n of the step) - that is the transposition;
-//   * the 128 x 32 slice of grad_y goes to a second LDS tile as it is;
+// transposed on its way to the matrix core.  A workgroup owns a 128 or 256 (m) x 128 (k) tile of grad_x and walks
+// N in steps of 32 rows:
+//   * 256 threads each take 16 consecutive k of one row n (one group: groups are >= 32 wide) and dequantise them to
+//     the reference's W16 (magic-number unpack, exact q - z, one multiply by the scale); the lanes of rows n and
+//     n + 1 swap half of their values and write dwords (n, n + 1) into an LDS tile stored k-major (row k holds the
+//     32 n of the step) - that is the transposition;
+//   * the 128 / 256 x 32 slice of grad_y goes to a second LDS tile as it is;
 //   * v_mfma_f32_16x16x32_f16 with A = rows of the k-major tile (8 consecutive n per lane) and B = rows of the
 //     grad_y tile: D[k][m], so a lane ends up with 4 consecutive k of one m.
 // LDS is double buffered and filled one step ahead, in the shadow of the current step's MFMAs; global loads run
-// two steps ahead; one barrier per step.  Three workgroups share a CU and cover each other's barriers.
+// two steps ahead; one barrier per step.  Three (two with the 256-row tile) workgroups share a CU and cover each
+// other's barriers.
 // Small M * K leaves the chip idle, so N is cut into slices whose float32 partial tiles a second kernel adds up.
 #include <hip/hip_runtime.h>
 
