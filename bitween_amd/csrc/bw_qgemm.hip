@@ -24,9 +24,16 @@ constexpr int WAVES = 4, NT = 4, MT = 8, BM = MT * 16, BN = WAVES * NT * 16;
 
 template <int BITS, int GROUP>
 struct GemmCfg {
-    static constexpr int VPI = 32 / BITS, VPL = 128 / BITS, CHUNK_K = 4 * VPL, MF = VPL / 8;
-    static constexpr int NG = (VPL > GROUP) ? VPL / GROUP : 1;
-    static constexpr int WPG = (GROUP >= VPL) ? 4 : 4 / NG;      // words of a lane load per group
+    // A lane takes WL adjacent 16-byte loads of a weight row per K step: VPL consecutive values.  Two loads
+    // at 8 bits, so that every format runs 4 or 8 MFMA steps per K step (the per-step costs - barrier,
+    // first fragments, scale and zero-point requests - are spread equally thin) and a lane's values never
+    // span more than one group of 32.
+    static constexpr int WL = BITS == 8 ? 2 : 1;
+    static constexpr int VPI = 32 / BITS, VPL = WL * 128 / BITS, CHUNK_K = 4 * VPL, MF = VPL / 8;
+    static constexpr int SPL = MF / WL;                          // MFMA steps per lane load
+    static constexpr int CHUNK_BYTES = 64 * WL;                  // of a packed weight row
+    static constexpr int NG = (VPL > GROUP) ? VPL / GROUP : 1;   // groups inside a lane's values
+    static constexpr int WPG = 4 * WL / NG;                      // words of a lane's values per group
     static constexpr int PITCH = CHUNK_K + 8;                    // halves per LDS row
     static constexpr int STAGE_BYTES = BM * PITCH * 2;
     static constexpr int UNIT = VPI > 8 ? VPI : 8;               // halves permuted together when staging x
@@ -130,7 +137,7 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
 #pragma unroll
     for (int j = 0; j < NT; j++) {
         const int row = n0 + 16 * j + nl;
-        w_off[j] = row < a.N ? (uint32_t)row * a.row_bytes + kq * 16 : kOob;
+        w_off[j] = row < a.N ? (uint32_t)row * a.row_bytes + kq * 16 * C::WL : kOob;
         m_off[j] = (uint32_t)min(row, a.N - 1) * groups * 2;
     }
     uint32_t x_off[C::XL];
@@ -143,7 +150,7 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
     u4 xr[C::XL * C::UW];
     // Two weight register sets, used alternately by even and odd K steps and never copied: a register move
     // of an outstanding load would stall on it.
-    struct WSet { u4 w[NT]; uint32_t s[NT][C::NG], z[NT][C::NG]; };   // 16-bit values, one register each
+    struct WSet { u4 w[NT][C::WL]; uint32_t s[NT][C::NG], z[NT][C::NG]; };   // 16-bit values, one register each
     WSet set0, set1;
 
     f4 acc[MT][NT];
@@ -170,9 +177,10 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
 #pragma unroll
         for (int j = 0; j < C::UW; j++) xr[i * C::UW + j] = __builtin_amdgcn_raw_buffer_load_b128(rx, off + j * 16, 0, 0);
     };
-    auto issue_w_tile = [&](int j, int c, WSet& ws) {
-        const bool in = c < c_end && c * 64 + kq * 16 < a.row_bytes;
-        ws.w[j] = __builtin_amdgcn_raw_buffer_load_b128(rw, in ? w_off[j] + c * 64 : kOob, 0, 0);
+    auto issue_w_load = [&](int j, int l, int c, WSet& ws) {
+        const int b = c * C::CHUNK_BYTES + l * 16;
+        const bool in = c < c_end && b + kq * 16 * C::WL < a.row_bytes;
+        ws.w[j][l] = __builtin_amdgcn_raw_buffer_load_b128(rw, in ? w_off[j] + b : kOob, 0, 0);
     };
     auto issue_meta = [&](int j, int which, int c, WSet& ws) {   // which: 0 = scales, 1 = zero points
         const int g0 = min((c * C::CHUNK_K + kq * C::VPL) / GROUP, groups - C::NG);
@@ -182,13 +190,16 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
             else ws.z[j][g] = __builtin_amdgcn_raw_buffer_load_b16(rz, m_off[j] + (g0 + g) * 2, 0, 0);
         }
     };
+    // Weight fragment of MFMA step t: values [8 t, 8 t + 8) of the lane's VPL, from lane load t / SPL.
+    auto unpack = [&](const WSet& ws, int j, int t, const GroupConst<BITS>* gcj) {
+        static_assert(C::WL == 1 || C::NG == 1, "two lane loads share one group");
+        return unpack_step<BITS>(ws.w[j][t / C::SPL], t % C::SPL, gcj, C::WPG);
+    };
 
     // One K step.  The 32 MFMAs of MFMA step t are issued in groups of 4 (one m-tile); between two groups
-    // sits one slice of other work, fenced so the compiler keeps it there:
-    //   t < last : the LDS read of one activation fragment and (every other slot) the unpack of one weight
-    //              fragment of step t+1;
-    //   t = last : one unit of the next chunk's activations (permute, LDS write, re-request for chunk c+2)
-    //              and (every other slot) the re-request of one weight tile for chunk c+2.
+    // sits one slice of other work, fenced so the compiler keeps it there: for t < last the LDS read of one
+    // activation fragment and (every other slot) the unpack of one weight fragment of step t+1, and in
+    // every step the staging and global requests listed at slot_requests below.
     // Requests past the last chunk are range-checked to zero by the hardware; no branches, so every wait
     // count is exact.
     auto step = [&](int c, const _Float16* cur, _Float16* nxt, WSet& ws) {
@@ -206,7 +217,7 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
         for (int i = 0; i < MT; i++) xf[0][i] = *reinterpret_cast<const h8*>(xp + i * 16 * C::PITCH);
 #pragma unroll
         for (int j = 0; j < NT; j++) {
-            const h8 f = unpack_step<BITS>(ws.w[j], 0, gc[j], C::WPG);
+            const h8 f = unpack(ws, j, 0, gc[j]);
 #pragma unroll
             for (int e = 0; e < 4; e++) wf[0][j][e] = h2{f[2 * e], f[2 * e + 1]};
         }
@@ -217,17 +228,13 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
         //                     step's constants are formed)
         //   last MFMA step  : weights for chunk c+2 (their registers are free after the last unpack)
         auto slot_requests = [&](int t, int i) {
-            constexpr int T_META = C::MF > 2 ? 1 : C::MF - 1;
+            static_assert(C::MF >= 4, "first, middle and last MFMA step are distinct");
             if (t == 0 && i < C::XL) {
                 stage_unit(i, nxt);
                 issue_x_unit(i, c + 2);
             }
-            if (t == T_META && (C::MF > 2 || (i & 1))) {
-                const int q = C::MF > 2 ? i : i / 2;              // 0 .. 2*NT-1 when MF > 2, else 0 .. NT-1
-                if (C::MF > 2) issue_meta(q / 2, q & 1, c + 2, ws);
-                else { issue_meta(q, 0, c + 2, ws); issue_meta(q, 1, c + 2, ws); }
-            }
-            if (t == C::MF - 1 && !(i & 1)) issue_w_tile(i / 2, c + 2, ws);
+            if (t == 1) issue_meta(i / 2, i & 1, c + 2, ws);
+            if (t == C::MF - 1 && (C::WL == 2 || !(i & 1))) issue_w_load(i / 2, C::WL == 2 ? (i & 1) : 0, c + 2, ws);
             asm volatile("" ::: "memory");
         };
 #pragma unroll
@@ -252,7 +259,7 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
                         if (t + 1 < C::MF) {
                             if (j == 0) {
                                 xf[nx][i] = *reinterpret_cast<const h8*>(xp + i * 16 * C::PITCH + 8 * (t + 1));
-                                wsrc = (i & 1) ? ws.w[jn][t + 1] >> 8 : ws.w[jn][t + 1];
+                                wsrc = (i & 1) ? ws.w[jn][0][t + 1] >> 8 : ws.w[jn][0][t + 1];
                                 pa = as_h2(and_or(wsrc, 0x000F000Fu, kMagic));
                             } else if (j == 1) {
                                 pb = as_h2(and_or(wsrc, 0x00F000F0u, kMagic));
@@ -277,7 +284,7 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
                     if (t + 1 < C::MF) {
                         xf[nx][i] = *reinterpret_cast<const h8*>(xp + i * 16 * C::PITCH + 8 * (t + 1));
                         if (i & 1) {
-                            const h8 f = unpack_step<BITS>(ws.w[i / 2], t + 1, gc[i / 2], C::WPG);
+                            const h8 f = unpack(ws, i / 2, t + 1, gc[i / 2]);
 #pragma unroll
                             for (int e = 0; e < 4; e++) wf[nx][i / 2][e] = h2{f[2 * e], f[2 * e + 1]};
                         }
@@ -310,11 +317,13 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
             __builtin_amdgcn_sched_barrier(0);
         }
 #pragma unroll
-        for (int j = 0; j < NT; j++) {
-            issue_w_tile(j, c, ws);
-            asm volatile("" ::: "memory");
-            __builtin_amdgcn_sched_barrier(0);
-        }
+        for (int j = 0; j < NT; j++)
+#pragma unroll
+            for (int l = 0; l < C::WL; l++) {
+                issue_w_load(j, l, c, ws);
+                asm volatile("" ::: "memory");
+                __builtin_amdgcn_sched_barrier(0);
+            }
     };
     issue_batch(c_begin, set0);
 #pragma unroll
@@ -414,6 +423,11 @@ inline int device_cus() {
     return cus;
 }
 
+inline int gemm_chunks(int64_t K, int bits) {   // K steps of a whole row: GemmCfg::CHUNK_BYTES each
+    const int64_t chunk = bits == 8 ? 128 : 64;
+    return (int)((K * bits / 8 + chunk - 1) / chunk);
+}
+
 inline GemmPlan gemm_plan(int64_t M, int64_t N, int nchunks, bool have_workspace) {
     GemmPlan p;
     p.tiles_n = (int)((N + BN - 1) / BN);
@@ -444,6 +458,7 @@ inline GemmPlan gemm_plan(int64_t M, int64_t N, int nchunks, bool have_workspace
 template <int BITS, int GROUP>
 int launch_gemm(GemmArgs a, void* workspace, size_t workspace_bytes, hipStream_t stream) {
     using C = GemmCfg<BITS, GROUP>;
+    static_assert(C::CHUNK_BYTES == (BITS == 8 ? 128 : 64), "gemm_chunks() counts K steps of this size");
     const size_t lds = 2 * (size_t)C::STAGE_BYTES;
     auto kern = qgemm_kernel<BITS, GROUP>;
     static uint64_t big_lds_devices = 0;                   // per instantiation
@@ -507,7 +522,7 @@ int bw_qgemm_generic(const void* x, int act_dtype, int64_t M, int64_t K, int64_t
 
 extern "C" size_t bw_qgemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int bits, int group) {
     if (!bw_shape_ok(N, K, bits, group) || M < 1 || M >= ((int64_t)1 << 31) || !bw_fast_shape(M, N, K, K, bits, group)) return 0;
-    return gemm_plan(M, N, (int)((K * bits / 8 + 63) / 64), true).ws_bytes;
+    return gemm_plan(M, N, gemm_chunks(K, bits), true).ws_bytes;
 }
 
 extern "C" int bw_qgemm_ws(const void* x, int act_dtype, int64_t M, int64_t K, int64_t ldx, const int32_t* qweight,
@@ -525,7 +540,7 @@ extern "C" int bw_qgemm_ws(const void* x, int act_dtype, int64_t M, int64_t K, i
     a.M = (int)M; a.N = (int)N; a.K = (int)K; a.ldx = (int)ldx; a.ldy = (int)ldy;
     a.groups = (int)(K / group);
     a.row_bytes = (int)(K * bits / 8);
-    a.nchunks = (a.row_bytes + 63) / 64;
+    a.nchunks = gemm_chunks(K, bits);
     a.x_bytes = (uint32_t)(((M - 1) * ldx + K) * 2);
     a.w_bytes = (uint32_t)(N * a.row_bytes);
     a.meta_bytes = (uint32_t)(N * a.groups * 2);
