@@ -34,6 +34,10 @@ struct GemmCfg {
     static constexpr int CHUNK_BYTES = 64 * WL;                  // of a packed weight row
     static constexpr int NG = (VPL > GROUP) ? VPL / GROUP : 1;   // groups inside a lane's values
     static constexpr int WPG = 4 * WL / NG;                      // words of a lane's values per group
+    // One K step = one group: the scales (zero points) of four consecutive steps are 8 adjacent bytes and can
+    // come in one request per tile instead of four (kernel parameter META4; needs rows of scales that
+    // start on 4-byte boundaries, i.e. an even number of groups).
+    static constexpr bool CAN_META4 = CHUNK_K == GROUP;
     static constexpr int PITCH = CHUNK_K + 8;                    // halves per LDS row
     static constexpr int STAGE_BYTES = BM * PITCH * 2;
     static constexpr int UNIT = VPI > 8 ? VPI : 8;               // halves permuted together when staging x
@@ -113,7 +117,7 @@ BW_DEV __amdgpu_buffer_rsrc_t make_rsrc(const void* p, uint32_t bytes) {
 //   the activations of step c+1 were requested one step earlier and are written to buffer (c+1)&1 after the
 //   MFMAs of step c; the weights of step c+1 likewise sit in `wn` and are moved to `wr`;
 //   then the loads of step c+2 are issued.  Every global load has a full K step (~2000 MFMA cycles) to land.
-template <int BITS, int GROUP>
+template <int BITS, int GROUP, bool META4>
 __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
     using C = GemmCfg<BITS, GROUP>;
     constexpr uint32_t kOob = 0x80000000u;
@@ -152,6 +156,7 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
     // of an outstanding load would stall on it.
     struct WSet { u4 w[NT][C::WL]; uint32_t s[NT][C::NG], z[NT][C::NG]; };   // 16-bit values, one register each
     WSet set0, set1;
+    u2 m_cur[NT][2], m_next[NT][2];                               // META4: [tile][scales, zero points] of 4 steps
 
     f4 acc[MT][NT];
 #pragma unroll
@@ -190,6 +195,9 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
             else ws.z[j][g] = __builtin_amdgcn_raw_buffer_load_b16(rz, m_off[j] + (g0 + g) * 2, 0, 0);
         }
     };
+    auto issue_meta4 = [&](int j, int which, int c, u2 (*m)[2]) {   // steps c .. c+3; next-row or zero past the row's end
+        m[j][which] = __builtin_amdgcn_raw_buffer_load_b64(which == 0 ? rs : rz, m_off[j] + c * 2, 0, 0);
+    };
     // Weight fragment of MFMA step t: values [8 t, 8 t + 8) of the lane's VPL, from lane load t / SPL.
     auto unpack = [&](const WSet& ws, int j, int t, const GroupConst<BITS>* gcj) {
         static_assert(C::WL == 1 || C::NG == 1, "two lane loads share one group");
@@ -202,14 +210,20 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
     // every step the staging and global requests listed at slot_requests below.
     // Requests past the last chunk are range-checked to zero by the hardware; no branches, so every wait
     // count is exact.
-    auto step = [&](int c, const _Float16* cur, _Float16* nxt, WSet& ws) {
+    // `ph` (META4 only): position of the step in its run of four, a constant after inlining.
+    auto step = [&](int c, const _Float16* cur, _Float16* nxt, WSet& ws, const int ph) {
         __builtin_amdgcn_sched_barrier(0);
         GroupConst<BITS> gc[NT][C::NG];
 #pragma unroll
         for (int j = 0; j < NT; j++)
 #pragma unroll
-            for (int g = 0; g < C::NG; g++)
-                gc[j][g].set(__builtin_bit_cast(_Float16, (uint16_t)ws.s[j][g]), __builtin_bit_cast(_Float16, (uint16_t)ws.z[j][g]));
+            for (int g = 0; g < C::NG; g++) {
+                if constexpr (META4)
+                    gc[j][g].set(__builtin_bit_cast(_Float16, (uint16_t)(m_cur[j][0][ph >> 1] >> (16 * (ph & 1)))),
+                                 __builtin_bit_cast(_Float16, (uint16_t)(m_cur[j][1][ph >> 1] >> (16 * (ph & 1)))));
+                else
+                    gc[j][g].set(__builtin_bit_cast(_Float16, (uint16_t)ws.s[j][g]), __builtin_bit_cast(_Float16, (uint16_t)ws.z[j][g]));
+            }
         const _Float16* xp = cur + nl * C::PITCH + kq * C::VPL;
         h8 xf[2][MT];
         h2 wf[2][NT][4];                                  // weight fragments as 4 register pairs each
@@ -233,7 +247,11 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
                 stage_unit(i, nxt);
                 issue_x_unit(i, c + 2);
             }
-            if (t == 1) issue_meta(i / 2, i & 1, c + 2, ws);
+            if constexpr (META4) {
+                if (t == 1 && ph == 0) issue_meta4(i / 2, i & 1, c + 4, m_next);
+            } else {
+                if (t == 1) issue_meta(i / 2, i & 1, c + 2, ws);
+            }
             if (t == C::MF - 1 && (C::WL == 2 || !(i & 1))) issue_w_load(i / 2, C::WL == 2 ? (i & 1) : 0, c + 2, ws);
             asm volatile("" ::: "memory");
         };
@@ -311,6 +329,7 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
         }
 #pragma unroll
         for (int j = 0; j < NT; j++) {
+            if constexpr (META4) break;
             issue_meta(j, 0, c, ws);
             issue_meta(j, 1, c, ws);
             asm volatile("" ::: "memory");
@@ -325,15 +344,40 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
                 __builtin_amdgcn_sched_barrier(0);
             }
     };
+    if constexpr (META4) {
+#pragma unroll
+        for (int j = 0; j < NT; j++) {
+            issue_meta4(j, 0, c_begin, m_cur);
+            issue_meta4(j, 1, c_begin, m_cur);
+            asm volatile("" ::: "memory");
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
     issue_batch(c_begin, set0);
 #pragma unroll
     for (int i = 0; i < C::XL; i++) stage_unit(i, buf0);
     __builtin_amdgcn_sched_barrier(0);
     issue_batch(c_begin + 1, set1);
     __syncthreads();
-    for (int c = c_begin; c < c_end; c += 2) {   // an odd chunk count runs one extra step on zeros
-        step(c, buf0, buf1, set0);
-        step(c + 1, buf1, buf0, set1);
+    if constexpr (META4) {
+        int c = c_begin;
+        for (; c + 2 < c_end; c += 4) {          // runs of four steps; the last may run one step on zeros
+            step(c, buf0, buf1, set0, 0);
+            step(c + 1, buf1, buf0, set1, 1);
+            step(c + 2, buf0, buf1, set0, 2);
+            step(c + 3, buf1, buf0, set1, 3);
+#pragma unroll
+            for (int j = 0; j < NT; j++) { m_cur[j][0] = m_next[j][0]; m_cur[j][1] = m_next[j][1]; }
+        }
+        if (c < c_end) {                         // one or two steps left
+            step(c, buf0, buf1, set0, 0);
+            step(c + 1, buf1, buf0, set1, 1);
+        }
+    } else {
+        for (int c = c_begin; c < c_end; c += 2) {   // an odd chunk count runs one extra step on zeros
+            step(c, buf0, buf1, set0, 0);
+            step(c + 1, buf1, buf0, set1, 0);
+        }
     }
     // acc[i][j][r] = y[m0 + 16 i + nl][n0 + 16 j + 4 kq + r]
     if (partial) {
@@ -460,9 +504,16 @@ int launch_gemm(GemmArgs a, void* workspace, size_t workspace_bytes, hipStream_t
     using C = GemmCfg<BITS, GROUP>;
     static_assert(C::CHUNK_BYTES == (BITS == 8 ? 128 : 64), "gemm_chunks() counts K steps of this size");
     const size_t lds = 2 * (size_t)C::STAGE_BYTES;
-    auto kern = qgemm_kernel<BITS, GROUP>;
-    static uint64_t big_lds_devices = 0;                   // per instantiation
-    if (lds > 64 * 1024 && !bw_allow_big_lds(reinterpret_cast<const void*>(kern), big_lds_devices)) return BW_ELAUNCH;
+    void (*kern)(const GemmArgs) = qgemm_kernel<BITS, GROUP, false>;
+    static uint64_t big_lds_devices[2] = {0, 0};           // per kernel
+    int which = 0;
+    if constexpr (C::CAN_META4) {
+        if (a.groups % 2 == 0 && bw_aligned(a.scale, 4) && bw_aligned(a.zp, 4)) {
+            kern = qgemm_kernel<BITS, GROUP, true>;
+            which = 1;
+        }
+    }
+    if (lds > 64 * 1024 && !bw_allow_big_lds(reinterpret_cast<const void*>(kern), big_lds_devices[which])) return BW_ELAUNCH;
     const GemmPlan p = gemm_plan(a.M, a.N, a.nchunks, workspace != nullptr);
     if (p.ws_bytes > workspace_bytes) return BW_EWORKSPACE;
     a.ws = (float*)workspace;

@@ -49,6 +49,31 @@ def test_ragged_shapes_through_the_abi(case):
     check_matmul(y[:, :n], x, qw, s16, z16, b16 if use_bias else None, bits, g)
 
 
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("groups,offset", [(12, 0), (12, 1), (13, 0), (14, 2), (14, 3), (43, 0)])
+def test_prefill_scale_rows_at_every_alignment(bits, groups, offset):
+    """The 128-group prefill kernel fetches the scales of four K steps in one request when a row of scales
+    starts on a 4-byte boundary; an odd number of groups or a base address off by one element must take the
+    per-step requests and give the same result.  K steps that are not a multiple of four end in a short run."""
+    from bitween_amd.kernels import hip_loader
+    lib = hip_loader.load()
+    g, n, m = 128, 300, 192
+    k = g * groups
+    _, qw, s16, z16, _ = quantized_layer(n, k, bits, g, seed=77 + groups, outliers=True)
+    x = np.random.default_rng(groups).standard_normal((m, k)).astype(np.float16)
+    sbuf = torch.zeros(n * groups + offset, dtype=torch.float16, device="cuda")
+    zbuf = torch.zeros(n * groups + offset, dtype=torch.float16, device="cuda")
+    sbuf[offset:] = to_gpu(s16).reshape(-1)
+    zbuf[offset:] = to_gpu(z16).reshape(-1)
+    xg, qg = to_gpu(x), to_gpu(qw)
+    y = torch.empty((m, n), dtype=torch.float16, device="cuda")
+    st = lib.bw_qgemm(xg.data_ptr(), 0, m, k, k, qg.data_ptr(), sbuf.data_ptr() + 2 * offset, zbuf.data_ptr() + 2 * offset,
+                      None, n, bits, g, y.data_ptr(), n, ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    assert st == 0
+    torch.cuda.synchronize()
+    check_matmul(y, x, qw, s16, z16, None, bits, g)
+
+
 @pytest.mark.parametrize("bits,g,n,k", [(4, 128, 5, 256), (8, 32, 33, 96), (2, 64, 17, 192), (4, 32, 1, 32)])
 def test_quantize_dequantize_ragged(bits, g, n, k):
     """Row counts that leave waves partly empty, with a padded row pitch on the way in and out."""
