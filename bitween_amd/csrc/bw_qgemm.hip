@@ -38,6 +38,14 @@ struct GemmCfg {
     // come in one request per tile instead of four (kernel parameter META4; needs rows of scales that
     // start on 4-byte boundaries, i.e. an even number of groups).
     static constexpr bool CAN_META4 = CHUNK_K == GROUP;
+    // Where the per-step side work sits (each placement measured per format, M = 512 and 2048):
+    // EARLY_W: the first weight fragments of a K step are unpacked under the last MFMA step of the step
+    // before (else at the start of the step, with the matrix pipe idle);
+    // T_STAGE: the MFMA step whose slots move the next chunk's activations to LDS and re-request them.
+    // 4 bits: early, last step (3-9 % over start-of-step / first step); 2 bits at group 32: early, last but
+    // one (5 %); 8 bits and 2 bits at larger groups were fastest as they were.
+    static constexpr bool EARLY_W = BITS == 4 || (BITS == 2 && GROUP == 32);
+    static constexpr int T_STAGE = BITS == 4 ? MF - 1 : (BITS == 2 && GROUP == 32) ? MF - 2 : 0;
     static constexpr int PITCH = CHUNK_K + 8;                    // halves per LDS row
     static constexpr int STAGE_BYTES = BM * PITCH * 2;
     static constexpr int UNIT = VPI > 8 ? VPI : 8;               // halves permuted together when staging x
@@ -113,10 +121,11 @@ BW_DEV __amdgpu_buffer_rsrc_t make_rsrc(const void* p, uint32_t bytes) {
 }
 
 // Software pipeline, one K step = one chunk:
-//   step c computes from LDS buffer c&1 and weight registers `wr`;
-//   the activations of step c+1 were requested one step earlier and are written to buffer (c+1)&1 after the
-//   MFMAs of step c; the weights of step c+1 likewise sit in `wn` and are moved to `wr`;
-//   then the loads of step c+2 are issued.  Every global load has a full K step (~2000 MFMA cycles) to land.
+//   step c computes from LDS buffer c&1 and the weight register set c&1 (two sets, used alternately and
+//   never copied);
+//   the activations of chunk c+1 were requested one step earlier and are written to buffer (c+1)&1 during
+//   step c, then re-requested for chunk c+2; the weights of chunk c+2 are requested into step c's own set
+//   once its last fragment is unpacked.  Every global load has a full K step (~2000 MFMA cycles) to land.
 template <int BITS, int GROUP, bool META4>
 __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
     using C = GemmCfg<BITS, GROUP>;
@@ -205,67 +214,84 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
     };
 
     // One K step.  The 32 MFMAs of MFMA step t are issued in groups of 4 (one m-tile); between two groups
-    // sits one slice of other work, fenced so the compiler keeps it there: for t < last the LDS read of one
-    // activation fragment and (every other slot) the unpack of one weight fragment of step t+1, and in
-    // every step the staging and global requests listed at slot_requests below.
+    // sits one slice of other work, fenced so the compiler keeps it there: the LDS read of one activation
+    // fragment and (every other slot) the unpack of one weight fragment of MFMA step t+1 - in the last MFMA
+    // step that is the first fragment of the NEXT K step, taken from the other register set, so a step starts
+    // with its weight fragments ready - plus the staging and global requests listed at slot_requests below.
     // Requests past the last chunk are range-checked to zero by the hardware; no branches, so every wait
     // count is exact.
     // `ph` (META4 only): position of the step in its run of four, a constant after inlining.
-    auto step = [&](int c, const _Float16* cur, _Float16* nxt, WSet& ws, const int ph) {
+    static_assert(C::MF % 2 == 0, "the fragment double buffer returns to slot 0 at the end of a step");
+    using GC = GroupConst<BITS>;
+    h8 xf[2][MT];
+    h2 wf[2][NT][4];                                      // weight fragments as 4 register pairs each
+    // group constants of tile j for the step that reads `from` (META4: half `half` of m_cur / m_next)
+    auto set_consts = [&](GC* gj, int j, const WSet& from, const u2 (*m)[2], int half) {
+#pragma unroll
+        for (int g = 0; g < C::NG; g++) {
+            if constexpr (META4)
+                gj[g].set(__builtin_bit_cast(_Float16, (uint16_t)(m[j][0][half >> 1] >> (16 * (half & 1)))),
+                          __builtin_bit_cast(_Float16, (uint16_t)(m[j][1][half >> 1] >> (16 * (half & 1)))));
+            else
+                gj[g].set(__builtin_bit_cast(_Float16, (uint16_t)from.s[j][g]), __builtin_bit_cast(_Float16, (uint16_t)from.z[j][g]));
+        }
+    };
+    auto step = [&](int c, const _Float16* cur, _Float16* nxt, WSet& ws, const WSet& wsn, GC (&gc)[NT][C::NG],
+                    GC (&gn)[NT][C::NG], const int ph) {
         __builtin_amdgcn_sched_barrier(0);
-        GroupConst<BITS> gc[NT][C::NG];
-#pragma unroll
-        for (int j = 0; j < NT; j++)
-#pragma unroll
-            for (int g = 0; g < C::NG; g++) {
-                if constexpr (META4)
-                    gc[j][g].set(__builtin_bit_cast(_Float16, (uint16_t)(m_cur[j][0][ph >> 1] >> (16 * (ph & 1)))),
-                                 __builtin_bit_cast(_Float16, (uint16_t)(m_cur[j][1][ph >> 1] >> (16 * (ph & 1)))));
-                else
-                    gc[j][g].set(__builtin_bit_cast(_Float16, (uint16_t)ws.s[j][g]), __builtin_bit_cast(_Float16, (uint16_t)ws.z[j][g]));
-            }
         const _Float16* xp = cur + nl * C::PITCH + kq * C::VPL;
-        h8 xf[2][MT];
-        h2 wf[2][NT][4];                                  // weight fragments as 4 register pairs each
 #pragma unroll
         for (int i = 0; i < MT; i++) xf[0][i] = *reinterpret_cast<const h8*>(xp + i * 16 * C::PITCH);
+        if constexpr (!C::EARLY_W) {
 #pragma unroll
-        for (int j = 0; j < NT; j++) {
-            const h8 f = unpack(ws, j, 0, gc[j]);
+            for (int j = 0; j < NT; j++) {
+                set_consts(gc[j], j, ws, m_cur, ph);
+                const h8 f = unpack(ws, j, 0, gc[j]);
 #pragma unroll
-            for (int e = 0; e < 4; e++) wf[0][j][e] = h2{f[2 * e], f[2 * e + 1]};
-        }
-        // At most one global request per slot, spread over the whole K step: a burst of requests backs up
-        // the address unit and the wave - which issues in order - stops feeding MFMAs.
-        //   first MFMA step : activations of chunk c+1 (requested a step ago) to LDS, re-request
-        //   middle          : scales and zero points for chunk c+2 (their registers are free once the
-        //                     step's constants are formed)
-        //   last MFMA step  : weights for chunk c+2 (their registers are free after the last unpack)
-        auto slot_requests = [&](int t, int i) {
-            static_assert(C::MF >= 4, "first, middle and last MFMA step are distinct");
-            if (t == 0 && i < C::XL) {
-                stage_unit(i, nxt);
-                issue_x_unit(i, c + 2);
+                for (int e = 0; e < 4; e++) wf[0][j][e] = h2{f[2 * e], f[2 * e + 1]};
             }
+        }
+        // At most one global request per slot, spread over the K step: a burst of requests backs up
+        // the address unit and the wave - which issues in order - stops feeding MFMAs.
+        //   second MFMA step : scales and zero points (for chunk c+2, or for the next run of four steps)
+        //   last MFMA step   : activations of chunk c+1 (requested a step ago) to LDS, re-request for c+2;
+        //                      weights for chunk c+2 (their registers are free after the last unpack).
+        // The last MFMA step has no fragment reads and is where these fit under the MFMAs.
+        auto slot_requests = [&](int t, int i) {
+            static_assert(C::MF >= 4, "second and last MFMA step are distinct");
             if constexpr (META4) {
                 if (t == 1 && ph == 0) issue_meta4(i / 2, i & 1, c + 4, m_next);
             } else {
                 if (t == 1) issue_meta(i / 2, i & 1, c + 2, ws);
             }
+            if (t == C::T_STAGE && i < C::XL) {
+                stage_unit(i, nxt);
+                issue_x_unit(i, c + 2);
+            }
             if (t == C::MF - 1 && (C::WL == 2 || !(i & 1))) issue_w_load(i / 2, C::WL == 2 ? (i & 1) : 0, c + 2, ws);
             asm volatile("" ::: "memory");
+        };
+        auto next_consts = [&](int j) {
+            if constexpr (META4) set_consts(gn[j], j, wsn, ph < 3 ? m_cur : m_next, ph < 3 ? ph + 1 : 0);
+            else set_consts(gn[j], j, wsn, m_cur, 0);
         };
 #pragma unroll
         for (int t = 0; t < C::MF; t++) {
             const int cu = t & 1, nx = cu ^ 1;
+            const bool last = t == C::MF - 1, early = last && C::EARLY_W;
 #pragma unroll
             for (int i = 0; i < MT; i++) {
                 if constexpr (BITS == 4) {
                     // An MFMA occupies the matrix pipe for 16 cycles but the issue port for 4: two or three
                     // VALU operations fit behind each one.  Slot i prepares half a weight fragment of
-                    // MFMA step t+1 (tile i/2, words' low or high byte pair) in four such pieces.
+                    // the next MFMA step (tile i/2, words' low or high byte pair) in four such pieces.
                     const int jn = i / 2;
-                    const GroupConst<4>& g4 = gc[jn][(t + 1 < C::MF ? t + 1 : t) / C::WPG];
+                    if (early && !(i & 1)) {
+                        __builtin_amdgcn_sched_barrier(0);
+                        next_consts(jn);
+                    }
+                    const GroupConst<4>& g4 = early ? gn[jn][0] : gc[jn][(last ? t : t + 1) / C::WPG];
+                    const uint32_t word = early ? wsn.w[jn][0][0] : ws.w[jn][0][last ? t : t + 1];
                     const h2 k16 = splat((_Float16)0.0625f);
                     uint32_t wsrc = 0;
                     h2 pa = {0, 0}, pb = {0, 0};
@@ -274,10 +300,10 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
                         __builtin_amdgcn_sched_barrier(0);
                         mfma_acc(acc[i][j], pack_h8(wf[cu][j]), xf[cu][i]);
                         __builtin_amdgcn_sched_barrier(0);
-                        if (t + 1 < C::MF) {
+                        if (!last || early) {
                             if (j == 0) {
-                                xf[nx][i] = *reinterpret_cast<const h8*>(xp + i * 16 * C::PITCH + 8 * (t + 1));
-                                wsrc = (i & 1) ? ws.w[jn][0][t + 1] >> 8 : ws.w[jn][0][t + 1];
+                                if (!last) xf[nx][i] = *reinterpret_cast<const h8*>(xp + i * 16 * C::PITCH + 8 * (t + 1));
+                                wsrc = (i & 1) ? word >> 8 : word;
                                 pa = as_h2(and_or(wsrc, 0x000F000Fu, kMagic));
                             } else if (j == 1) {
                                 pb = as_h2(and_or(wsrc, 0x00F000F0u, kMagic));
@@ -299,13 +325,13 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
 #pragma unroll
                     for (int j = 0; j < NT; j++) mfma_acc(acc[i][j], pack_h8(wf[cu][j]), xf[cu][i]);
                     __builtin_amdgcn_sched_barrier(0);
-                    if (t + 1 < C::MF) {
-                        xf[nx][i] = *reinterpret_cast<const h8*>(xp + i * 16 * C::PITCH + 8 * (t + 1));
-                        if (i & 1) {
-                            const h8 f = unpack(ws, i / 2, t + 1, gc[i / 2]);
+                    if (!last) xf[nx][i] = *reinterpret_cast<const h8*>(xp + i * 16 * C::PITCH + 8 * (t + 1));
+                    if (!(i & 1)) {
+                        if (early) next_consts(i / 2);
+                    } else if (!last || early) {
+                        const h8 f = early ? unpack(wsn, i / 2, 0, gn[i / 2]) : unpack(ws, i / 2, t + 1, gc[i / 2]);
 #pragma unroll
-                            for (int e = 0; e < 4; e++) wf[nx][i / 2][e] = h2{f[2 * e], f[2 * e + 1]};
-                        }
+                        for (int e = 0; e < 4; e++) wf[nx][i / 2][e] = h2{f[2 * e], f[2 * e + 1]};
                     }
                     slot_requests(t, i);
                 }
@@ -357,26 +383,54 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
 #pragma unroll
     for (int i = 0; i < C::XL; i++) stage_unit(i, buf0);
     __builtin_amdgcn_sched_barrier(0);
-    issue_batch(c_begin + 1, set1);
+    // second batch in the order of a steady-state step
+    if constexpr (C::T_STAGE == 0) {
+        issue_batch(c_begin + 1, set1);
+    } else {
+    if constexpr (!META4) {
+#pragma unroll
+        for (int j = 0; j < NT; j++) {
+            issue_meta(j, 0, c_begin + 1, set1);
+            issue_meta(j, 1, c_begin + 1, set1);
+            asm volatile("" ::: "memory");
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < MT; i++) {
+        if (i < C::XL) issue_x_unit(i, c_begin + 1);
+        if (C::WL == 2 || !(i & 1)) issue_w_load(i / 2, C::WL == 2 ? (i & 1) : 0, c_begin + 1, set1);
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    }
+    GC gc0[NT][C::NG], gc1[NT][C::NG];
+#pragma unroll
+    for (int j = 0; j < NT; j++) {
+        set_consts(gc0[j], j, set0, m_cur, 0);
+        const h8 f = unpack(set0, j, 0, gc0[j]);
+#pragma unroll
+        for (int e = 0; e < 4; e++) wf[0][j][e] = h2{f[2 * e], f[2 * e + 1]};
+    }
     __syncthreads();
     if constexpr (META4) {
         int c = c_begin;
         for (; c + 2 < c_end; c += 4) {          // runs of four steps; the last may run one step on zeros
-            step(c, buf0, buf1, set0, 0);
-            step(c + 1, buf1, buf0, set1, 1);
-            step(c + 2, buf0, buf1, set0, 2);
-            step(c + 3, buf1, buf0, set1, 3);
+            step(c, buf0, buf1, set0, set1, gc0, gc1, 0);
+            step(c + 1, buf1, buf0, set1, set0, gc1, gc0, 1);
+            step(c + 2, buf0, buf1, set0, set1, gc0, gc1, 2);
+            step(c + 3, buf1, buf0, set1, set0, gc1, gc0, 3);
 #pragma unroll
             for (int j = 0; j < NT; j++) { m_cur[j][0] = m_next[j][0]; m_cur[j][1] = m_next[j][1]; }
         }
         if (c < c_end) {                         // one or two steps left
-            step(c, buf0, buf1, set0, 0);
-            step(c + 1, buf1, buf0, set1, 1);
+            step(c, buf0, buf1, set0, set1, gc0, gc1, 0);
+            step(c + 1, buf1, buf0, set1, set0, gc1, gc0, 1);
         }
     } else {
         for (int c = c_begin; c < c_end; c += 2) {   // an odd chunk count runs one extra step on zeros
-            step(c, buf0, buf1, set0, 0);
-            step(c + 1, buf1, buf0, set1, 0);
+            step(c, buf0, buf1, set0, set1, gc0, gc1, 0);
+            step(c + 1, buf1, buf0, set1, set0, gc1, gc0, 0);
         }
     }
     // acc[i][j][r] = y[m0 + 16 i + nl][n0 + 16 j + 4 kq + r]
