@@ -612,7 +612,48 @@ __global__ void qgemm_generic_kernel(const _Float16* __restrict__ x, int M, int 
     y[(int64_t)m * ldy + n] = (_Float16)acc;
 }
 
+// bfloat16 -> float16 of a row-major matrix, 8 values (16 bytes) per unit; a thread converts the units
+// idx, idx + T, idx + 2T, idx + 3T (T = all threads) with every load issued before the first store.
+__global__ __launch_bounds__(256) void cast_bf16_f16_kernel(const uint16_t* __restrict__ x, uint16_t* __restrict__ y,
+                                                            int64_t units, int upr, int64_t ldx, int64_t ldy) {
+    const int64_t t0 = (int64_t)blockIdx.x * blockDim.x + threadIdx.x, stride = (int64_t)gridDim.x * blockDim.x;
+    u4 v[4];
+    int64_t dst[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const int64_t u = t0 + i * stride;
+        dst[i] = -1;
+        if (u < units) {
+            const int64_t r = u / upr, c = (u - r * upr) * 8;
+            v[i] = *reinterpret_cast<const u4*>(x + r * ldx + c);
+            dst[i] = r * ldy + c;
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        if (dst[i] < 0) continue;
+        u4 o;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const float lo = __builtin_bit_cast(float, v[i][j] << 16), hi = __builtin_bit_cast(float, v[i][j] & 0xFFFF0000u);
+            o[j] = as_u32(h2{(_Float16)lo, (_Float16)hi});
+        }
+        *reinterpret_cast<u4*>(y + dst[i]) = o;
+    }
+}
+
 }  // namespace
+
+extern "C" int bw_cast_bf16_f16(const void* x, int64_t rows, int64_t cols, int64_t ldx, void* y, int64_t ldy, void* stream) {
+    if (!x || !y || rows < 1 || cols < 1 || ldx < cols || ldy < cols) return BW_EINVAL;
+    if (cols % 8 || ldx % 8 || ldy % 8 || cols / 8 >= ((int64_t)1 << 31)) return BW_EUNSUPPORTED;
+    if (!bw_aligned(x, 16) || !bw_aligned(y, 16)) return BW_EALIGN;
+    const int64_t units = rows * (cols / 8), blocks = (units + 4 * 256 - 1) / (4 * 256);
+    if (blocks >= ((int64_t)1 << 31)) return BW_EUNSUPPORTED;
+    hipLaunchKernelGGL(cast_bf16_f16_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, (const uint16_t*)x,
+                       (uint16_t*)y, units, (int)(cols / 8), ldx, ldy);
+    return hipGetLastError() == hipSuccess ? BW_OK : BW_ELAUNCH;
+}
 
 int bw_qgemm_generic(const void* x, int act_dtype, int64_t M, int64_t K, int64_t ldx, const int32_t* qweight,
                      const void* scale16, const void* zp16, const void* bias, int64_t N, int bits, int group, void* y,

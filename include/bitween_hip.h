@@ -123,6 +123,13 @@ int bw_qlinear(const void* x, int act_dtype, int64_t M, int64_t K, int64_t ldx,
                const int32_t* qweight, const void* scale16, const void* zp16, const void* bias,
                int64_t N, int bits, int group, void* y, int64_t ldy, void* stream);
 
+/* x.to(float16) of a bfloat16 activation matrix ahead of the prefill kernel
+ * replaces the cast in QuantizedLinearFunction.forward (bitween/modules.py:74) for bfloat16 x beyond the rows
+ * that bw_qgemv / bw_qlinear convert in-kernel.  Round to nearest even, as the tensor cast.
+ *   x [rows][ldx] bfloat16, y [rows][ldy] float16; cols, ldx, ldy multiples of 8 and 16-byte-aligned pointers,
+ *   otherwise BW_EUNSUPPORTED / BW_EALIGN (the Python forward then uses the tensor cast). */
+int bw_cast_bf16_f16(const void* x, int64_t rows, int64_t cols, int64_t ldx, void* y, int64_t ldy, void* stream);
+
 /* Input gradient, fused with the dequantisation:  grad_x[M][K] = grad_y[M][N] @ W16[N][K]
  * replaces QuantizedLinearFunction.backward (bitween/modules.py:108-141), which unpacks the weights, forms
  * scale * (q - zp), casts it to grad_output's dtype and calls matmul; for float16 gradients that cast gives the

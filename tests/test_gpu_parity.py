@@ -599,3 +599,29 @@ def test_validated_buffer_cache_follows_replaced_buffers():
     assert torch.equal(qf(x.to(torch.bfloat16)), qf(x.to(torch.bfloat16).to(torch.float16)))
     xs = torch.randn(3, 2 * k, device="cuda", dtype=torch.float16)[:, ::2]     # strided x falls back to the general path
     assert torch.equal(qf(xs), qf(xs.contiguous()))
+
+
+def test_bf16_cast_matches_tensor_cast_bit_for_bit():
+    """bw_cast_bf16_f16 is the x.to(float16) of the reference's forward (bitween/modules.py:74): every bfloat16 bit
+    pattern, through a padded row pitch on both sides, against torch's own cast."""
+    import ctypes
+    from bitween_amd.kernels import hip_loader as hip
+    lib = hip.load()
+    allbits = torch.arange(-32768, 32768, dtype=torch.int32).to(torch.int16).cuda().view(torch.bfloat16)   # 65536 patterns
+    rows, cols, ldx, ldy = 64, 1024, 1024 + 8, 1024 + 24
+    xbuf = torch.zeros((rows, ldx), dtype=torch.bfloat16, device="cuda")
+    xbuf[:, :cols] = allbits.view(rows, cols)
+    ybuf = torch.full((rows, ldy), 7.0, dtype=torch.float16, device="cuda")
+    st = lib.bw_cast_bf16_f16(xbuf.data_ptr(), rows, cols, ldx, ybuf.data_ptr(), ldy,
+                              ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    assert st == 0
+    torch.cuda.synchronize()
+    want = xbuf[:, :cols].to(torch.float16)
+    assert torch.equal(ybuf[:, :cols].view(torch.int16), want.view(torch.int16))
+    assert (ybuf[:, cols:] == 7.0).all()
+    # layouts the kernel does not take are refused, and the Python forward falls back to the tensor cast
+    assert lib.bw_cast_bf16_f16(xbuf.data_ptr(), rows, 1020, ldx, ybuf.data_ptr(), ldy, None) == -2
+    assert lib.bw_cast_bf16_f16(xbuf.data_ptr() + 2, rows, cols, ldx, ybuf.data_ptr(), ldy, None) == -3
+    for shape in ((200, 1020), (64, 4096), (2048, 4096)):      # odd K, below and above the size where the kernel takes over
+        x = torch.randn(*shape, device="cuda").to(torch.bfloat16)
+        assert torch.equal(hip._bf16_to_f16(x), x.to(torch.float16))
