@@ -204,7 +204,10 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
             else ws.z[j][g] = __builtin_amdgcn_raw_buffer_load_b16(rz, m_off[j] + (g0 + g) * 2, 0, 0);
         }
     };
-    auto issue_meta4 = [&](int j, int which, int c, u2 (*m)[2]) {   // steps c .. c+3; next-row or zero past the row's end
+    // Scales (zero points) of steps c .. c+3.  Past the row's last group this reads the next row's (or zero past
+    // the buffer); no step that runs ever uses those: a META4 launch has an even group count and even slices, so
+    // the K loop below never pads with a zero step, and what the last step prepares for its successor is dropped.
+    auto issue_meta4 = [&](int j, int which, int c, u2 (*m)[2]) {
         m[j][which] = __builtin_amdgcn_raw_buffer_load_b64(which == 0 ? rs : rz, m_off[j] + c * 2, 0, 0);
     };
     // Weight fragment of MFMA step t: values [8 t, 8 t + 8) of the lane's VPL, from lane load t / SPL.

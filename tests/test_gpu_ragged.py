@@ -74,6 +74,41 @@ def test_prefill_scale_rows_at_every_alignment(bits, groups, offset):
     check_matmul(y, x, qw, s16, z16, None, bits, g)
 
 
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("groups", [13, 14, 15, 16])
+def test_prefill_rows_do_not_see_their_neighbours_scales(bits, groups):
+    """The K loop runs in steps of two or four groups and pads with zero steps; a row whose scale or zero point
+    is Inf / NaN (its own outputs are then not finite, as in the reference) must leave every other row as it was."""
+    from bitween_amd.kernels import hip_loader
+    lib = hip_loader.load()
+    g, n, m = 128, 64, 130
+    k = g * groups
+    _, qw, s16, z16, _ = quantized_layer(n, k, bits, g, seed=5 + groups)
+    x = to_gpu(np.random.default_rng(groups).standard_normal((m, k)).astype(np.float16))
+    qg = to_gpu(qw)
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    def run(s, z):
+        sg, zg = to_gpu(s), to_gpu(z)
+        y = torch.empty((m, n), dtype=torch.float16, device="cuda")
+        assert lib.bw_qgemm(x.data_ptr(), 0, m, k, k, qg.data_ptr(), sg.data_ptr(), zg.data_ptr(), None, n, bits, g,
+                            y.data_ptr(), n, stream) == 0
+        torch.cuda.synchronize()
+        return y
+
+    clean = run(s16, z16)
+    assert torch.isfinite(clean).all()
+    bad_rows = [7, 20, 63]
+    s_bad, z_bad = s16.copy(), z16.copy()
+    s_bad[7, :] = np.inf
+    z_bad[20, :] = np.nan
+    s_bad[63, 0] = np.nan
+    dirty = run(s_bad, z_bad)
+    keep = [r for r in range(n) if r not in bad_rows]
+    assert torch.equal(dirty[:, keep], clean[:, keep])
+    assert not torch.isfinite(dirty[:, bad_rows]).all()
+
+
 @pytest.mark.parametrize("bits,g,n,k", [(4, 128, 5, 256), (8, 32, 33, 96), (2, 64, 17, 192), (4, 32, 1, 32)])
 def test_quantize_dequantize_ragged(bits, g, n, k):
     """Row counts that leave waves partly empty, with a padded row pitch on the way in and out."""
