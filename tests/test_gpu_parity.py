@@ -625,3 +625,41 @@ def test_bf16_cast_matches_tensor_cast_bit_for_bit():
     for shape in ((200, 1020), (64, 4096), (2048, 4096)):      # odd K, below and above the size where the kernel takes over
         x = torch.randn(*shape, device="cuda").to(torch.bfloat16)
         assert torch.equal(hip._bf16_to_f16(x), x.to(torch.float16))
+
+
+@pytest.mark.parametrize("m,dtype", [(1, torch.float16), (16, torch.bfloat16), (64, torch.float16), (160, torch.float16),
+                                      (2048, torch.bfloat16)])
+def test_forward_under_graph_capture_replays_like_eager(m, dtype):
+    """A captured forward of two QuantizedLinear layers (decode, 16-row launches, prefill with its split-K workspace
+    and, for bfloat16 prefill input, the cast kernel) replayed with new inputs gives what the eager call gives,
+    bit for bit, on every replay; eager work and synchronisations sit between the replays."""
+    from bitween_amd import QuantizedLinear
+    torch.manual_seed(m)
+    k, h = 2048, 1024
+    lin1 = torch.nn.Linear(k, h, bias=True, dtype=torch.float16, device="cuda")
+    lin2 = torch.nn.Linear(h, k, bias=False, dtype=torch.float16, device="cuda")
+    q1 = QuantizedLinear.from_float(lin1, bits=4, group_size=128)
+    q2 = QuantizedLinear.from_float(lin2, bits=8, group_size=64)
+
+    def net(x):
+        return q2(torch.nn.functional.silu(q1(x)).to(dtype))
+
+    static_x = torch.randn(m, k, device="cuda").to(dtype)
+    with torch.no_grad():
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(2):
+                net(static_x)
+        torch.cuda.current_stream().wait_stream(side)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            static_y = net(static_x)
+        for i in range(4):
+            x = torch.randn(m, k, device="cuda").to(dtype) * (1 + i)
+            want = net(x)
+            torch.cuda.synchronize()
+            static_x.copy_(x)
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(static_y, want), f"replay {i}"
