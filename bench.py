@@ -190,6 +190,26 @@ def extras_prefill(torch, hip, QuantizedLinear, layers):
     return out
 
 
+def extras_prefill_other_formats(torch, hip, QuantizedLinear, layers):
+    """Prefill at the other widths of the mixed-precision recipe (attention int8 g128, four down_proj int2 g32) and
+    int4 g64, 4096 -> 14336, against the same fp16 hipBLASLt GEMM."""
+    out, k, n = {}, 4096, 14336
+    for bits, g in ((8, 128), (4, 64), (2, 32)):
+        q = make_layer(torch, QuantizedLinear, k, n, bits, g, seed=7)
+        w16 = hip.dequantize(q.qweight, q.scale, q.zero_point, g, bits, torch.float16)
+        for mm in (512, 2048):
+            x = torch.randn(mm, k, device="cuda", dtype=torch.float16)
+            # 60 untimed calls first: the first large GEMMs of a fresh process run ~18 % slow (clocks, first touch of
+            # the workspace), whichever kernel they are
+            us_q = time_calls(torch, lambda: hip.quantized_gemm_hip(x, q.qweight, q.scale, q.zero_point, None, bits, g), 20, 60)
+            us_b = time_calls(torch, lambda: torch.matmul(x, w16.T), 20, 20)
+            fl = 2.0 * mm * n * k
+            out[f"w{bits}g{g}_{k}x{n}_M{mm}"] = {"us": round(us_q, 1), "TFLOPs": round(fl / us_q / 1e6, 1),
+                                                 "hipblaslt_fp16_us": round(us_b, 1), "frac_of_hipblaslt": round(us_b / us_q, 3)}
+        del q, w16
+    return out
+
+
 def extras_quantize(torch, hip, QuantizedLinear, layers):
     """Quantiser: fp16 weights in, packed words + fp16 scale / zero point out (the from_float path)."""
     out = {}
@@ -473,7 +493,7 @@ def extras_opt125m_fc1(torch, hip, QuantizedLinear, layers):
 
 EXTRAS = {"opt125m_fc1": extras_opt125m_fc1, "decode": extras_decode, "decode_infinity_cache_hot": extras_decode_hot,
           "decode_other_formats": extras_decode_other_formats, "hipblaslt_fp16_decode": extras_hipblaslt_decode,
-          "prefill": extras_prefill, "quantize": extras_quantize, "mixed_precision_model": extras_mixed_precision_model, "eager_call": extras_eager_call,
+          "prefill": extras_prefill, "prefill_other_formats": extras_prefill_other_formats, "quantize": extras_quantize, "mixed_precision_model": extras_mixed_precision_model, "eager_call": extras_eager_call,
           "decode_fused_siblings": extras_decode_fused_siblings,
           # the heavy sections last: the GEMMs and the 7B model leave the board warm, which shows in the decode timings
           "backward": extras_backward, "llama7b_end_to_end": extras_llama7b_end_to_end}
