@@ -716,12 +716,19 @@ extern "C" int bw_qgemm(const void* x, int act_dtype, int64_t M, int64_t K, int6
     return bw_qgemm_ws(x, act_dtype, M, K, ldx, qweight, scale16, zp16, bias, N, bits, group, y, ldy, nullptr, 0, stream);
 }
 
+// Rows up to which bw_qlinear stays on the decode kernel (16 rows per launch; the later launches find the weights
+// in L2 / Infinity Cache).  Two launches always beat a mostly empty 128-row MFMA tile; a third does only while the
+// packed weights are small (4096 x 4096 at 4 or 8 bits: 13-17 us against 17-20 us), not for 20 MiB and more
+// (4096 x 11008 at 4 bits: 24-28 us against 22-23 us; at 8 bits 37-41 against 27).
+extern "C" int bw_qlinear_decode_rows(int64_t N, int64_t K, int bits) {
+    if (N < 1 || K < 1 || !bw_bits_ok(bits)) return 0;
+    return N * (K * bits / 8) < ((int64_t)20 << 20) ? 48 : 32;
+}
+
 extern "C" int bw_qlinear(const void* x, int act_dtype, int64_t M, int64_t K, int64_t ldx, const int32_t* qweight,
                           const void* scale16, const void* zp16, const void* bias, int64_t N, int bits, int group,
                           void* y, int64_t ldy, void* stream) {
-    // up to 48 rows the HBM-bound kernel, 16 rows per launch (the later launches find the weights in L2),
-    // beats a mostly empty 128-row MFMA tile
-    if (M >= 1 && M <= 48 && (act_dtype == BW_F16 || act_dtype == BW_BF16)) {
+    if (M >= 1 && M <= bw_qlinear_decode_rows(N, K, bits) && (act_dtype == BW_F16 || act_dtype == BW_BF16)) {
         for (int64_t m0 = 0; m0 < M; m0 += 16) {
             const int st = bw_qgemv((const _Float16*)x + m0 * ldx, act_dtype, M - m0 < 16 ? M - m0 : 16, K, ldx, qweight, scale16,
                                     zp16, bias, N, bits, group, (_Float16*)y + m0 * ldy, ldy, stream);

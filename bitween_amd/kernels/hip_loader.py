@@ -19,9 +19,9 @@ _lib = None
 BW_F16, BW_BF16, BW_F32, BW_I32 = 0, 1, 2, 3
 _DTYPE_CODE = {torch.float16: BW_F16, torch.bfloat16: BW_BF16, torch.float32: BW_F32, torch.int32: BW_I32}
 
-ABI_VERSION = 4            # what bw_abi_version() of a matching library returns
+ABI_VERSION = 5            # what bw_abi_version() of a matching library returns
 ENTRY_POINTS = ("bw_abi_version", "bw_strerror", "bw_quantize_pack", "bw_quantize_pack_add", "bw_dequantize", "bw_qgemv", "bw_qgemm",
-                "bw_qgemm_ws", "bw_qgemm_workspace_bytes", "bw_qlinear", "bw_qdgrad", "bw_qdgrad_workspace_bytes", "bw_cast_bf16_f16")
+                "bw_qgemm_ws", "bw_qgemm_workspace_bytes", "bw_qlinear", "bw_qdgrad", "bw_qdgrad_workspace_bytes", "bw_cast_bf16_f16", "bw_qlinear_decode_rows")
 
 
 class BitweenHipError(RuntimeError):
@@ -64,6 +64,8 @@ def load():
     lib.bw_qdgrad.restype = i32
     lib.bw_cast_bf16_f16.argtypes = [vp, i64, i64, i64, vp, i64, vp]
     lib.bw_cast_bf16_f16.restype = i32
+    lib.bw_qlinear_decode_rows.argtypes = [i64, i64, i32]
+    lib.bw_qlinear_decode_rows.restype = i32
     for name in ("bw_quantize_pack", "bw_quantize_pack_add", "bw_dequantize", "bw_qgemv", "bw_qgemm", "bw_qgemm_ws", "bw_qlinear"):
         getattr(lib, name).restype = i32
     for name in ("bw_qgemv", "bw_qgemm", "bw_qlinear"):
@@ -189,11 +191,13 @@ def _matmul(entry, x, qweight, scale, zero_point, bias, bits, group_size):
     if qweight.dtype is not torch.int32 or scale.dtype is not torch.float16 or zero_point.dtype is not torch.float16:
         raise TypeError("qweight must be int32 and scale / zero_point float16 (the QuantizedLinear buffers)")
     m = x.shape[0]
+    # rows that bw_qlinear keeps on the decode kernel: 32, and up to 48 for small layers
+    decode_rows = 32 if m <= 32 or entry != "bw_qlinear" else load().bw_qlinear_decode_rows(qweight.shape[0], x.shape[1], bits)
     act = BW_F16
     if x.dtype is torch.bfloat16:
         # the decode kernels round bfloat16 to float16 as they stage x (the reference's x.to(float16),
         # bitween/modules.py:74, without the extra kernel); the prefill kernel wants float16 in memory
-        if entry == "bw_qgemv" or (entry == "bw_qlinear" and m <= 48):
+        if entry == "bw_qgemv" or (entry == "bw_qlinear" and m <= decode_rows):
             act = BW_BF16
         else:
             x = _bf16_to_f16(x)
@@ -226,8 +230,8 @@ def _matmul(entry, x, qweight, scale, zero_point, bias, bits, group_size):
     if bias is not None:
         bias_ptr = (bias if bias.is_contiguous() else bias.contiguous()).data_ptr()
     with _on_device(x.device) as index:
-        if (entry == "bw_qgemm" and m > 16) or (entry == "bw_qlinear" and m > 48):
-            # prefill (bw_qlinear itself keeps M <= 48 on the decode kernel): give the library a split-K
+        if (entry == "bw_qgemm" and m > 16) or (entry == "bw_qlinear" and m > decode_rows):
+            # prefill (bw_qlinear itself keeps fewer rows on the decode kernel): give the library a split-K
             # workspace when the shape wants one
             nbytes = lib.bw_qgemm_workspace_bytes(m, n, k, bits, group_size)
             ws = torch.empty(nbytes, dtype=torch.uint8, device=x.device) if nbytes else None
@@ -265,12 +269,16 @@ def make_decode_plan(qweight, scale, zero_point, bias, bits, group_size):
     load()
     index = qweight.device.index if qweight.device.index is not None else torch.cuda.current_device()
     return (qweight, scale, zero_point, bias, qweight.data_ptr(), scale.data_ptr(), zero_point.data_ptr(),
-            None if bias is None else bias.data_ptr(), n, k, bits, group_size, index)
+            None if bias is None else bias.data_ptr(), n, k, bits, group_size, index,
+            load().bw_qlinear_decode_rows(n, k, bits))
 
 
 def decode_with_plan(plan, x, m):
-    """bw_qlinear for up to 48 rows with buffers validated by make_decode_plan: only x is looked at.  Returns None
-    when x does not qualify (layout, device, dtype) - the caller then takes quantized_matmul_hip."""
+    """bw_qlinear on its decode path with buffers validated by make_decode_plan: only x is looked at.  Returns None
+    when x does not qualify (layout, device, dtype, more rows than the decode path takes for this layer) - the
+    caller then takes quantized_matmul_hip."""
+    if m > plan[13]:
+        return None
     dt = x.dtype
     if dt is torch.float16:
         act = BW_F16

@@ -87,7 +87,7 @@ int bw_dequantize(const int32_t* qweight, const void* scale, int scale_dtype, co
  * reference dequantizes; products accumulate in float32; y is rounded once
  * (the reference rounds before and after the bias add; within its 1e-2
  * tolerance, main.py:471-477).
- *   x      [M][ldx] of act_dtype: BW_F16, or BW_BF16 for bw_qgemv and for bw_qlinear up to 48 rows - the
+ *   x      [M][ldx] of act_dtype: BW_F16, or BW_BF16 for bw_qgemv and for bw_qlinear while it stays on the decode kernel - the
  *          kernel then rounds every value to float16 as it reads it, which is the reference's
  *          x.to(float16) (bitween/modules.py:74) without a separate pass; other entry points return
  *          BW_EUNSUPPORTED for BW_BF16.  y [M][ldy] is float16 in every case, as in the reference.
@@ -97,7 +97,8 @@ int bw_dequantize(const int32_t* qweight, const void* scale, int scale_dtype, co
  * bw_qgemv: decode path, 1 <= M <= 16, HBM-bound, no workspace.
  * bw_qgemm: prefill path, any M >= 1, MFMA-bound.
  * bw_qlinear: picks between them by M (what the Python forward calls): the decode kernel, 16 rows per
- *             launch, up to M = 48; the prefill kernel (without a workspace) beyond. */
+ *             launch, up to M = bw_qlinear_decode_rows(N, K, bits) (48, or 32 for layers of 20 MiB of packed
+ *             weights and more); the prefill kernel (without a workspace) beyond. */
 int bw_qgemv(const void* x, int act_dtype, int64_t M, int64_t K, int64_t ldx,
              const int32_t* qweight, const void* scale16, const void* zp16, const void* bias,
              int64_t N, int bits, int group, void* y, int64_t ldy, void* stream);
@@ -118,6 +119,8 @@ int bw_qgemm_ws(const void* x, int act_dtype, int64_t M, int64_t K, int64_t ldx,
                 const int32_t* qweight, const void* scale16, const void* zp16, const void* bias,
                 int64_t N, int bits, int group, void* y, int64_t ldy,
                 void* workspace, size_t workspace_bytes, void* stream);
+
+int bw_qlinear_decode_rows(int64_t N, int64_t K, int bits);
 
 int bw_qlinear(const void* x, int act_dtype, int64_t M, int64_t K, int64_t ldx,
                const int32_t* qweight, const void* scale16, const void* zp16, const void* bias,

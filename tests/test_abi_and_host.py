@@ -28,7 +28,7 @@ def test_library_exports_every_declared_symbol():
     for name in declared:
         assert hasattr(lib, name), name
     lib.bw_abi_version.restype = ctypes.c_int
-    assert lib.bw_abi_version() == hip_loader.ABI_VERSION == 4
+    assert lib.bw_abi_version() == hip_loader.ABI_VERSION == 5
     lib.bw_strerror.restype = ctypes.c_char_p
     assert lib.bw_strerror(0) == b"ok" and b"invalid" in lib.bw_strerror(-1)
 
@@ -75,6 +75,16 @@ def test_split_k_workspace_size_is_a_pure_host_function():
     assert ws(128, 256, 128, 4, 128) == 0
     assert ws(128, 256, 100, 4, 32) == 0
     assert ws(128, 20, 96, 4, 48) == 0
+
+
+def test_decode_rows_switch_is_a_pure_host_function():
+    """bw_qlinear keeps up to 48 rows on the decode kernel for small layers and 32 for 20 MiB of packed weights and
+    more (three 16-row launches over a large layer lose to one prefill launch)."""
+    from bitween_amd.kernels import hip_loader
+    rows = hip_loader.load().bw_qlinear_decode_rows
+    assert rows(4096, 4096, 4) == 48 and rows(4096, 4096, 8) == 48 and rows(4096, 11008, 2) == 48
+    assert rows(11008, 4096, 4) == 32 and rows(4096, 11008, 8) == 32 and rows(14336, 4096, 4) == 32
+    assert rows(0, 4096, 4) == 0 and rows(4096, 4096, 3) == 0
 
 
 def test_host_layer_error_conventions_without_gpu():

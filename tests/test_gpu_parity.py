@@ -663,3 +663,35 @@ def test_forward_under_graph_capture_replays_like_eager(m, dtype):
             graph.replay()
             torch.cuda.synchronize()
             assert torch.equal(static_y, want), f"replay {i}"
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_rows_33_to_48_on_a_large_layer_take_the_prefill_kernel(dtype):
+    """For a layer of 20 MiB of packed weights and more bw_qlinear hands 33-48 rows to the prefill kernel; the module
+    forward (validated-buffer path, bfloat16 cast included) must follow it and agree with the C entry point."""
+    import ctypes
+    from bitween_amd import QuantizedLinear
+    from bitween_amd.kernels import hip_loader as hip
+    lib = hip.load()
+    k, n, bits, g = 4096, 11008, 4, 128
+    assert lib.bw_qlinear_decode_rows(n, k, bits) == 32
+    lin = torch.nn.Linear(k, n, bias=True, dtype=torch.float16, device="cuda")
+    q = QuantizedLinear.from_float(lin, bits=bits, group_size=g)
+    w16 = hip.dequantize(q.qweight, q.scale, q.zero_point, g, bits, torch.float16)
+    for m in (32, 33, 40, 48):
+        x = torch.randn(m, k, device="cuda").to(dtype)
+        with torch.no_grad():
+            y = q(x)
+        x16 = x.to(torch.float16)
+        ref = x16.double() @ w16.double().T + q.bias.double()
+        mag = x16.double().abs() @ w16.double().abs().T + 1.0
+        assert ((y.double() - ref).abs() <= 2.0 ** -10 * ref.abs() + 2.0 ** -12 * mag).all()
+        yc = torch.empty_like(y)
+        st = lib.bw_qlinear(x16.data_ptr(), 0, m, k, k, q.qweight.data_ptr(), q.scale.data_ptr(), q.zero_point.data_ptr(),
+                            q.bias.data_ptr(), n, bits, g, yc.data_ptr(), n, ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+        assert st == 0
+        torch.cuda.synchronize()
+        if m <= 32:
+            assert torch.equal(y, yc)                            # same decode launches either way
+        else:
+            assert ((y.double() - yc.double()).abs() <= 2.0 ** -9 * ref.abs() + 2.0 ** -12 * mag).all()   # split-K or not
