@@ -218,8 +218,8 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
 
     // One K step.  The 32 MFMAs of MFMA step t are issued in groups of 4 (one m-tile); between two groups
     // sits one slice of other work, fenced so the compiler keeps it there: the LDS read of one activation
-    // fragment and (every other slot) the unpack of one weight fragment of MFMA step t+1 - in the last MFMA
-    // step that is the first fragment of the NEXT K step, taken from the other register set, so a step starts
+    // fragment and (every other slot) the unpack of one weight fragment of MFMA step t+1 - with EARLY_W the last
+    // MFMA step prepares the first fragment of the NEXT K step, from the other register set, so that a step starts
     // with its weight fragments ready - plus the staging and global requests listed at slot_requests below.
     // Requests past the last chunk are range-checked to zero by the hardware; no branches, so every wait
     // count is exact.
@@ -256,10 +256,10 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
         }
         // At most one global request per slot, spread over the K step: a burst of requests backs up
         // the address unit and the wave - which issues in order - stops feeding MFMAs.
-        //   second MFMA step : scales and zero points (for chunk c+2, or for the next run of four steps)
-        //   last MFMA step   : activations of chunk c+1 (requested a step ago) to LDS, re-request for c+2;
-        //                      weights for chunk c+2 (their registers are free after the last unpack).
-        // The last MFMA step has no fragment reads and is where these fit under the MFMAs.
+        //   second MFMA step  : scales and zero points (for chunk c+2, or for the next run of four steps)
+        //   MFMA step T_STAGE : activations of chunk c+1 (requested a step ago) to LDS, re-request for c+2
+        //   last MFMA step    : weights for chunk c+2 (their registers are free after the last unpack).
+        // The last MFMA step reads no fragments of its own K step, which is why the 4-bit staging fits there.
         auto slot_requests = [&](int t, int i) {
             static_assert(C::MF >= 4, "second and last MFMA step are distinct");
             if constexpr (META4) {
