@@ -172,6 +172,17 @@ static inline bool bw_shape_ok(int64_t N, int64_t K, int bits, int group) {
 }
 static inline bool bw_aligned(const void* p, size_t a) { return ((uintptr_t)p & (a - 1)) == 0; }
 
+// Compute units of the current device (256 on MI355X); asked once.
+static inline int bw_device_cus() {
+    static const int cus = [] {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess)
+            n = 0;
+        return n > 0 ? n : 256;
+    }();
+    return cus;
+}
+
 // A kernel that wants more than 64 KiB of dynamic LDS has to be told so once per device.  `done` is the caller's
 // static bit mask of devices already served for that kernel (a race sets the attribute twice, which is harmless).
 static inline bool bw_allow_big_lds(const void* kernel, uint64_t& done) {

@@ -75,6 +75,8 @@ struct GemvArgs {
     int M, N, K, ldx, ldy;
     int groups, nchunks, row_bytes;
     int x_bf16;                              // x holds bfloat16: every value is rounded to float16 as it is staged
+    int ntiles, nsteps;                      // qgemv_tiles_kernel / qgemv_rounds_kernel: 16-row tiles of N; tiles or rounds per workgroup
+    int meta_lds_off;                        // qgemv_tiles_kernel: where the scale blocks start in LDS
 };
 
 // two bfloat16 -> two float16, round to nearest even (what torch's .to(float16) does)
@@ -226,6 +228,411 @@ __global__ __launch_bounds__((64 * GemvCfg<BITS, GROUP, MT>::MAX_WAVES)) void qg
     }
 }
 
+BW_DEV float half_of(uint32_t word, int hi) {
+    return (float)__builtin_bit_cast(_Float16, (uint16_t)(hi ? word >> 16 : word));
+}
+
+// ---- 3 <= M <= 16, K <= 4096: every request of a workgroup in flight at once ----------------------------------
+//
+// qgemv_kernel re-reads and re-stages its slice of x in every round of every 16-row workgroup, and a wave only
+// has one round of weights requested at a time: with 4 to 16 activation rows the x traffic (from L2) is several
+// times the weight traffic (from HBM) and the rounds serialise on memory latency.  Here K fits one round: wave w
+// of up to 16 owns chunks [w KBW, +KBW) of every row, stages its slice of x once, and then runs the workgroup's
+// NT tiles of 16 rows (tiles b, b + grid, b + 2 grid, ...) against it.  The grid is sized so that every
+// workgroup is resident at once: x is read once per workgroup, not per tile.  Each tile has its own accumulators;
+// the partial sums of the waves meet in LDS once, at the end (in the space of the x tiles, which are dead by then).
+// Scales and zero points of a tile's 16 rows are one contiguous block of each array: the workgroup fetches it with
+// 4-byte requests that cover whole cache lines (a lane fetching its own two bytes costs a cache-line lookup per
+// row and request: sixteen times the lookups of the weights themselves) and passes it on through LDS as (scale,
+// zero point) pairs.
+// The registers that requests land in are not touched until the code that uses them, so every wait sits where
+// the data is needed; nothing is requested under a branch (a request under a branch costs a full wait).
+// What bounds it: a CU keeps a limited number of cache lines requested at once, and a line of x from L2 holds
+// its place for a few hundred cycles, a line of weights from HBM for over a thousand: the x lines of 16
+// activation rows (128 KB per CU at K = 4096) add about 2 us to what the weights alone need.
+template <int BITS, int GROUP, int MT, int NT>
+__global__ __launch_bounds__(1024) void qgemv_tiles_kernel(const GemvArgs a) {
+    using C = GemvCfg<BITS, GROUP, MT>;
+    constexpr int KBW = BITS == 4 ? 2 : (BITS == 8 ? 4 : 1);     // chunks per wave: 256 values of K
+    constexpr int BK = KBW * C::CHUNK_K, PITCH = BK + 8, UPR = BK / C::UNIT, XL = (MT * UPR + 63) / 64;
+    constexpr int X_BYTES = MT * PITCH * 2, UW = C::UNIT / 8;
+    constexpr int kOutPerTile = 16 * MT;
+    constexpr uint32_t kOob = 0x80000000u;
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nwaves = blockDim.x >> 6;
+    const int nl = lane & 15, kq = lane >> 4;
+    const int groups = a.groups, GP = groups | 1;         // odd row pitch: the 16 rows hit different banks
+    // LDS: [x tile of wave 0] ... [x tile of wave n-1][(scale, zero point) pairs: NT blocks of 16 x GP][counter];
+    // at the end the partial sums (NT x waves blocks of MT x 16 floats) take the place of the x tiles
+    _Float16* xs = reinterpret_cast<_Float16*>(smem + wave * X_BYTES);
+    float* red = reinterpret_cast<float*>(smem);
+    uint32_t* meta = reinterpret_cast<uint32_t*>(smem + a.meta_lds_off);
+    const __amdgpu_buffer_rsrc_t rw = make_rsrc(a.qweight, a.w_bytes), rx = make_rsrc(a.x, a.x_bytes),
+                                 rs = make_rsrc(a.scale, a.meta_bytes), rz = make_rsrc(a.zp, a.meta_bytes),
+                                 rb = make_rsrc(a.bias, a.bias ? (uint32_t)a.N * 2 : 0u);   // no bias: every read returns zero
+    auto tile_of = [&](int t) { return (int)blockIdx.x + t * (int)gridDim.x; };
+    auto barrier = [&]() {
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+    };
+
+    // "scales are in LDS" counter: the waves that bring them in count up, the others look before their first tile.
+    // A workgroup barrier there instead would hold every wave until the slowest one has staged its x.
+    uint32_t* ready = meta + NT * 16 * GP;
+    if (tid == 0) *ready = 0u;
+    barrier();
+
+    // ---- requests, small things first (they return in order): scales / zero points of every tile (entries 2 tid,
+    // 2 tid + 1 of each 16 x groups block: K <= 256 * waves, so one 4-byte request per thread covers a block), the
+    // bias of the outputs this thread will store, x, and the weights of the first two tiles; the later tiles'
+    // weights are requested as the tiles before them are worked on (a wave that requests everything first sits in
+    // the request queue until most of it has come back, with its x waiting to be staged)
+    uint32_t ms[NT], mz[NT], bias2[NT];
+#pragma unroll
+    for (int t = 0; t < NT; t++) {
+        uint32_t off = (uint32_t)tile_of(t) * 16 * groups * 2 + tid * 4;
+        asm volatile("" : "+v"(off));                         // a value of its own: the select below stays a select
+        off = (tile_of(t) < a.ntiles && tid < 8 * groups) ? off : kOob;
+        ms[t] = __builtin_amdgcn_raw_buffer_load_b32(rs, off, 0, 0);
+        mz[t] = __builtin_amdgcn_raw_buffer_load_b32(rz, off, 0, 0);
+    }
+    // output o = tid + j * threads of the workgroup's NT * 16 * MT: tile o / (16 MT), row (o / 16) % MT, column o % 16
+#pragma unroll
+    for (int j = 0; j < NT; j++) {
+        const int o = tid + j * (int)blockDim.x, tile = tile_of(o / kOutPerTile);
+        uint32_t off = ((uint32_t)tile * 16 + (o & 15)) * 2 & ~3u;
+        asm volatile("" : "+v"(off));
+        bias2[j] = __builtin_amdgcn_raw_buffer_load_b32(rb, (o < NT * kOutPerTile && tile < a.ntiles) ? off : kOob, 0, 0);
+    }
+    // Every workgroup reads the same x: each starts at a different row, so that the CUs of an XCD are not all
+    // asking the same L2 channel at the same time.
+    const int xrot = (int)(blockIdx.x % XL);
+    u4 xr[XL * UW];
+#pragma unroll
+    for (int j = 0; j < XL; j++) {
+        const int jr = j + xrot < XL ? j + xrot : j + xrot - XL;
+        const int u = lane + 64 * jr, m = u / UPR, k = wave * BK + (u - m * UPR) * C::UNIT;
+        uint32_t off = (uint32_t)(m * a.ldx + k) * 2;
+        asm volatile("" : "+v"(off));
+        off = (m < a.M && k < a.K) ? off : kOob;
+#pragma unroll
+        for (int q = 0; q < UW; q++) xr[j * UW + q] = __builtin_amdgcn_raw_buffer_load_b128(rx, off + q * 16, 0, 0);
+    }
+    asm volatile("" ::: "memory");
+    u4 wr[NT][KBW];
+    auto issue_w = [&](int t) {
+        const uint32_t n = (uint32_t)tile_of(t) * 16 + nl;
+#pragma unroll
+        for (int b = 0; b < KBW; b++) {
+            const int c = wave * KBW + b;
+            uint32_t off = n * a.row_bytes + c * 64 + kq * 16;
+            asm volatile("" : "+v"(off));
+            off = (tile_of(t) < a.ntiles && c < a.nchunks) ? off : kOob;
+            wr[t][b] = __builtin_amdgcn_raw_buffer_load_b128(rw, off, 0, 0);
+        }
+        asm volatile("" ::: "memory");
+    };
+    issue_w(0);
+    if constexpr (NT > 1) issue_w(1);
+
+    // ---- scales / zero points -> LDS as pairs, by the waves whose threads hold entries
+    const int meta_waves = (8 * groups + 63) / 64;
+    if (wave < meta_waves) {                                  // wave-uniform
+#pragma unroll
+        for (int t = 0; t < NT; t++) {
+            uint32_t sv = ms[t], zv = mz[t];
+            asm volatile("" : "+v"(sv), "+v"(zv));            // the wait for them belongs here
+            const int e = 2 * tid;                            // first of the two entries: row e / groups, column e % groups
+            if (e < 16 * groups) {
+                const int r = e / groups, c = e - r * groups; // groups is even: both entries lie in row r
+                uint32_t* dst = meta + t * 16 * GP + r * GP + c;
+                dst[0] = __builtin_amdgcn_perm(zv, sv, 0x05040100u);
+                dst[1] = __builtin_amdgcn_perm(zv, sv, 0x07060302u);
+            }
+        }
+        if (lane == 0) __hip_atomic_fetch_add(ready, 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
+    }
+    // ---- x -> this wave's LDS tile, permuted to the unpack order
+#pragma unroll
+    for (int j = 0; j < XL; j++) {
+        const int jr = j + xrot < XL ? j + xrot : j + xrot - XL;
+        const int u = lane + 64 * jr, m = u / UPR, ku = u - m * UPR;
+        if (m < MT) {
+            uint32_t in[4 * UW], o[4 * UW];
+#pragma unroll
+            for (int q = 0; q < UW; q++) { in[4 * q] = xr[j * UW + q][0]; in[4 * q + 1] = xr[j * UW + q][1]; in[4 * q + 2] = xr[j * UW + q][2]; in[4 * q + 3] = xr[j * UW + q][3]; }
+            if (a.x_bf16) {
+#pragma unroll
+                for (int q = 0; q < 4 * UW; q++) in[q] = bf16x2_to_f16x2(in[q]);
+            }
+            permute_unit<BITS>(in, o);
+            u4* dst = reinterpret_cast<u4*>(xs + m * PITCH + ku * C::UNIT);
+#pragma unroll
+            for (int q = 0; q < UW; q++) dst[q] = u4{o[4 * q], o[4 * q + 1], o[4 * q + 2], o[4 * q + 3]};
+        }
+    }
+    __builtin_amdgcn_wave_barrier();
+    while (__hip_atomic_load(ready, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP) < (uint32_t)meta_waves) __builtin_amdgcn_s_sleep(1);
+
+    // ---- the tiles, as their weights arrive
+    f4 acc[NT][2];
+    const int arow = nl < MT ? nl : MT - 1;              // MFMA rows >= MT repeat a valid row; never stored
+#pragma unroll
+    for (int t = 0; t < NT; t++) {
+        if (t + 2 < NT) issue_w(t + 2);
+        acc[t][0] = acc[t][1] = f4{0.f, 0.f, 0.f, 0.f};
+        const uint32_t* mrow = meta + t * 16 * GP + nl * GP;
+#pragma unroll
+        for (int b = 0; b < KBW; b++) {
+            u4 wv = wr[t][b];
+            asm volatile("" : "+v"(wv));                      // use the registers here and not before
+            // (a chunk may reach past the end of K: those lanes take the row's last groups, their x is zero)
+            const int gb = min(((wave * KBW + b) * C::CHUNK_K + kq * C::VPL) / GROUP, groups - C::NG);
+            GroupConst<BITS> gc[C::NG];
+#pragma unroll
+            for (int g = 0; g < C::NG; g++) {
+                const uint32_t sz = mrow[gb + g];
+                gc[g].set(__builtin_bit_cast(_Float16, (uint16_t)sz), __builtin_bit_cast(_Float16, (uint16_t)(sz >> 16)));
+            }
+            h2 wp[C::VPL / 2];
+            dequant_lane16<BITS, C::NG, !C::POST>(wv, gc, wp);
+            const _Float16* xp = xs + arow * PITCH + b * C::CHUNK_K + kq * C::VPL;
+            if constexpr (C::POST) {
+                f4 part = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int s = 0; s < C::MF; s++)
+                    part = __builtin_amdgcn_mfma_f32_16x16x32_f16(*reinterpret_cast<const h8*>(xp + 8 * s), pack_h8(wp + 4 * s), part, 0, 0, 0);
+                const float sf = (float)gc[0].s[0];
+#pragma unroll
+                for (int q = 0; q < 4; q++) acc[t][b & 1][q] = __builtin_fmaf(sf, part[q], acc[t][b & 1][q]);
+            } else {
+#pragma unroll
+                for (int s = 0; s < C::MF; s++)
+                    acc[t][s & 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(*reinterpret_cast<const h8*>(xp + 8 * s), pack_h8(wp + 4 * s), acc[t][s & 1], 0, 0, 0);
+            }
+        }
+    }
+
+    // ---- partial sums of the waves -> y, all tiles at once: red[(t * waves + w) * MT * 16 + (m / 4) * 64 + n * 4 + m % 4]
+    barrier();                                                // every wave is through with the x tiles
+    if (4 * kq < MT) {
+#pragma unroll
+        for (int t = 0; t < NT; t++) {
+            f4 v;
+#pragma unroll
+            for (int r = 0; r < 4; r++) v[r] = acc[t][0][r] + acc[t][1][r];
+            *reinterpret_cast<f4*>(red + ((t * nwaves + wave) * MT + 4 * kq) * 16 + nl * 4) = v;
+        }
+    }
+    barrier();
+#pragma unroll
+    for (int j = 0; j < NT; j++) {                            // the launch makes the workgroup at least 16 MT threads
+        const int o = tid + j * (int)blockDim.x, t = o / kOutPerTile, m = (o >> 4) % MT, n = tile_of(t) * 16 + (o & 15);
+        uint32_t b2 = bias2[j];
+        asm volatile("" : "+v"(b2));
+        if (o < NT * kOutPerTile) {
+            float v = 0.f;
+            for (int w = 0; w < nwaves; w++) v += red[((t * nwaves + w) * MT + (m & ~3)) * 16 + (o & 15) * 4 + (m & 3)];
+            v += half_of(b2, o & 1);
+            if (m < a.M && n < a.N) a.y[(int64_t)m * a.ldy + n] = (_Float16)v;
+        }
+    }
+}
+
+// ---- 3 <= M <= 16, long K: one 16-row tile per workgroup, rounds of K -------------------------------------------
+//
+// Wave w of up to 16 owns chunks [(r waves + w) KBW, +KBW) of round r.  The weights of DEPTH rounds are requested
+// ahead in registers (all rounds, for the usual shapes; else a ring that is refilled as it drains); x is restaged
+// per round into the wave's own LDS tile.  The tile's whole block of scales and zero points comes in once, at
+// the start, as in qgemv_tiles_kernel.
+template <int BITS, int GROUP, int MT, int DEPTH, bool LOOP>
+__global__ __launch_bounds__(1024) void qgemv_rounds_kernel(const GemvArgs a) {
+    using C = GemvCfg<BITS, GROUP, MT>;
+    constexpr int KBW = BITS == 4 ? 2 : (BITS == 8 ? 4 : 1);     // chunks per wave and round: 256 values of K
+    constexpr int BK = KBW * C::CHUNK_K, PITCH = BK + 8, UPR = BK / C::UNIT, XL = (MT * UPR + 63) / 64;
+    constexpr int X_BYTES = MT * PITCH * 2, UW = C::UNIT / 8;
+    constexpr int ME = 4;                                 // 4-byte requests (two entries) per thread for the scale block
+    constexpr uint32_t kOob = 0x80000000u;
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nwaves = blockDim.x >> 6;
+    const int nl = lane & 15, kq = lane >> 4;
+    const int groups = a.groups, GP = groups | 1;         // odd row pitch: the 16 rows hit different banks
+    const int tile = (int)blockIdx.x, nsteps = a.nsteps;
+    // LDS: [x tile of wave 0] ... [x tile of wave n-1][partial sums, one MT x 16 block per wave][(scale, zero point)]
+    _Float16* xs = reinterpret_cast<_Float16*>(smem + wave * X_BYTES);
+    float* red = reinterpret_cast<float*>(smem + nwaves * X_BYTES);
+    uint32_t* meta = reinterpret_cast<uint32_t*>(smem + nwaves * (X_BYTES + MT * 64));
+    const __amdgpu_buffer_rsrc_t rw = make_rsrc(a.qweight, a.w_bytes), rx = make_rsrc(a.x, a.x_bytes),
+                                 rs = make_rsrc(a.scale, a.meta_bytes), rz = make_rsrc(a.zp, a.meta_bytes),
+                                 rb = make_rsrc(a.bias, a.bias ? (uint32_t)a.N * 2 : 0u);   // no bias: every read returns zero
+    // the next round's x is requested before this round's arithmetic where the registers allow (16 rows of x in
+    // flight plus three rounds of weights do not fit 128 registers), else right behind it
+    constexpr bool XPRE = MT < 16;
+
+    u4 xr[XL * UW];
+    u4 wr[DEPTH][KBW];
+    uint32_t ms[ME], mz[ME];
+    auto issue_x = [&](int i) {
+        const int k0 = (i * nwaves + wave) * BK;
+#pragma unroll
+        for (int j = 0; j < XL; j++) {
+            const int u = lane + 64 * j, m = u / UPR, k = k0 + (u - m * UPR) * C::UNIT;
+            uint32_t off = (uint32_t)(m * a.ldx + k) * 2;
+            asm volatile("" : "+v"(off));                     // a value of its own: the select below stays a select
+            off = (i < nsteps && m < a.M && k < a.K) ? off : kOob;
+#pragma unroll
+            for (int q = 0; q < UW; q++) xr[j * UW + q] = __builtin_amdgcn_raw_buffer_load_b128(rx, off + q * 16, 0, 0);
+        }
+        asm volatile("" ::: "memory");
+    };
+    auto issue_w = [&](int d, int i) {
+        const int c0 = (i * nwaves + wave) * KBW;
+        const uint32_t n = (uint32_t)tile * 16 + nl;
+#pragma unroll
+        for (int b = 0; b < KBW; b++) {
+            uint32_t off = n * a.row_bytes + (c0 + b) * 64 + kq * 16;
+            asm volatile("" : "+v"(off));
+            off = (i < nsteps && c0 + b < a.nchunks) ? off : kOob;
+            wr[d][b] = __builtin_amdgcn_raw_buffer_load_b128(rw, off, 0, 0);
+        }
+        asm volatile("" ::: "memory");
+    };
+    auto stage_x = [&]() {
+#pragma unroll
+        for (int j = 0; j < XL; j++) {
+            const int u = lane + 64 * j, m = u / UPR, ku = u - m * UPR;
+            if (m < MT) {
+                uint32_t in[4 * UW], o[4 * UW];
+#pragma unroll
+                for (int q = 0; q < UW; q++) { in[4 * q] = xr[j * UW + q][0]; in[4 * q + 1] = xr[j * UW + q][1]; in[4 * q + 2] = xr[j * UW + q][2]; in[4 * q + 3] = xr[j * UW + q][3]; }
+                if (a.x_bf16) {
+#pragma unroll
+                    for (int q = 0; q < 4 * UW; q++) in[q] = bf16x2_to_f16x2(in[q]);
+                }
+                permute_unit<BITS>(in, o);
+                u4* dst = reinterpret_cast<u4*>(xs + m * PITCH + ku * C::UNIT);
+#pragma unroll
+                for (int q = 0; q < UW; q++) dst[q] = u4{o[4 * q], o[4 * q + 1], o[4 * q + 2], o[4 * q + 3]};
+            }
+        }
+    };
+    auto barrier = [&]() {
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+    };
+
+    // ---- requests, small things first (they return in order): the tile's scales and zero points (entries 2 e,
+    // 2 e + 1 of its 16 x groups block for e = tid, tid + threads, ...), its bias, x of round 0, the weights
+    const uint32_t mbase = (uint32_t)tile * 16 * groups * 2;
+#pragma unroll
+    for (int j = 0; j < ME; j++) {
+        const int e = tid + j * (int)blockDim.x;
+        uint32_t off = mbase + e * 4;
+        asm volatile("" : "+v"(off));
+        off = e < 8 * groups ? off : kOob;
+        ms[j] = __builtin_amdgcn_raw_buffer_load_b32(rs, off, 0, 0);
+        mz[j] = __builtin_amdgcn_raw_buffer_load_b32(rz, off, 0, 0);
+    }
+    uint32_t bias2 = __builtin_amdgcn_raw_buffer_load_b32(rb, ((uint32_t)tile * 16 + nl) * 2 & ~3u, 0, 0);
+    issue_x(0);
+#pragma unroll
+    for (int d = 0; d < DEPTH; d++) issue_w(d, d);
+    // scales / zero points -> LDS as pairs
+#pragma unroll
+    for (int j = 0; j < ME; j++) {
+        const int e = 2 * (tid + j * (int)blockDim.x);        // first of the two entries: row e / groups, column e % groups
+        uint32_t sv = ms[j], zv = mz[j];
+        asm volatile("" : "+v"(sv), "+v"(zv));                // the wait for them belongs here
+        if (e < 16 * groups) {
+            const int r = e / groups, c = e - r * groups;     // groups is even: both entries lie in row r
+            meta[r * GP + c] = __builtin_amdgcn_perm(zv, sv, 0x05040100u);
+            meta[r * GP + c + 1] = __builtin_amdgcn_perm(zv, sv, 0x07060302u);
+        }
+    }
+    barrier();
+
+    f4 acc[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
+    const int arow = nl < MT ? nl : MT - 1;              // MFMA rows >= MT repeat a valid row; never stored
+    const uint32_t* mrow = meta + nl * GP;
+    // one round from ring slot d; false = past the last round
+    auto run_step = [&](int d, int i) -> bool {
+        if (i >= nsteps) return false;                        // uniform over the workgroup
+        if (i > 0) __builtin_amdgcn_wave_barrier();           // the reads of the round before are done
+        stage_x();
+        __builtin_amdgcn_wave_barrier();
+        if constexpr (XPRE) issue_x(i + 1);                   // past the last round: range-checked to nothing
+        const int c0 = (i * nwaves + wave) * KBW;
+#pragma unroll
+        for (int b = 0; b < KBW; b++) {
+            u4 wv = wr[d][b];
+            asm volatile("" : "+v"(wv));                      // use the round's registers here and not before
+            // (a chunk may reach past the end of K: those lanes take the row's last groups, their x is zero)
+            const int gb = min(((c0 + b) * C::CHUNK_K + kq * C::VPL) / GROUP, groups - C::NG);
+            GroupConst<BITS> gc[C::NG];
+#pragma unroll
+            for (int g = 0; g < C::NG; g++) {
+                const uint32_t sz = mrow[gb + g];
+                gc[g].set(__builtin_bit_cast(_Float16, (uint16_t)sz), __builtin_bit_cast(_Float16, (uint16_t)(sz >> 16)));
+            }
+            h2 wp[C::VPL / 2];
+            dequant_lane16<BITS, C::NG, !C::POST>(wv, gc, wp);
+            const _Float16* xp = xs + arow * PITCH + b * C::CHUNK_K + kq * C::VPL;
+            if constexpr (C::POST) {
+                f4 part = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int s = 0; s < C::MF; s++)
+                    part = __builtin_amdgcn_mfma_f32_16x16x32_f16(*reinterpret_cast<const h8*>(xp + 8 * s), pack_h8(wp + 4 * s), part, 0, 0, 0);
+                const float sf = (float)gc[0].s[0];
+#pragma unroll
+                for (int q = 0; q < 4; q++) acc[b & 1][q] = __builtin_fmaf(sf, part[q], acc[b & 1][q]);
+            } else {
+#pragma unroll
+                for (int s = 0; s < C::MF; s++)
+                    acc[s & 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(*reinterpret_cast<const h8*>(xp + 8 * s), pack_h8(wp + 4 * s), acc[s & 1], 0, 0, 0);
+            }
+        }
+        if constexpr (!XPRE) {
+            __builtin_amdgcn_wave_barrier();                  // the round's reads of the x tile are done
+            issue_x(i + 1);
+        }
+        if constexpr (LOOP) issue_w(d, i + DEPTH);            // refill the slot
+        return true;
+    };
+    if constexpr (LOOP) {
+        for (int i0 = 0; i0 < nsteps; i0 += DEPTH) {
+            bool more = true;
+#pragma unroll
+            for (int d = 0; d < DEPTH; d++) more = more && run_step(d, i0 + d);
+            if (!more) break;
+        }
+    } else {
+        // at most DEPTH rounds: straight code, every wait count exact, nothing requested that is not used
+        bool more = true;
+#pragma unroll
+        for (int d = 0; d < DEPTH; d++) more = more && run_step(d, d);
+    }
+
+    // partial sums of the waves -> y
+    if (4 * kq < MT) {
+#pragma unroll
+        for (int r = 0; r < 4; r++)
+            if (4 * kq + r < MT) red[(wave * MT + 4 * kq + r) * 16 + nl] = acc[0][r] + acc[1][r];
+    }
+    asm volatile("" : "+v"(bias2));
+    barrier();
+    if (tid < 16 * MT) {                                      // the launch makes the workgroup at least this large
+        const int m = tid >> 4, n = tile * 16 + nl;
+        if (m < a.M && n < a.N) {
+            float v = 0.f;
+            for (int w = 0; w < nwaves; w++) v += red[(w * MT + m) * 16 + nl];
+            v += half_of(bias2, nl & 1);
+            a.y[(int64_t)m * a.ldy + n] = (_Float16)v;
+        }
+    }
+}
+
 // ---- 4-bit, M <= 2: integer operands, scale and zero point taken out of the inner loop -------------------
 //
 // A masked packed word is already a float16: bits 0-3 of a half are the subnormal q * 2^-24, bits 4-7 the
@@ -242,9 +649,6 @@ __global__ __launch_bounds__((64 * GemvCfg<BITS, GROUP, MT>::MAX_WAVES)) void qg
 // the partial sum of group g alone and gets that group's scale and zero point.
 // Results agree with the per-weight float16 dequantisation to float32 rounding: a one-hot x still returns
 // the reference's W16 column bit for bit.
-BW_DEV float half_of(uint32_t word, int hi) {
-    return (float)__builtin_bit_cast(_Float16, (uint16_t)(hi ? word >> 16 : word));
-}
 
 // sum over aligned runs of LANES (4, 8 or 16) lanes; every lane of a run ends up with the run's total
 template <int LANES>
@@ -716,6 +1120,85 @@ int launch_w2(const GemvArgs& a, hipStream_t stream) {
 
 constexpr int kLdsBudget = 150 * 1024;
 
+template <int BITS, int GROUP, int MT, int NT>
+int launch_tiles_nt(const GemvArgs& a, int grid, int nwaves, size_t lds, hipStream_t stream) {
+    auto kern = qgemv_tiles_kernel<BITS, GROUP, MT, NT>;
+    static uint64_t big_lds_devices = 0;                   // per instantiation
+    if (lds > 64 * 1024 && !bw_allow_big_lds(reinterpret_cast<const void*>(kern), big_lds_devices)) return BW_ELAUNCH;
+    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(nwaves * 64), lds, stream, a);
+    return hipGetLastError() == hipSuccess ? BW_OK : BW_ELAUNCH;
+}
+
+template <int BITS, int GROUP, int MT, int DEPTH, bool LOOP>
+int launch_rounds_depth(const GemvArgs& a, int grid, int nwaves, size_t lds, hipStream_t stream) {
+    auto kern = qgemv_rounds_kernel<BITS, GROUP, MT, DEPTH, LOOP>;
+    static uint64_t big_lds_devices = 0;                   // per instantiation
+    if (lds > 64 * 1024 && !bw_allow_big_lds(reinterpret_cast<const void*>(kern), big_lds_devices)) return BW_ELAUNCH;
+    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(nwaves * 64), lds, stream, a);
+    return hipGetLastError() == hipSuccess ? BW_OK : BW_ELAUNCH;
+}
+
+// 3 <= M <= 16 through qgemv_tiles_kernel (K fits one round of a workgroup) or qgemv_rounds_kernel.
+// BW_EUNSUPPORTED = this layout is not taken (scale arrays that 4-byte requests cannot address, a scale block that
+// does not fit LDS, short K, more rounds than the registers hold); the caller falls back to qgemv_kernel
+template <int BITS, int GROUP, int MT>
+int launch_tiles(GemvArgs a, hipStream_t stream) {
+    using C = GemvCfg<BITS, GROUP, MT>;
+    constexpr int KBW = BITS == 4 ? 2 : (BITS == 8 ? 4 : 1);
+    constexpr int X_BYTES = MT * (KBW * C::CHUNK_K + 8) * 2;
+    constexpr size_t kLds = 160 * 1024;
+    // 4-byte requests for scales, zero points and bias: aligned arrays, an even number of entries per row
+    if (!bw_aligned(a.scale, 4) || !bw_aligned(a.zp, 4) || a.groups % 2 || (a.bias && (!bw_aligned(a.bias, 4) || a.N % 2)))
+        return BW_EUNSUPPORTED;
+    const size_t meta_lds = (size_t)16 * (a.groups | 1) * 4;
+    int nwaves = (a.nchunks + KBW - 1) / KBW;
+    if (nwaves > 16) nwaves = 16;
+    while (nwaves > 1 && (size_t)nwaves * (X_BYTES + MT * 64) + meta_lds > kLds) nwaves--;
+    const int rounds = (a.nchunks + nwaves * KBW - 1) / (nwaves * KBW);
+    if (nwaves * 64 < 16 * MT) return BW_EUNSUPPORTED;
+    a.ntiles = (a.N + 15) / 16;
+    if (rounds == 1) {
+        // every workgroup resident at once (a CU holds 16 waves of this kernel: up to 128 registers each), each
+        // running up to NTMAX tiles
+        constexpr int NTMAX = BITS == 8 ? (MT == 16 ? 2 : 3) : 4;
+        const int slots = bw_device_cus() * (16 / nwaves);
+        int nt = (a.ntiles + slots - 1) / slots;
+        if (nt > NTMAX) nt = NTMAX;
+        size_t xred;
+        while (true) {
+            xred = (size_t)nwaves * X_BYTES;                                     // x tiles, later the partial sums
+            if (xred < (size_t)nt * nwaves * MT * 64) xred = (size_t)nt * nwaves * MT * 64;
+            if (xred + nt * meta_lds + 16 <= kLds || nt == 1) break;
+            nt--;
+        }
+        const size_t lds = xred + nt * meta_lds + 16;                            // + the "scales are in LDS" counter
+        if (lds > kLds) return BW_EUNSUPPORTED;
+        const int grid = (a.ntiles + nt - 1) / nt;
+        a.meta_lds_off = (int)xred;
+        a.nsteps = nt;
+        if (nt == 1) return launch_tiles_nt<BITS, GROUP, MT, 1>(a, grid, nwaves, lds, stream);
+        if (nt == 2) return launch_tiles_nt<BITS, GROUP, MT, 2>(a, grid, nwaves, lds, stream);
+        if constexpr (NTMAX >= 3)
+            if (nt == 3) return launch_tiles_nt<BITS, GROUP, MT, 3>(a, grid, nwaves, lds, stream);
+        if constexpr (NTMAX >= 4)
+            if (nt == 4) return launch_tiles_nt<BITS, GROUP, MT, 4>(a, grid, nwaves, lds, stream);
+        return BW_EUNSUPPORTED;
+    }
+    // rounds: the tile's whole scale block comes in with at most four 4-byte requests per thread
+    const size_t lds = (size_t)nwaves * (X_BYTES + MT * 64) + meta_lds;
+    if (lds > kLds || 8 * a.groups > 4 * nwaves * 64) return BW_EUNSUPPORTED;
+    a.nsteps = rounds;
+    // Rounds a workgroup keeps requested ahead: all of them while they fit the 128 registers a wave of a 16-wave
+    // workgroup has (8-bit rounds are four 16-byte loads per lane), else a ring of two where that fits.
+    constexpr int RMAX = (BITS == 8 && MT >= 8) ? 2 : 3;
+    constexpr bool RRING = BITS != 8 && MT < 16;
+    if (rounds == 2) return launch_rounds_depth<BITS, GROUP, MT, 2, false>(a, a.ntiles, nwaves, lds, stream);
+    if constexpr (RMAX >= 3)
+        if (rounds == 3) return launch_rounds_depth<BITS, GROUP, MT, 3, false>(a, a.ntiles, nwaves, lds, stream);
+    if constexpr (RRING) return launch_rounds_depth<BITS, GROUP, MT, 2, true>(a, a.ntiles, nwaves, lds, stream);
+    return BW_EUNSUPPORTED;
+}
+
 template <int BITS, int GROUP, int MT, int KB>
 int launch_gemv_kb(const GemvArgs& a, hipStream_t stream) {
     using C = GemvCfg<BITS, GROUP, MT>;
@@ -772,6 +1255,12 @@ int launch_gemv(const GemvArgs& a, hipStream_t stream) {
         }
     }
     if (a.M == 1) return launch_gemv_mt<BITS, GROUP, 1>(a, stream);
+    static const bool old_path = getenv("BW_OLD_GEMV") != nullptr;
+    if (a.M > 2 && !old_path) {
+        const int st = a.M <= 4 ? launch_tiles<BITS, GROUP, 4>(a, stream)
+                                : (a.M <= 8 ? launch_tiles<BITS, GROUP, 8>(a, stream) : launch_tiles<BITS, GROUP, 16>(a, stream));
+        if (st != BW_EUNSUPPORTED) return st;
+    }
     if (a.M <= 4) return launch_gemv_mt<BITS, GROUP, 4>(a, stream);
     if (a.M <= 8) return launch_gemv_mt<BITS, GROUP, 8>(a, stream);
     return launch_gemv_mt<BITS, GROUP, 16>(a, stream);
