@@ -1174,6 +1174,9 @@ int launch_tiles(GemvArgs a, hipStream_t stream) {
         const size_t lds = xred + nt * meta_lds + 16;                            // + the "scales are in LDS" counter
         if (lds > kLds) return BW_EUNSUPPORTED;
         const int grid = (a.ntiles + nt - 1) / nt;
+        // 8 bits (four 16-byte loads per lane and tile, so fewer tiles fit the registers): measured to pay only
+        // with more than one tile per workgroup and every workgroup resident
+        if (BITS == 8 && (nt < 2 || grid > slots)) return BW_EUNSUPPORTED;
         a.meta_lds_off = (int)xred;
         a.nsteps = nt;
         if (nt == 1) return launch_tiles_nt<BITS, GROUP, MT, 1>(a, grid, nwaves, lds, stream);
@@ -1237,8 +1240,27 @@ int launch_gemv_mt(const GemvArgs& a, hipStream_t stream) {
     return launch_gemv_kb<BITS, GROUP, MT, 1>(a, stream);
 }
 
+// Rows from which qgemv_tiles_kernel (K fits one round: at most 16 * KBW chunks) or qgemv_rounds_kernel beats
+// the kernels below, from timing the Llama-shaped layers on MI355X (4096 x 4096, 4096 -> 11008, 11008 -> 4096) at
+// M = 1, 2, 4, 8, 16; 99 = never.  The formats with a subnormal-operand kernel keep it for M <= 2 where that wins;
+// long rows pay more per round for x than qgemv_kernel's smaller rounds do, so 4-bit at groups of 64 and 128 and
+// 8-bit stay there.
+template <int BITS, int GROUP>
+int tiles_min_rows(int nchunks) {
+    constexpr int KBW = BITS == 4 ? 2 : (BITS == 8 ? 4 : 1);
+    const bool one_round = nchunks <= 16 * KBW;
+    if (BITS == 8) return one_round ? 2 : 99;
+    if (BITS == 4) return GROUP == 128 ? (one_round ? 3 : 99) : GROUP == 64 ? (one_round ? 2 : 99) : (one_round ? 1 : 2);
+    return GROUP == 32 ? 1 : (one_round ? (GROUP == 64 ? 1 : 2) : 3);
+}
+
 template <int BITS, int GROUP>
 int launch_gemv(const GemvArgs& a, hipStream_t stream) {
+    if (a.M >= tiles_min_rows<BITS, GROUP>(a.nchunks)) {
+        const int st = a.M <= 4 ? launch_tiles<BITS, GROUP, 4>(a, stream)
+                                : (a.M <= 8 ? launch_tiles<BITS, GROUP, 8>(a, stream) : launch_tiles<BITS, GROUP, 16>(a, stream));
+        if (st != BW_EUNSUPPORTED) return st;
+    }
     if constexpr (BITS == 4) {
         // rows of the MFMA tile in use = M * groups per chunk, at most 4.  With groups of 64 the doubled
         // activation rows cost more than the cheaper unpack saves until the weights reach about 16 MiB.
@@ -1255,12 +1277,6 @@ int launch_gemv(const GemvArgs& a, hipStream_t stream) {
         }
     }
     if (a.M == 1) return launch_gemv_mt<BITS, GROUP, 1>(a, stream);
-    static const bool old_path = getenv("BW_OLD_GEMV") != nullptr;
-    if (a.M > 2 && !old_path) {
-        const int st = a.M <= 4 ? launch_tiles<BITS, GROUP, 4>(a, stream)
-                                : (a.M <= 8 ? launch_tiles<BITS, GROUP, 8>(a, stream) : launch_tiles<BITS, GROUP, 16>(a, stream));
-        if (st != BW_EUNSUPPORTED) return st;
-    }
     if (a.M <= 4) return launch_gemv_mt<BITS, GROUP, 4>(a, stream);
     if (a.M <= 8) return launch_gemv_mt<BITS, GROUP, 8>(a, stream);
     return launch_gemv_mt<BITS, GROUP, 16>(a, stream);
