@@ -700,12 +700,9 @@ extern "C" int bw_qgemm_ws(const void* x, int act_dtype, int64_t M, int64_t K, i
     hipStream_t st = (hipStream_t)stream;
 #define BW_CASE(B, G) \
     if (bits == B && group == G) return launch_gemm<B, G>(a, workspace, workspace_bytes, st);
-    BW_CASE(4, 128)
-#ifndef BW_FAST_BUILD
-    BW_CASE(4, 64) BW_CASE(4, 32)
+    BW_CASE(4, 128) BW_CASE(4, 64) BW_CASE(4, 32)
     BW_CASE(8, 128) BW_CASE(8, 64) BW_CASE(8, 32)
     BW_CASE(2, 128) BW_CASE(2, 64) BW_CASE(2, 32)
-#endif
 #undef BW_CASE
     return BW_EUNSUPPORTED;
 }
