@@ -16,6 +16,8 @@
 // apply (odd K or group size): correct for everything the reference accepts.
 #include "bw_common.h"
 
+#include <atomic>
+
 bool bw_fast_shape(int64_t M, int64_t N, int64_t K, int64_t ldx, int bits, int group);
 
 namespace {
@@ -705,6 +707,30 @@ extern "C" int bw_qgemm_ws(const void* x, int act_dtype, int64_t M, int64_t K, i
     BW_CASE(2, 128) BW_CASE(2, 64) BW_CASE(2, 32)
 #undef BW_CASE
     return BW_EUNSUPPORTED;
+}
+
+// ---- the same without a caller's workspace: the split-K partial tiles go to a device array of the library ----
+// For callers that cannot allocate (code under graph capture, serving loops, harnesses that forbid it).  The array
+// is one per GPU, shared by every call on that GPU and kept for the life of the process.
+constexpr size_t kScratchBytes = (size_t)32 << 20;       // 256 partial tiles of 128 x 256 floats: one full round
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+constexpr int kMaxDevices = 64;
+static std::atomic<void*> g_scratch_ptr[kMaxDevices];    // device address of `scratch` on each GPU, looked up once
+
+extern "C" int bw_qgemm_static(const void* x, int act_dtype, int64_t M, int64_t K, int64_t ldx, const int32_t* qweight,
+                               const void* scale16, const void* zp16, const void* bias, int64_t N, int bits, int group,
+                               void* y, int64_t ldy, void* stream) {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return BW_ELAUNCH;
+    void* ptr = g_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (!ptr) {
+        // `scratch` names the array in host code only as a handle: its memory on the current device is at the
+        // address this returns (each GPU holds its own copy at its own address)
+        if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess || !ptr) return BW_ELAUNCH;
+        g_scratch_ptr[dev].store(ptr, std::memory_order_release);
+    }
+    if (bw_qgemm_workspace_bytes(M, N, K, bits, group) > kScratchBytes) return BW_EWORKSPACE;
+    return bw_qgemm_ws(x, act_dtype, M, K, ldx, qweight, scale16, zp16, bias, N, bits, group, y, ldy, ptr, kScratchBytes, stream);
 }
 
 extern "C" int bw_qgemm(const void* x, int act_dtype, int64_t M, int64_t K, int64_t ldx, const int32_t* qweight,

@@ -461,7 +461,7 @@ extern "C" int bw_dequantize(const int32_t* qweight, const void* scale, int scal
     return BW_EINVAL;
 }
 
-extern "C" int bw_abi_version(void) { return 5; }
+extern "C" int bw_abi_version(void) { return 6; }
 
 extern "C" const char* bw_strerror(int status) {
     switch (status) {

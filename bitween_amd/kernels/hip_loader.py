@@ -19,9 +19,9 @@ _lib = None
 BW_F16, BW_BF16, BW_F32, BW_I32 = 0, 1, 2, 3
 _DTYPE_CODE = {torch.float16: BW_F16, torch.bfloat16: BW_BF16, torch.float32: BW_F32, torch.int32: BW_I32}
 
-ABI_VERSION = 5            # what bw_abi_version() of a matching library returns
+ABI_VERSION = 6            # what bw_abi_version() of a matching library returns
 ENTRY_POINTS = ("bw_abi_version", "bw_strerror", "bw_quantize_pack", "bw_quantize_pack_add", "bw_dequantize", "bw_qgemv", "bw_qgemm",
-                "bw_qgemm_ws", "bw_qgemm_workspace_bytes", "bw_qlinear", "bw_qdgrad", "bw_qdgrad_workspace_bytes", "bw_cast_bf16_f16", "bw_qlinear_decode_rows")
+                "bw_qgemm_ws", "bw_qgemm_static", "bw_qgemm_workspace_bytes", "bw_qlinear", "bw_qdgrad", "bw_qdgrad_workspace_bytes", "bw_cast_bf16_f16", "bw_qlinear_decode_rows")
 
 
 class BitweenHipError(RuntimeError):
@@ -53,7 +53,7 @@ def load():
     lib.bw_quantize_pack_add.argtypes = [vp, vp, i32, i32, i64, i64, i64, i64, i32, i32, vp, vp, i32, vp, i32, vp]
     lib.bw_dequantize.argtypes = [vp, vp, i32, vp, i32, i64, i64, i32, i32, vp, i32, i64, vp]
     mm = [vp, i32, i64, i64, i64, vp, vp, vp, vp, i64, i32, i32, vp, i64, vp]
-    for name in ("bw_qgemv", "bw_qgemm", "bw_qlinear"):
+    for name in ("bw_qgemv", "bw_qgemm", "bw_qlinear", "bw_qgemm_static"):
         getattr(lib, name).argtypes = mm
     lib.bw_qgemm_ws.argtypes = mm[:-1] + [vp, ctypes.c_size_t, vp]
     lib.bw_qgemm_workspace_bytes.argtypes = [i64, i64, i64, i32, i32]
@@ -66,7 +66,7 @@ def load():
     lib.bw_cast_bf16_f16.restype = i32
     lib.bw_qlinear_decode_rows.argtypes = [i64, i64, i32]
     lib.bw_qlinear_decode_rows.restype = i32
-    for name in ("bw_quantize_pack", "bw_quantize_pack_add", "bw_dequantize", "bw_qgemv", "bw_qgemm", "bw_qgemm_ws", "bw_qlinear"):
+    for name in ("bw_quantize_pack", "bw_quantize_pack_add", "bw_dequantize", "bw_qgemv", "bw_qgemm", "bw_qgemm_ws", "bw_qgemm_static", "bw_qlinear"):
         getattr(lib, name).restype = i32
     for name in ("bw_qgemv", "bw_qgemm", "bw_qlinear"):
         _ENTRY[name] = getattr(lib, name)

@@ -120,6 +120,18 @@ int bw_qgemm_ws(const void* x, int act_dtype, int64_t M, int64_t K, int64_t ldx,
                 int64_t N, int bits, int group, void* y, int64_t ldy,
                 void* workspace, size_t workspace_bytes, void* stream);
 
+/* bw_qgemm_ws without a workspace argument and without any allocation: the split-K partial tiles go to a device
+ * array that the library itself holds (32 MiB per GPU that the library runs on, kept until the process ends),
+ * so results are those of bw_qgemm_ws, bit for bit.  No counterpart in the reference; it is for callers that
+ * cannot allocate: code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.
+ * The first call on a device looks up the array's address there (hipGetSymbolAddress); no call allocates,
+ * frees or synchronises.  A shape whose partial tiles exceed the array returns BW_EWORKSPACE (none does on a
+ * 256-CU device).  Every call on a GPU shares that GPU's array: calls that overlap in time on one GPU (two
+ * streams, two threads) race on it - serialise them or use bw_qgemm_ws with a workspace per stream. */
+int bw_qgemm_static(const void* x, int act_dtype, int64_t M, int64_t K, int64_t ldx,
+                    const int32_t* qweight, const void* scale16, const void* zp16, const void* bias,
+                    int64_t N, int bits, int group, void* y, int64_t ldy, void* stream);
+
 int bw_qlinear_decode_rows(int64_t N, int64_t K, int bits);
 
 int bw_qlinear(const void* x, int act_dtype, int64_t M, int64_t K, int64_t ldx,
