@@ -60,10 +60,14 @@ BW_DEV void load_vals(const void* w, int64_t off, float* v) {
     }
 }
 
-// scale and zero point of one group from its extrema, exactly as functional.py:25-26
+// scale and zero point of one group from its extrema, exactly as functional.py:25-26.  The division by the
+// Python scalar Qmax is a true division in eager torch on the CPU; on a GPU torch multiplies by the float32
+// reciprocal of a scalar divisor instead (one float32 rounding of the product, then the tensor's type), which
+// differs in the last bit of most float32 scales: `recip` selects that arithmetic.
 template <int MATH>
-BW_DEV void group_params(float lo, float hi, float qmax, float& s, float& zf) {
-    s = rnd<MATH>(__fdiv_rn(rnd<MATH>(__fsub_rn(hi, lo)), qmax));
+BW_DEV void group_params(float lo, float hi, float qmax, bool recip, float& s, float& zf) {
+    const float range = rnd<MATH>(__fsub_rn(hi, lo));
+    s = rnd<MATH>(recip ? __fmul_rn(range, __fdiv_rn(1.0f, qmax)) : __fdiv_rn(range, qmax));
     s = fmaxf(s, rnd<MATH>(1e-8f));
     zf = rintf(rnd<MATH>(__fdiv_rn(-lo, s)));
     zf = fminf(fmaxf(zf, 0.f), qmax);
@@ -89,7 +93,7 @@ __global__ __launch_bounds__(256) void quantize_pack_kernel(const void* __restri
                                                             int64_t N, int K, int64_t ldw, int64_t ldd,
                                                             int group, int lpg, int32_t* __restrict__ qweight,
                                                             void* __restrict__ scale, int scale_dtype,
-                                                            void* __restrict__ zp, int zp_dtype) {
+                                                            void* __restrict__ zp, int zp_dtype, int recip) {
     constexpr int VPI = 32 / BITS, VPT = VPI * WPT;
     constexpr float QMAX = (float)((1 << BITS) - 1);
     const int tpr = K / VPT;                             // threads per row; grid.x covers them, grid.y the rows
@@ -116,7 +120,7 @@ __global__ __launch_bounds__(256) void quantize_pack_kernel(const void* __restri
             hi = fmaxf(hi, __shfl_xor(hi, d));
         }
         float s, zf;
-        group_params<MATH>(lo, hi, QMAX, s, zf);
+        group_params<MATH>(lo, hi, QMAX, recip != 0, s, zf);
         float t[VPT];
         if constexpr (MATH == BW_F32) {
             const float r0 = __builtin_amdgcn_rcpf(s);
@@ -166,7 +170,7 @@ __global__ __launch_bounds__(256) void quantize_pack_generic_kernel(const void* 
                                                                     int64_t N, int K, int64_t ldw, int64_t ldd,
                                                                     int bits, int group, int32_t* __restrict__ qweight,
                                                                     void* __restrict__ scale, int scale_dtype,
-                                                                    void* __restrict__ zp, int zp_dtype) {
+                                                                    void* __restrict__ zp, int zp_dtype, int recip) {
     const int vpi = 32 / bits, words = K / vpi, groups = K / group;
     const float qmax = (float)((1 << bits) - 1);
     const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -190,7 +194,7 @@ __global__ __launch_bounds__(256) void quantize_pack_generic_kernel(const void* 
                 lo = fminf(lo, x);
                 hi = fmaxf(hi, x);
             }
-            group_params<MATH>(lo, hi, qmax, s, zf);
+            group_params<MATH>(lo, hi, qmax, recip != 0, s, zf);
             gprev = g;
             if (k == g * group) {                        // the thread holding a group's first value stores its parameters
                 store_meta(scale, scale_dtype, row * groups + g, s);
@@ -348,40 +352,40 @@ bool quantize_fits(const void* w, const void* delta, int64_t K, int64_t ldw, int
 
 template <int BITS, int WDT, int MATH, int WPT>
 int launch_quantize(const void* w, const void* delta, int64_t N, int64_t K, int64_t ldw, int64_t ldd, int group,
-                    int32_t* qweight, void* scale, int sdt, void* zp, int zdt, hipStream_t st) {
+                    int32_t* qweight, void* scale, int sdt, void* zp, int zdt, int recip, hipStream_t st) {
     constexpr int VPT = 32 / BITS * WPT;
     const int tpr = (int)(K / VPT);
     const int block = tpr >= 256 ? 256 : ((tpr + 63) / 64) * 64;
     dim3 grid((unsigned)((tpr + block - 1) / block), (unsigned)(N < 65535 ? N : 65535));
     hipLaunchKernelGGL((quantize_pack_kernel<BITS, WDT, MATH, WPT>), grid, dim3(block), 0, st, w, delta, N, (int)K, ldw, ldd,
-                       group, group / VPT, qweight, scale, sdt, zp, zdt);
+                       group, group / VPT, qweight, scale, sdt, zp, zdt, recip);
     return hipGetLastError() == hipSuccess ? BW_OK : BW_ELAUNCH;
 }
 
 template <int BITS, int WDT, int MATH>
 int launch_quantize_bits(const void* w, const void* delta, int64_t N, int64_t K, int64_t ldw, int64_t ldd, int group,
-                         int32_t* qweight, void* scale, int sdt, void* zp, int zdt, hipStream_t st) {
+                         int32_t* qweight, void* scale, int sdt, void* zp, int zdt, int recip, hipStream_t st) {
     // 32 bytes of input per thread where the shape allows, else one word per thread, else the generic kernel
     constexpr int VPI = 32 / BITS;
     constexpr int WIDE = (WDT == BW_F32 ? 8 : 16) / VPI;
     if constexpr (WIDE > 1) {
         if (quantize_fits<BITS, WDT, WIDE>(w, delta, K, ldw, ldd, group, qweight))
-            return launch_quantize<BITS, WDT, MATH, WIDE>(w, delta, N, K, ldw, ldd, group, qweight, scale, sdt, zp, zdt, st);
+            return launch_quantize<BITS, WDT, MATH, WIDE>(w, delta, N, K, ldw, ldd, group, qweight, scale, sdt, zp, zdt, recip, st);
     }
     if (quantize_fits<BITS, WDT, 1>(w, delta, K, ldw, ldd, group, qweight))
-        return launch_quantize<BITS, WDT, MATH, 1>(w, delta, N, K, ldw, ldd, group, qweight, scale, sdt, zp, zdt, st);
+        return launch_quantize<BITS, WDT, MATH, 1>(w, delta, N, K, ldw, ldd, group, qweight, scale, sdt, zp, zdt, recip, st);
     const int64_t total = N * (K / VPI);
     hipLaunchKernelGGL((quantize_pack_generic_kernel<WDT, MATH>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, w,
-                       delta, N, (int)K, ldw, ldd, BITS, group, qweight, scale, sdt, zp, zdt);
+                       delta, N, (int)K, ldw, ldd, BITS, group, qweight, scale, sdt, zp, zdt, recip);
     return hipGetLastError() == hipSuccess ? BW_OK : BW_ELAUNCH;
 }
 
 template <int WDT, int MATH>
 int dispatch_bits(int bits, const void* w, const void* delta, int64_t N, int64_t K, int64_t ldw, int64_t ldd, int group,
-                  int32_t* qweight, void* scale, int sdt, void* zp, int zdt, hipStream_t st) {
-    if (bits == 2) return launch_quantize_bits<2, WDT, MATH>(w, delta, N, K, ldw, ldd, group, qweight, scale, sdt, zp, zdt, st);
-    if (bits == 4) return launch_quantize_bits<4, WDT, MATH>(w, delta, N, K, ldw, ldd, group, qweight, scale, sdt, zp, zdt, st);
-    return launch_quantize_bits<8, WDT, MATH>(w, delta, N, K, ldw, ldd, group, qweight, scale, sdt, zp, zdt, st);
+                  int32_t* qweight, void* scale, int sdt, void* zp, int zdt, int recip, hipStream_t st) {
+    if (bits == 2) return launch_quantize_bits<2, WDT, MATH>(w, delta, N, K, ldw, ldd, group, qweight, scale, sdt, zp, zdt, recip, st);
+    if (bits == 4) return launch_quantize_bits<4, WDT, MATH>(w, delta, N, K, ldw, ldd, group, qweight, scale, sdt, zp, zdt, recip, st);
+    return launch_quantize_bits<8, WDT, MATH>(w, delta, N, K, ldw, ldd, group, qweight, scale, sdt, zp, zdt, recip, st);
 }
 
 }  // namespace
@@ -390,6 +394,8 @@ extern "C" int bw_quantize_pack_add(const void* w, const void* delta, int w_dtyp
                                     int64_t ldw, int64_t ldd, int bits, int group, int32_t* qweight, void* scale,
                                     int scale_dtype, void* zp, int zp_dtype, void* stream) {
     if (!w || !qweight || !scale || !zp) return BW_EINVAL;
+    const int recip = (math_dtype & BW_SCALE_RECIPROCAL) != 0;
+    math_dtype &= ~BW_SCALE_RECIPROCAL;
     if (!bw_shape_ok(N, K, bits, group) || ldw < K || (delta && ldd < K)) return BW_EINVAL;
     if (w_dtype != BW_F16 && w_dtype != BW_BF16 && w_dtype != BW_F32) return BW_EINVAL;
     if (scale_dtype != BW_F32 && scale_dtype != BW_F16 && scale_dtype != BW_BF16) return BW_EINVAL;
@@ -402,7 +408,7 @@ extern "C" int bw_quantize_pack_add(const void* w, const void* delta, int w_dtyp
     hipStream_t st = (hipStream_t)stream;
 #define BW_Q(WD, MD) \
     if (w_dtype == WD && math_dtype == MD) \
-        return dispatch_bits<WD, MD>(bits, w, delta, N, K, ldw, ldd, group, qweight, scale, scale_dtype, zp, zp_dtype, st);
+        return dispatch_bits<WD, MD>(bits, w, delta, N, K, ldw, ldd, group, qweight, scale, scale_dtype, zp, zp_dtype, recip, st);
     BW_Q(BW_F32, BW_F32) BW_Q(BW_F16, BW_F32) BW_Q(BW_BF16, BW_F32) BW_Q(BW_F16, BW_F16) BW_Q(BW_BF16, BW_BF16)
 #undef BW_Q
     return BW_EINVAL;

@@ -4,9 +4,35 @@ libbitween_hip.so.  Tensors that live on the CPU are staged through the GPU
 and the results returned on the input's device; without a GPU these
 functions raise (there is no CPU implementation in this package).
 """
+import os
+
 import torch
 
 from .kernels import hip_loader as _hip
+
+
+# How `(w_max - w_min) / Qmax` (bitween/functional.py:25) is rounded.  Eager torch divides a tensor by a Python
+# scalar exactly on the CPU and multiplies by the float32 reciprocal on a GPU; the two differ in the last bit of
+# most float32 scales.  "ieee" (default) is the CPU arithmetic, the source as written; "torch_device" reproduces
+# what the reference computes when it quantises on a GPU.  BITWEEN_SCALE_DIVISION sets the initial choice.
+_SCALE_DIVISIONS = ("ieee", "torch_device")
+_scale_division = os.environ.get("BITWEEN_SCALE_DIVISION", "ieee")
+if _scale_division not in _SCALE_DIVISIONS:
+    raise ValueError(f"BITWEEN_SCALE_DIVISION must be one of {_SCALE_DIVISIONS}, got {_scale_division!r}")
+
+
+def set_scale_division(mode: str) -> str:
+    """Choose the rounding of the scale division for quantize_rtn and QuantizedLinear.from_float: "ieee" or
+    "torch_device".  Returns the previous choice."""
+    global _scale_division
+    if mode not in _SCALE_DIVISIONS:
+        raise ValueError(f"scale division must be one of {_SCALE_DIVISIONS}, got {mode!r}")
+    previous, _scale_division = _scale_division, mode
+    return previous
+
+
+def get_scale_division() -> str:
+    return _scale_division
 
 
 def _gpu_for(t):
@@ -52,7 +78,8 @@ def _quantize(weight, bits, group_size, value):
     dev = _gpu_for(weight)
     w = weight.to(dev)
     qweight, scale, zp = _hip.quantize_pack(w, bits, group_size, math_dtype=weight.dtype, scale_dtype=weight.dtype,
-                                            zp_dtype=torch.int32, delta=None if value is None else value.to(dev))
+                                            zp_dtype=torch.int32, delta=None if value is None else value.to(dev),
+                                            scale_reciprocal=_scale_division == "torch_device")
     if not weight.is_cuda:
         qweight, scale, zp = qweight.to(weight.device), scale.to(weight.device), zp.to(weight.device)
     return qweight, scale, zp, group_size

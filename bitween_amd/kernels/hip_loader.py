@@ -17,6 +17,7 @@ _LIB_PATH = os.environ.get("BITWEEN_HIP_LIB") or os.path.join(
 _lib = None
 
 BW_F16, BW_BF16, BW_F32, BW_I32 = 0, 1, 2, 3
+BW_SCALE_RECIPROCAL = 0x100   # flag for math_dtype: scale = (max - min) * fl32(1 / Qmax), as eager torch computes it on a GPU
 _DTYPE_CODE = {torch.float16: BW_F16, torch.bfloat16: BW_BF16, torch.float32: BW_F32, torch.int32: BW_I32}
 
 ABI_VERSION = 6            # what bw_abi_version() of a matching library returns
@@ -96,9 +97,10 @@ def _stream(device):
     return torch._C._cuda_getCurrentRawStream(device.index if device.index is not None else torch.cuda.current_device())
 
 
-def quantize_pack(weight, bits, group_size, math_dtype, scale_dtype, zp_dtype, delta=None):
+def quantize_pack(weight, bits, group_size, math_dtype, scale_dtype, zp_dtype, delta=None, scale_reciprocal=False):
     """weight [N,K] on GPU (f16/bf16/f32) -> (qweight int32, scale, zero_point) per bw_quantize_pack; with
-    `delta` (same shape and dtype) the kernel quantises weight + delta (bw_quantize_pack_add)."""
+    `delta` (same shape and dtype) the kernel quantises weight + delta (bw_quantize_pack_add).
+    `scale_reciprocal`: the scale as eager torch forms it on a GPU (BW_SCALE_RECIPROCAL)."""
     require_gpu(weight, "quantize_pack")
     if weight.stride(-1) != 1:
         weight = weight.contiguous()
@@ -116,7 +118,7 @@ def quantize_pack(weight, bits, group_size, math_dtype, scale_dtype, zp_dtype, d
     zp = torch.empty((n, k // group_size), dtype=zp_dtype, device=dev)
     with torch.cuda.device(dev):
         st = load().bw_quantize_pack_add(weight.data_ptr(), None if delta is None else delta.data_ptr(),
-                                         _DTYPE_CODE[weight.dtype], _DTYPE_CODE[math_dtype], n, k, weight.stride(0),
+                                         _DTYPE_CODE[weight.dtype], _DTYPE_CODE[math_dtype] | (BW_SCALE_RECIPROCAL if scale_reciprocal else 0), n, k, weight.stride(0),
                                          0 if delta is None else delta.stride(0), bits, group_size, qweight.data_ptr(),
                                          scale.data_ptr(), _DTYPE_CODE[scale_dtype], zp.data_ptr(),
                                          _DTYPE_CODE[zp_dtype], _stream(dev))

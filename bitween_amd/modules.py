@@ -9,6 +9,7 @@ import weakref
 import torch
 import torch.nn as nn
 
+from . import functional as _functional
 from .kernels import hip_loader as _hip
 
 
@@ -137,7 +138,8 @@ class QuantizedLinear(nn.Module):
                 raise _hip.BitweenHipError("QuantizedLinear.from_float needs a ROCm GPU (no CPU implementation)")
             weight = weight.to("cuda")
         qweight, scale, zero_point = _hip.quantize_pack(weight, bits, group_size, math_dtype=torch.float32,
-                                                        scale_dtype=torch.float16, zp_dtype=torch.float16)
+                                                        scale_dtype=torch.float16, zp_dtype=torch.float16,
+                                                        scale_reciprocal=_functional.get_scale_division() == "torch_device")
         # the constructor's zero buffers are built on the meta device (no memory, no host-to-device copy) and
         # replaced by the kernel's outputs, which already have the buffers' shapes and dtypes
         with torch.device("meta"):

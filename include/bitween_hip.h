@@ -31,6 +31,13 @@ extern "C" {
 
 typedef enum bw_dtype { BW_F16 = 0, BW_BF16 = 1, BW_F32 = 2, BW_I32 = 3 } bw_dtype;
 
+/* Flag for the math_dtype argument of bw_quantize_pack / bw_quantize_pack_add (OR it in): form the scale as
+ * (max - min) * fl32(1 / Qmax) instead of (max - min) / Qmax.  bitween/functional.py:25 divides a tensor by the
+ * Python scalar Qmax: eager torch performs that as a true division on the CPU and, on a GPU, as a
+ * multiplication by the float32 reciprocal, which rounds differently in the last bit of most float32 scales
+ * (and so moves a few zero points and packed values per layer).  Without the flag: the CPU arithmetic. */
+enum { BW_SCALE_RECIPROCAL = 0x100 };
+
 typedef enum bw_status {
     BW_OK = 0,
     BW_EINVAL = -1,       /* bad bits / group / shape / null pointer            */
@@ -52,7 +59,8 @@ const char* bw_strerror(int status);
  *   w          [N][ldw] of w_dtype (BW_F16 | BW_BF16 | BW_F32), row pitch ldw elements
  *   math_dtype dtype the arithmetic is rounded to after every operation:
  *              BW_F32 = what from_float does (upcast first, modules.py:191);
- *              BW_F16 / BW_BF16 = eager torch ops on a half tensor.
+ *              BW_F16 / BW_BF16 = eager torch ops on a half tensor;
+ *              optionally | BW_SCALE_RECIPROCAL (eager torch on a GPU, see above).
  *   qweight    int32 [N][K*bits/32]
  *   scale      [N][K/group] of scale_dtype (BW_F32 | BW_F16 | BW_BF16); a 16-bit
  *              type applies the module's round-to-nearest-even store

@@ -23,11 +23,14 @@ def build():
 def load():
     global _lib
     if _lib is None:
-        if not os.path.exists(_SO):
+        src = os.path.join(_HERE, "rtn_oracle.c")
+        if not os.path.exists(_SO) or (os.path.exists(src) and os.path.getmtime(src) > os.path.getmtime(_SO)):
             build()
         lib = ctypes.CDLL(_SO)
         i64, i32, vp = ctypes.c_int64, ctypes.c_int, ctypes.c_void_p
         lib.orc_quantize_rtn_f32.argtypes = [vp, i64, i64, i32, i32, vp, vp, vp]
+        lib.orc_quantize_rtn_f32_div.argtypes = [vp, i64, i64, i32, i32, i32, vp, vp, vp]
+        lib.orc_quantize_rtn_f32_div.restype = ctypes.c_int
         lib.orc_dequantize_f32.argtypes = [vp, vp, vp, i64, i64, i32, i32, vp]
         lib.orc_dequantize_f16.argtypes = [vp, vp, vp, i64, i64, i32, i32, vp]
         lib.orc_qlinear_forward.argtypes = [vp, i64, i64, vp, vp, vp, vp, i64, i32, i32, vp]
@@ -41,13 +44,13 @@ def _p(a):
     return a.ctypes.data_as(ctypes.c_void_p)
 
 
-def quantize_rtn_f32(w, bits, group_size):
+def quantize_rtn_f32(w, bits, group_size, scale_div="ieee"):
     w = np.ascontiguousarray(w, np.float32)
     n, k = w.shape
     qw = np.empty((n, k * bits // 32), np.int32)
     s = np.empty((n, k // group_size), np.float32)
     z = np.empty((n, k // group_size), np.int32)
-    rc = load().orc_quantize_rtn_f32(_p(w), n, k, bits, group_size, _p(qw), _p(s), _p(z))
+    rc = load().orc_quantize_rtn_f32_div(_p(w), n, k, bits, group_size, int(scale_div == "reciprocal"), _p(qw), _p(s), _p(z))
     if rc:
         raise ValueError("orc_quantize_rtn_f32 rejected its arguments")
     return qw, s, z

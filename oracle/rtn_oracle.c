@@ -59,8 +59,17 @@ float orc_f16_to_f32(uint16_t h) { return f16_bits_to_f32(h); }
 
 /* w [n][k] float32 -> qweight int32 [n][k*bits/32], scale f32 [n][k/g],
  * zero_point int32 [n][k/g].  Returns 0, or -1 for bad arguments. */
+int orc_quantize_rtn_f32_div(const float* w, int64_t n, int64_t k, int bits, int g, int reciprocal,
+                             int32_t* qweight, float* scale, int32_t* zero_point);
 int orc_quantize_rtn_f32(const float* w, int64_t n, int64_t k, int bits, int g,
                          int32_t* qweight, float* scale, int32_t* zero_point) {
+    return orc_quantize_rtn_f32_div(w, n, k, bits, g, 0, qweight, scale, zero_point);
+}
+
+/* reciprocal != 0: the scale as eager torch forms it on a GPU, (hi - lo) * (1.0f / qmax); else the true
+ * division of the CPU path. */
+int orc_quantize_rtn_f32_div(const float* w, int64_t n, int64_t k, int bits, int g, int reciprocal,
+                             int32_t* qweight, float* scale, int32_t* zero_point) {
     if (!(bits == 2 || bits == 4 || bits == 8) || g < 1 || k % g || k % (32 / bits)) return -1;
     const float qmax = (float)((1 << bits) - 1);
     const int vpi = 32 / bits;
@@ -73,7 +82,8 @@ int orc_quantize_rtn_f32(const float* w, int64_t n, int64_t k, int bits, int g,
             const float* p = w + r * k + gi * g;
             float lo = p[0], hi = p[0];
             for (int i = 1; i < g; i++) { if (p[i] < lo) lo = p[i]; if (p[i] > hi) hi = p[i]; }
-            float s = (hi - lo) / qmax;                    /* functional.py:25 */
+            const float range = hi - lo;
+            float s = reciprocal ? range * (1.0f / qmax) : range / qmax;   /* functional.py:25 */
             if (s < 1e-8f) s = 1e-8f;
             float zf = clampf(rintf(-lo / s), 0.0f, qmax); /* functional.py:26 */
             scale[r * groups + gi] = s;

@@ -12,7 +12,7 @@ round-half-to-even, which is what torch.round does.
 How each function is pinned (see tests/test_oracle_pins.py):
   pack_words / unpack_words   closed form sum(q_i << (i*bits)) mod 2**32 in
                               Python integers, hand-written words, round trip
-  quantize_rtn (f32 math)     exact-rational evaluation with explicit
+  quantize_rtn (f32 math)     (both scale_div modes) exact-rational evaluation with explicit
                               round-to-nearest-even per operation, hand-derived
                               known answers, invariants, C restatement
   quantize_rtn (f16/bf16)     same exact-rational check with binary16/bfloat16
@@ -76,8 +76,16 @@ def unpack_words(qweight, bits):
     return vals.reshape(u.shape[0], -1).astype(np.int32)
 
 
-def quantize_rtn(weight, bits=8, group_size=32, math="f32"):
+def quantize_rtn(weight, bits=8, group_size=32, math="f32", scale_div="ieee"):
     """bitween/functional.py:3-45.
+
+    scale_div: how the division of a tensor by the Python scalar Qmax (:25) is
+    carried out.  "ieee" = a correctly rounded division, what eager torch does
+    on the CPU.  "reciprocal" = what eager torch does on a GPU for a scalar
+    divisor: a multiplication by float32(1) / float32(Qmax), the product
+    rounded to float32 and then to the tensor's type (pinned on the GPU box
+    against torch itself, tests/test_gpu_eager_torch.py, and by exact-rational
+    vectors).
 
     Returns (qweight int32 [N,K*bits/32], scale [N,G], zero_point int32 [N,G],
     q int32 [N,K]).  `math` is the dtype the reference would compute in, i.e.
@@ -99,7 +107,12 @@ def quantize_rtn(weight, bits=8, group_size=32, math="f32"):
     w_max = wg.max(axis=-1, keepdims=True)                       # :23
     with np.errstate(all="ignore"):
         rng = _round_to(w_max - w_min, math)
-        scale = _round_to(rng / qmax, math)                      # :25
+        if scale_div == "ieee":
+            scale = _round_to(rng / qmax, math)                  # :25
+        elif scale_div == "reciprocal":
+            scale = _round_to((rng * (np.float32(1.0) / qmax)).astype(np.float32), math)
+        else:
+            raise ValueError(scale_div)
         floor = _round_to(np.float32(1e-8).reshape(1), math)[0]  # 1e-8 is 0 in f16
         scale = np.maximum(scale, floor)
         zp_f = _round_to((-w_min) / scale, math)                 # :26

@@ -66,7 +66,7 @@ def make_weight(kind, rng, n, k, g, bits):
     return np.ascontiguousarray(w, np.float32)
 
 
-def exact_case(w, bits, g, fmt):
+def exact_case(w, bits, g, fmt, scale_div="ieee"):
     n, k = w.shape
     groups = k // g
     q = np.zeros((n, k), np.int32)
@@ -79,7 +79,7 @@ def exact_case(w, bits, g, fmt):
         for gi in range(groups):
             vals = [float(v) for v in w[r, gi * g:(gi + 1) * g]]
             try:
-                s, z, qq = quantize_group_exact(vals, bits, fmt)
+                s, z, qq = quantize_group_exact(vals, bits, fmt, scale_div)
             except ZeroDivisionError:
                 valid[r, gi] = False                 # reference divides by zero here: unpinned
                 continue
@@ -129,6 +129,26 @@ def main():
                             y[m, r] = float(sum(Fraction(float(a)) * Fraction(float(b)) for a, b in zip(x[m], case["w16"][r])))
                     out[key + "_x"] = x
                     out[key + "_y64"] = y
+                    idx += 1
+    # the same path with the scale formed by the float32 reciprocal (eager torch on a GPU): names end in ":recip"
+    for fmt, kinds in (("f32", ["normal_f32", "normal_f16", "outliers", "ties", "large"]), ("f16", ["normal_f16"]), ("bf16", ["normal_f16"])):
+        for bits in (2, 4, 8):
+            for g in (32, 128):
+                for kind in kinds:
+                    rng = np.random.default_rng(77000 + 1000 * bits + g + len(kind))
+                    n, k = 4, 2 * g
+                    w = make_weight(kind, rng, n, k, g, bits)
+                    if fmt == "f16":
+                        w = w.astype(np.float16).astype(np.float32)
+                    if fmt == "bf16":
+                        w = _to_bf16(w)
+                    case = exact_case(w, bits, g, fmt, "reciprocal")
+                    key = f"c{idx:03d}"
+                    names.append(f"{key}:{fmt}:{bits}:{g}:{kind}:recip")
+                    out[key + "_w"] = w
+                    for name, arr in case.items():
+                        if name not in ("w16", "w32"):
+                            out[f"{key}_{name}"] = arr
                     idx += 1
     out["names"] = np.array(names)
     path = os.path.join(HERE, "rtn_exact_vectors.npz")

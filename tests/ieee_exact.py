@@ -50,16 +50,24 @@ def rint_even(x):
     return int(f)
 
 
-def quantize_group_exact(values, bits, fmt="f32"):
+def quantize_group_exact(values, bits, fmt="f32", scale_div="ieee"):
     """RTN of one group, following bitween/functional.py:22-29 operation by
     operation.  values: floats already representable in fmt.
+    scale_div "ieee": (hi - lo) / Qmax is one correctly rounded division (eager
+    torch on the CPU).  "reciprocal": eager torch on a GPU multiplies by the
+    float32 reciprocal of a scalar divisor: r = RN32(1 / Qmax), then
+    RN32((hi - lo) * r), then - for a 16-bit tensor - a second rounding to fmt.
     Returns (scale Fraction, zero_point int, q list[int])."""
     w = [Fraction(v) for v in values]
     for v in w:
         assert rn(v, fmt) == v, "input not representable in the math format"
     qmax = (1 << bits) - 1
     lo, hi = min(w), max(w)
-    scale = rn(rn(hi - lo, fmt) / qmax, fmt)
+    if scale_div == "ieee":
+        scale = rn(rn(hi - lo, fmt) / qmax, fmt)
+    else:
+        assert scale_div == "reciprocal"
+        scale = rn(rn(rn(hi - lo, fmt) * rn(Fraction(1, qmax), "f32"), "f32"), fmt)
     import struct
     floor32 = Fraction(struct.unpack("f", struct.pack("f", 1e-8))[0])   # the float32 nearest 1e-8
     floor = rn(floor32, fmt) if fmt != "f32" else floor32               # 0 in f16

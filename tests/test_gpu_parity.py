@@ -14,7 +14,9 @@ from gpu_util import check_matmul, make_weight, quantized_layer, to_gpu
 pytestmark = pytest.mark.gpu
 
 GOLD = np.load(os.path.join(os.path.dirname(__file__), "golden", "rtn_exact_vectors.npz"))
-CASES = [str(s) for s in GOLD["names"]]
+ALL_CASES = [str(s) for s in GOLD["names"]]
+CASES = [c for c in ALL_CASES if not c.endswith(":recip")]          # scale by true division (eager torch on the CPU)
+RECIP_CASES = [c for c in ALL_CASES if c.endswith(":recip")]        # scale by the float32 reciprocal (eager torch on a GPU)
 TORCH_DT = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}
 COMBOS = [(b, g) for b in (2, 4, 8) for g in (32, 64, 128)]
 
@@ -60,6 +62,38 @@ def test_quantize_matches_exact_vectors(name):
     assert np.array_equal(q[vq], GOLD[key + "_q"][vq])
     if valid.all():
         assert np.array_equal(qw.cpu().numpy(), GOLD[key + "_qweight"])
+
+
+@pytest.mark.parametrize("name", RECIP_CASES)
+def test_quantize_with_reciprocal_scale_matches_exact_vectors(name):
+    """set_scale_division("torch_device"): the scale as eager torch forms it on a GPU, (max - min) * fl32(1 / Qmax)."""
+    import bitween_amd
+    key, fmt, bits, g = name.split(":")[:4]
+    bits, g = int(bits), int(g)
+    w = torch.from_numpy(GOLD[key + "_w"]).to(TORCH_DT[fmt]).cuda()
+    previous = bitween_amd.set_scale_division("torch_device")
+    try:
+        qw, scale, zp, _ = bitween_amd.quantize_rtn(w, bits, g)
+        if fmt == "f32":
+            lin = torch.nn.Linear(w.shape[1], w.shape[0], bias=False)
+            lin.weight.data = w.clone()
+            layer = bitween_amd.QuantizedLinear.from_float(lin, bits, g)
+    finally:
+        bitween_amd.set_scale_division(previous)
+    valid = GOLD[key + "_valid"]
+    assert np.array_equal(zp.cpu().numpy()[valid], GOLD[key + "_zp"][valid])
+    exp_scale = GOLD[key + "_scale"]
+    if fmt == "f32":
+        assert np.array_equal(_bits_of(scale)[valid], exp_scale.view(np.uint32)[valid])
+        assert np.array_equal(layer.qweight.cpu().numpy(), GOLD[key + "_qweight"])
+        assert np.array_equal(_bits_of(layer.scale), GOLD[key + "_scale16"].view(np.uint16))
+    elif fmt == "f16":
+        assert np.array_equal(_bits_of(scale)[valid], exp_scale.astype(np.float16).view(np.uint16)[valid])
+    else:
+        assert np.array_equal(_bits_of(scale)[valid], _bf16_bits(exp_scale)[valid])
+    q = orc.unpack_words(qw.cpu().numpy(), bits)
+    vq = np.repeat(valid, g, axis=1)
+    assert np.array_equal(q[vq], GOLD[key + "_q"][vq])
 
 
 @pytest.mark.parametrize("name", [c for c in CASES if c.split(":")[1] == "f32"])

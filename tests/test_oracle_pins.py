@@ -15,11 +15,13 @@ import pytest
 from oracle import c_oracle, rtn_oracle as orc
 
 GOLD = np.load(os.path.join(os.path.dirname(__file__), "golden", "rtn_exact_vectors.npz"))
-CASES = [str(s) for s in GOLD["names"]]
+ALL_CASES = [str(s) for s in GOLD["names"]]
+CASES = [c for c in ALL_CASES if not c.endswith(":recip")]          # scale by true division (eager torch on the CPU)
+RECIP_CASES = [c for c in ALL_CASES if c.endswith(":recip")]        # scale by the float32 reciprocal (eager torch on a GPU)
 
 
 def _case(name):
-    key, fmt, bits, g, kind = name.split(":")
+    key, fmt, bits, g, kind = name.split(":")[:5]
     return key, fmt, int(bits), int(g), kind
 
 
@@ -44,6 +46,37 @@ def test_numpy_oracle_matches_exact_vectors(name):
         y, y64 = orc.qlinear_forward(GOLD[key + "_x"], qw, s16, z16, None, bits, g)
         ref = GOLD[key + "_y64"]
         assert np.allclose(y64, ref, rtol=1e-12, atol=1e-12 * np.abs(ref).max())
+
+
+@pytest.mark.parametrize("name", RECIP_CASES)
+def test_oracles_match_exact_vectors_with_reciprocal_scale(name):
+    """scale = RN(RN32((max - min) * RN32(1 / Qmax))): the arithmetic of eager torch on a GPU for functional.py:25."""
+    key, fmt, bits, g, _ = _case(name)
+    w = GOLD[key + "_w"]
+    valid = GOLD[key + "_valid"]
+    qw, scale, zp, q = orc.quantize_rtn(w, bits, g, math=fmt, scale_div="reciprocal")
+    vq = np.repeat(valid, g, axis=1)
+    assert np.array_equal(scale.view(np.uint32)[valid], GOLD[key + "_scale"].view(np.uint32)[valid])
+    assert np.array_equal(zp[valid], GOLD[key + "_zp"][valid])
+    assert np.array_equal(q[vq], GOLD[key + "_q"][vq])
+    if valid.all():
+        assert np.array_equal(qw, GOLD[key + "_qweight"])
+    if fmt == "f32":
+        qw_c, s_c, z_c = c_oracle.quantize_rtn_f32(w, bits, g, scale_div="reciprocal")
+        assert np.array_equal(qw_c, GOLD[key + "_qweight"]) and np.array_equal(z_c, GOLD[key + "_zp"])
+        assert np.array_equal(s_c.view(np.uint32), GOLD[key + "_scale"].view(np.uint32))
+
+
+def test_reciprocal_scale_differs_from_true_division_where_expected():
+    """The two roundings are different functions: on random float32 ranges most scales differ by one ulp (the
+    flag is not a no-op), while zero points and packed values move only in a few groups."""
+    w = (np.random.default_rng(5).standard_normal((64, 1024)) * 0.02).astype(np.float32)
+    _, s_a, z_a, q_a = orc.quantize_rtn(w, 4, 128)
+    _, s_b, z_b, q_b = orc.quantize_rtn(w, 4, 128, scale_div="reciprocal")
+    differ = (s_a.view(np.uint32) != s_b.view(np.uint32)).mean()
+    assert 0.3 < differ < 0.95
+    assert np.abs(s_a.view(np.int32).astype(np.int64) - s_b.view(np.int32).astype(np.int64)).max() <= 1
+    assert (q_a != q_b).mean() < 0.01
 
 
 @pytest.mark.parametrize("name", [c for c in CASES if c.split(":")[1] == "f32"])
