@@ -487,7 +487,7 @@ def test_error_conventions_on_gpu():
 
 @pytest.mark.parametrize("bits,g,k,n", [(4, 128, 4096, 11008), (4, 128, 11008, 4096), (8, 128, 4096, 11008),
                                         (4, 64, 4096, 11008), (2, 32, 4096, 11008), (4, 128, 4096, 4096),
-                                        (4, 32, 11008, 4096), (4, 64, 11008, 4096)])
+                                        (4, 32, 11008, 4096), (4, 64, 11008, 4096), (2, 32, 11008, 4096)])
 def test_full_size_properties(bits, g, k, n):
     """Full-size layers (Llama-2-7B shapes), checked through size-independent properties:
       * a one-hot activation row returns a column of W16 bit-for-bit (the fused kernels reproduce the
@@ -539,10 +539,18 @@ def test_full_size_properties(bits, g, k, n):
     assert np.array_equal(q.qweight[rows].cpu().numpy(), qw_o)
     assert np.array_equal(_bits_of(q.scale[rows]), s16.view(np.uint16))
     assert np.array_equal(q.zero_point[rows].float().cpu().numpy(), z_o.astype(np.float32))
-    for m in (1, 16):
+    for m in (1, 2, 4, 8, 16):
         x = torch.randn(m, k, device="cuda", dtype=torch.float16, generator=g_t)
         y = q(x)
         check_matmul(y[:, rows], x.cpu().numpy(), qw_o, s16, z16, None, bits, g)
+    # one-hot rows through the 16-row decode kernels as well (rows 7..15 stay zero)
+    x = torch.zeros(16, k, device="cuda", dtype=torch.float16)
+    for i, c in enumerate(cols):
+        x[2 * i, c] = 1.0
+    y = hip.quantized_gemv_hip(x, q.qweight, q.scale, q.zero_point, None, bits, g)
+    for i, c in enumerate(cols):
+        assert torch.equal(y[2 * i], w16[:, c])
+    assert (y[1::2] == 0).all()
     x = torch.randn(256, k, device="cuda", dtype=torch.float16, generator=g_t)
     y = q(x)
     check_matmul(y[:, rows], x.cpu().numpy(), qw_o, s16, z16, None, bits, g)
@@ -729,3 +737,47 @@ def test_rows_33_to_48_on_a_large_layer_take_the_prefill_kernel(dtype):
             assert torch.equal(y, yc)                            # same decode launches either way
         else:
             assert ((y.double() - yc.double()).abs() <= 2.0 ** -9 * ref.abs() + 2.0 ** -12 * mag).all()   # split-K or not
+
+
+@pytest.mark.parametrize("k,n", [(4096, 14336), (14336, 4096)])
+@pytest.mark.parametrize("m", [128, 512, 2048])
+@pytest.mark.parametrize("xdtype", [torch.float16, torch.bfloat16])
+def test_prefill_llama3_8b_mlp_shapes_at_full_size(k, n, m, xdtype):
+    """The prefill configuration at its own shapes (Llama-3-8B MLP, 4-bit g128, 128 / 512 / 2048 rows, float16 and
+    bfloat16 activations): through the split and the unsplit plan, one-hot rows return columns of W16 bit for bit and
+    random rows meet the matmul bars on a strided sample of output columns whose weights the oracle quantised
+    (main.py:444-466 is the formula, x.to(float16) of modules.py:74 for bfloat16)."""
+    import ctypes
+    hip = _hip()
+    lib = hip.load()
+    bits, g = 4, 128
+    g_t = torch.Generator(device="cuda").manual_seed(k // 7 + m)
+    w = (torch.randn(n, k, device="cuda", generator=g_t) * 0.02).half()
+    layer = torch.nn.Linear(k, n, bias=False, device="cuda", dtype=torch.float16)
+    layer.weight.data = w
+    import bitween_amd
+    q = bitween_amd.QuantizedLinear.from_float(layer, bits, g)
+    w16 = hip.dequantize(q.qweight, q.scale, q.zero_point, g, bits, torch.float16)
+    rows = np.unique(np.concatenate([np.arange(0, n, n // 40), [255, 256, n - 257, n - 1]]))
+    qw_o, s_o, z_o, _ = orc.quantize_rtn(w[rows].float().cpu().numpy(), bits, g)
+    s16, z16 = orc.store_module_buffers(s_o, z_o)
+    assert np.array_equal(q.qweight[rows].cpu().numpy(), qw_o)
+    x = torch.randn(m, k, device="cuda", generator=g_t).to(xdtype)
+    hot = {0: 0, 1: k - 1, 5: 129, m // 2 + 1: k // 2, m - 1: 4095}            # row -> column of its single 1
+    for r, c in hot.items():
+        x[r] = 0
+        x[r, c] = 1.0
+    x16 = x.to(torch.float16)
+    # the forward as the module runs it (bfloat16 cast + split-K workspace where the plan wants one)
+    y_split = hip.quantized_matmul_hip(x, q.qweight, q.scale, q.zero_point, None, bits, g)
+    # the same kernel without a workspace: nothing is split
+    y_plain = torch.empty((m, n), dtype=torch.float16, device="cuda")
+    st = lib.bw_qgemm(x16.data_ptr(), 0, m, k, k, q.qweight.data_ptr(), q.scale.data_ptr(), q.zero_point.data_ptr(), None, n,
+                      bits, g, y_plain.data_ptr(), n, ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    assert st == 0
+    torch.cuda.synchronize()
+    x_np = x16.cpu().numpy()
+    for y in (y_split, y_plain):
+        for r, c in hot.items():
+            assert torch.equal(y[r], w16[:, c])
+        check_matmul(y[:, rows], x_np, qw_o, s16, z16, None, bits, g)
