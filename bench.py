@@ -3,18 +3,16 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-extras]
 
-A step is one decode pass (M = 1) over the seven quantised linears of a
-Llama-2-7B decoder layer (q/k/v/o 4096x4096, gate/up 4096->11008, down
-11008->4096; 4-bit, group 128), inputs resident in HBM.  Successive steps use
-different layers' weights (--layers distinct copies, > 256 MiB in total) so
-the Infinity Cache cannot serve them.  `value` is algorithmic bytes per step
-(packed weights + scales + zero points + activations in + out) over the time
-per step, in GB/s.  The launches of a step are replayed from a HIP graph so
-the Python interpreter is not what is being timed.
+A step is one decode pass (M = 1) through the 224 quantised linears of a 32-layer Llama-2-7B-shaped decoder
+(per layer q/k/v/o 4096x4096, gate/up 4096->11008, down 11008->4096; 4-bit, group 128), inputs resident in
+HBM: --layers distinct layers' weights (8: 860 MB, more than the 256 MiB Infinity Cache holds) are run through
+32 / layers times.  `value` is algorithmic bytes per step (packed weights + scales + zero points + activations
+in + out) over the time per step, in GB/s.  A step is one HIP graph of 224 launches, so the Python
+interpreter is not what is being timed and a run of 20 steps lasts about 25 ms.
 
-Also reported on the same JSON line: the roofline of the decode kernel, the
-CPU restatement timed on the host cores, and (unless --no-extras) per-M decode
-rates, prefill TFLOP/s next to same-run fp16 hipBLASLt, and quantiser rates.
+Also reported on the same JSON line: the roofline of the decode kernel (overall and per layer shape, next to
+this board's measured stream-copy rate), the CPU path timed on the host cores, and (unless --no-extras)
+per-M decode rates, prefill TFLOP/s next to same-run fp16 hipBLASLt, quantiser rates and the end-to-end decoder.
 """
 import argparse
 import json
@@ -26,6 +24,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
+MODEL_LAYERS = 32          # decoder layers a headline step stands for (Llama-2-7B)
 MFMA_F16_PEAK_TFLOPS = 2500.0
 LLAMA7B_LINEARS = [("q_proj", 4096, 4096), ("k_proj", 4096, 4096), ("v_proj", 4096, 4096), ("o_proj", 4096, 4096),
                    ("gate_proj", 4096, 11008), ("up_proj", 4096, 11008), ("down_proj", 11008, 4096)]   # name, K, N
@@ -74,28 +73,99 @@ def graph_of(torch, fn):
     return g
 
 
-def cpu_baseline(bits, g):
-    """The C restatement of the reference path (oracle/rtn_oracle.c: dequantise to float16 values, float64
-    dot, float16 out) timed on this host for one 4096x4096 M=1 forward, OpenMP over the host's cores."""
+def _cpu_info():
+    model, cores = "unknown", set()
+    try:
+        phys = core = None
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name") and model == "unknown":
+                model = line.split(":", 1)[1].strip()
+            elif line.startswith("physical id"):
+                phys = line.split(":", 1)[1].strip()
+            elif line.startswith("core id"):
+                core = line.split(":", 1)[1].strip()
+            elif not line.strip():
+                if core is not None:
+                    cores.add((phys, core))
+                phys = core = None
+    except OSError:
+        pass
+    try:
+        usable = len(os.sched_getaffinity(0))
+    except AttributeError:
+        usable = os.cpu_count() or 1
+    return model, len(cores) or (os.cpu_count() or 1), usable
+
+
+def cpu_baseline():
+    """The reference's CPU path on this host: oracle/torch_cpu_path.py, the eager-torch restatement of
+    bitween/functional.py:3-71 + the module's float16 stores + main.py:462-466, on the one configuration that runs on
+    the CPU (an OPT-125m fc1: 768 -> 3072, 4-bit g128, M = 1 and 16), timed as the reference times things
+    (bitween/benchmark.py:191-218: 10 warm-ups, 50 runs, perf_counter) with torch's default thread count and with 1
+    thread.  `value` = algorithmic bytes of the M = 1 forward over its time at the default thread count.  A second
+    entry times the scalar C port (oracle/rtn_oracle.c, OpenMP) on one 4096 x 4096 layer."""
     import numpy as np
-    from oracle import c_oracle, rtn_oracle as orc
-    k = n = 4096
+    import torch
+    from oracle import c_oracle, rtn_oracle as orc, torch_cpu_path as tcp
+    k, n, bits, g = 768, 3072, 4, 128
+    gen = torch.Generator().manual_seed(0)
+    w16 = (torch.randn(n, k, generator=gen) * 0.02).half()
+    xs = {m: torch.randn(m, k, generator=gen).half() for m in (1, 16)}
+    qw, s16, z16 = tcp.module_buffers(w16, bits, g)
+
+    def timed(fn):
+        for _ in range(10):
+            fn()
+        t0 = time.perf_counter()
+        for _ in range(50):
+            fn()
+        return (time.perf_counter() - t0) / 50 * 1e3
+
+    model, physical, usable = _cpu_info()
+    default_threads = torch.get_num_threads()
+    legs = {}
+    for label, threads in (("default_threads", default_threads), ("1_thread", 1)):
+        torch.set_num_threads(threads)
+        legs[label] = {"torch_threads": torch.get_num_threads(),
+                       "quantize_pack_ms": round(timed(lambda: tcp.module_buffers(w16, bits, g)), 3),
+                       "forward_M1_ms": round(timed(lambda: tcp.forward(xs[1], qw, s16, z16, None, bits, g)), 3),
+                       "forward_M16_ms": round(timed(lambda: tcp.forward(xs[16], qw, s16, z16, None, bits, g)), 3)}
+    torch.set_num_threads(default_threads)
+    # the scalar C port on one Llama-sized layer (what the GPU headline runs 224 of per step)
+    kk = nn = 4096
     rng = np.random.default_rng(0)
-    w = (rng.standard_normal((n, k)) * 0.02).astype(np.float16).astype(np.float32)
-    qw, s, z = c_oracle.quantize_rtn_f32(w, bits, g)
-    s16, z16 = orc.store_module_buffers(s, z)
-    x = rng.standard_normal((1, k)).astype(np.float16)
-    cores = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
-    c_oracle.qlinear_forward(x, qw, s16, z16, None, bits, g)
-    t0 = time.perf_counter()
-    reps = 0
-    while time.perf_counter() - t0 < 10.0:
-        c_oracle.qlinear_forward(x, qw, s16, z16, None, bits, g)
+    wl = (rng.standard_normal((nn, kk)) * 0.02).astype(np.float16).astype(np.float32)
+    qwl, sl, zl = c_oracle.quantize_rtn_f32(wl, bits, g)
+    sl16, zl16 = orc.store_module_buffers(sl, zl)
+    xl = rng.standard_normal((1, kk)).astype(np.float16)
+    c_oracle.qlinear_forward(xl, qwl, sl16, zl16, None, bits, g)
+    t0, reps = time.perf_counter(), 0
+    while time.perf_counter() - t0 < 4.0:
+        c_oracle.qlinear_forward(xl, qwl, sl16, zl16, None, bits, g)
         reps += 1
-    dt = (time.perf_counter() - t0) / reps
-    return {"value": round(decode_bytes(1, k, n, bits, g) / dt / 1e9, 3), "unit": "GB/s", "cores": cores, "kind": "port",
-            "sample": f"{reps} forwards of one 4096x4096 W4 g128 linear, M=1 ({dt * 1e3:.2f} ms each), "
-                      "oracle/rtn_oracle.c orc_qlinear_forward with OpenMP"}
+    c_ms = (time.perf_counter() - t0) / reps * 1e3
+    omp = int(os.environ.get("OMP_NUM_THREADS", usable))
+    fwd = legs["default_threads"]["forward_M1_ms"]
+    return {"value": round(decode_bytes(1, k, n, bits, g) / (fwd * 1e-3) / 1e9, 3), "unit": "GB/s",
+            "cores": legs["default_threads"]["torch_threads"], "kind": "port",
+            "sample": "OPT-125m fc1 (768 -> 3072, W4 g128): 10 warm-ups + 50 runs each of quantize+pack and of the "
+                      "forward at M = 1 / 16, eager torch on the host (oracle/torch_cpu_path.py), at torch's default "
+                      "thread count and at 1 thread; value = M = 1 forward at the default thread count",
+            "cpu_model": model, "physical_cores": physical, "usable_cpus": usable,
+            "opt125m_fc1_torch_cpu": legs,
+            "c_port_4096x4096_M1": {"forward_ms": round(c_ms, 2), "GBps": round(decode_bytes(1, kk, nn, bits, g) / c_ms / 1e6, 3),
+                                    "omp_threads": omp, "runs": reps}}
+
+
+def copy_probe(torch):
+    """This board's stream-copy rate: a 1 GiB device-to-device copy (read + write bytes over device time)."""
+    src = torch.empty(1 << 30, dtype=torch.uint8, device="cuda").fill_(1)
+    dst = torch.empty_like(src)
+    for _ in range(3):
+        dst.copy_(src)
+    us = time_calls(torch, lambda: dst.copy_(src), 10, 2)
+    del src, dst
+    return round(2 * (1 << 30) / us / 1e3, 1)
 
 
 # ---- extras: every section takes (torch, hip, QuantizedLinear, layers) and returns a JSON-able dict; `layers`
@@ -389,7 +459,7 @@ def extras_llama7b_end_to_end(torch, hip, QuantizedLinear, layers):
         recipe["model.layers.%d.mlp.down_proj" % i] = (2, 32)
     ids = torch.randint(0, 32000, (1, 512), device="cuda", generator=torch.Generator(device="cuda").manual_seed(0))
 
-    def run(m, new_tokens=256):
+    def run(m, new_tokens=64):
         with torch.no_grad():
             torch.cuda.synchronize()
             t0 = time.perf_counter()
@@ -425,7 +495,53 @@ def extras_llama7b_end_to_end(torch, hip, QuantizedLinear, layers):
     run(qmodel, 8)
     pre, tps = run(qmodel)
     res["fused_siblings_prefill512_ms"], res["fused_siblings_decode_tokens_per_s"] = round(pre, 1), round(tps, 1)
-    res["note"] = "eager transformers loop: host-bound (hundreds of small launches per token), not a kernel figure"
+    res["note"] = ("drop-in check only: an eager transformers loop, 64 new tokens, host-bound (about a thousand small "
+                   "launches per token); the measured end-to-end configuration is llama7b_decoder_graph")
+    return res
+
+
+def extras_llama7b_decoder_graph(torch, hip, QuantizedLinear, layers):
+    """BASELINE's end-to-end configuration: a 32-layer Llama-7B-shaped decoder (bench_decoder.py: hidden 4096, 32
+    heads, MLP 11008, vocab 32000, random weights), Bitween(...).quantize(rtn=True, ignore_layers=[lm_head,
+    embed_tokens], layer_config = attention 8-bit g128, MLP 4-bit g128, down_proj of layers 0, 1, 30, 31 2-bit g32),
+    then a 512-token random prompt and 256 greedy tokens at batch 1 with one decode step captured in a HIP graph
+    and replayed.  The glue (RMSNorm, rotary, cache update, attention, SwiGLU) is plain torch: about 20 small
+    launches per layer next to the 4-7 of the linears."""
+    import bitween_amd
+    import bench_decoder as bd
+    nlayers, prompt, new_tokens = 32, 512, 256
+    with torch.device("cuda"):
+        model = bd.Decoder(layers=nlayers, max_len=prompt + new_tokens).half()
+    model.init_weights(seed=0)
+    ids = torch.randint(0, 32000, (prompt,), device="cuda", generator=torch.Generator(device="cuda").manual_seed(0))
+    res = {}
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    qmodel = bitween_amd.Bitween(model, bits=4, group_size=128).quantize(
+        rtn=True, ignore_layers=["lm_head", "embed_tokens"], layer_config=bd.mixed_recipe(nlayers), verbose=False)
+    torch.cuda.synchronize()
+    res["bitween_quantize_call_s"] = round(time.perf_counter() - t0, 3)
+    del model
+    qlin = [mod for mod in qmodel.modules() if isinstance(mod, QuantizedLinear)]
+    res["quantized_linears"] = len(qlin)
+    by = sum(decode_bytes(1, q.in_features, q.out_features, q.bits, q.group_size) for q in qlin)
+    by_all = by + 2 * 32000 * 4096                                   # + the float16 lm_head
+    res["bytes_per_token_quantized_linears"] = by
+    res["byte_ceiling_tokens_per_s"] = round(HBM_PEAK_GBPS * 1e9 / by_all, 1)
+    qmodel.alloc_state()
+    for label, fuse in (("per_module_launches", False), ("fused_siblings", True)):
+        if fuse:
+            bitween_amd.fuse_sibling_linears(qmodel)
+        bd.generate(qmodel, ids, 4)                                   # warm every kernel and the allocator
+        graph = bd.capture_step(qmodel)
+        pre_ms, dec_s, toks = bd.generate(qmodel, ids, new_tokens, graph)
+        _, eager_s, toks_eager = bd.generate(qmodel, ids, 32)
+        res[label] = {"prefill512_ms": round(pre_ms, 2), "decode_tokens_per_s": round((new_tokens - 1) / dec_s, 1),
+                      "decode_ms_per_token": round(dec_s / (new_tokens - 1) * 1e3, 3),
+                      "fraction_of_byte_ceiling": round((new_tokens - 1) / dec_s * by_all / (HBM_PEAK_GBPS * 1e9), 3),
+                      "eager_loop_tokens_per_s": round(31 / eager_s, 1),
+                      "graph_tokens_equal_eager_tokens": bool(torch.equal(toks[:32], toks_eager))}
+        del graph
     return res
 
 
@@ -496,14 +612,15 @@ EXTRAS = {"opt125m_fc1": extras_opt125m_fc1, "decode": extras_decode, "decode_in
           "prefill": extras_prefill, "prefill_other_formats": extras_prefill_other_formats, "quantize": extras_quantize, "mixed_precision_model": extras_mixed_precision_model, "eager_call": extras_eager_call,
           "decode_fused_siblings": extras_decode_fused_siblings,
           # the heavy sections last: the GEMMs and the 7B model leave the board warm, which shows in the decode timings
-          "backward": extras_backward, "llama7b_end_to_end": extras_llama7b_end_to_end}
+          "backward": extras_backward, "llama7b_decoder_graph": extras_llama7b_decoder_graph,
+          "transformers_drop_in_check": extras_llama7b_end_to_end}
 
 
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=400)
-    ap.add_argument("--warmup", type=int, default=40)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--layers", type=int, default=8, help="distinct weight sets rotated through")
     ap.add_argument("--m", type=int, default=1, help="decode batch of the headline number")
     ap.add_argument("--no-graph", action="store_true")
@@ -532,7 +649,7 @@ def main():
         for _ in range(5):
             dst.copy_(src)
         torch.cuda.synchronize()
-        print(json.dumps({"copy_probe_bytes": 256 << 20, "launches": 5}))
+        print(json.dumps({"copy_probe_bytes": 256 << 20, "launches": 5, "copy_gbps_1GiB": copy_probe(torch)}))
         return
 
     layers = [[make_layer(torch, QuantizedLinear, k, n, bits, g, seed=100 * li + i)
@@ -541,47 +658,32 @@ def main():
         print(json.dumps({args.only: EXTRAS[args.only](torch, hip, QuantizedLinear, layers)}))
         return
     xs = {k: torch.randn(m, k, device="cuda", dtype=torch.float16) for k in (4096, 11008)}
-    step_bytes = sum(decode_bytes(m, k, n, bits, g) for _, k, n in LLAMA7B_LINEARS)
-    launches_per_step = len(LLAMA7B_LINEARS)
+    passes = max(1, MODEL_LAYERS // args.layers)           # a step = one token through MODEL_LAYERS decoder layers
+    layer_bytes = sum(decode_bytes(m, k, n, bits, g) for _, k, n in LLAMA7B_LINEARS)
+    step_bytes = layer_bytes * passes * args.layers
+    launches_per_step = len(LLAMA7B_LINEARS) * passes * args.layers
 
-    def run_layer(li):
-        for q in layers[li]:
-            hip.quantized_gemv_hip(xs[q.in_features], q.qweight, q.scale, q.zero_point, None, bits, g)
+    def run_linears(select):
+        for _ in range(passes):
+            for layer in layers:
+                for q in layer:
+                    if select(q):
+                        hip.quantized_gemv_hip(xs[q.in_features], q.qweight, q.scale, q.zero_point, None, bits, g)
 
-    per_layer_graphs = None
     if args.no_graph:
-        def do_steps(first, count):
-            for s in range(first, first + count):
-                run_layer(s % args.layers)
+        def one_step():
+            run_linears(lambda q: True)
     else:
-        per_layer = [graph_of(torch, lambda li=li: run_layer(li)) for li in range(args.layers)]
-        full = graph_of(torch, lambda: [run_layer(li) for li in range(args.layers)])
-        PASSES = 4                                         # a long graph amortises the cost of launching it
-        many = graph_of(torch, lambda: [run_layer(li) for _ in range(PASSES) for li in range(args.layers)])
-        per_layer_graphs = (per_layer, full, many)
+        one_step = graph_of(torch, lambda: run_linears(lambda q: True)).replay
 
-        def do_steps(first, count):
-            s = first
-            while count > 0:
-                if s % args.layers == 0 and count >= PASSES * args.layers:
-                    many.replay()
-                    s += PASSES * args.layers
-                    count -= PASSES * args.layers
-                elif s % args.layers == 0 and count >= args.layers:
-                    full.replay()
-                    s += args.layers
-                    count -= args.layers
-                else:
-                    per_layer[s % args.layers].replay()
-                    s += 1
-                    count -= 1
-
-    do_steps(0, args.warmup)
+    for _ in range(args.warmup):
+        one_step()
     torch.cuda.synchronize()
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
     e0.record()
-    do_steps(args.warmup, args.steps)
+    for _ in range(args.steps):
+        one_step()
     e1.record()
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3
@@ -591,15 +693,30 @@ def main():
     us_per_launch = ms_per_step * 1e3 / launches_per_step
     bytes_per_launch = step_bytes / launches_per_step
 
+    # the same launches shape by shape (each shape's launches of a step as a graph of their own): where the step's
+    # time goes, and what fraction of the HBM peak each shape reaches
+    per_shape = {}
+    if not args.no_graph:
+        for (kk, nn) in sorted({(k, n) for _, k, n in LLAMA7B_LINEARS}):
+            count = sum(1 for _, k, n in LLAMA7B_LINEARS if (k, n) == (kk, nn)) * passes * args.layers
+            gr = graph_of(torch, lambda: run_linears(lambda q: (q.in_features, q.out_features) == (kk, nn)))
+            us = time_calls(torch, gr.replay, max(3, args.steps // 2), 2) / count
+            by = decode_bytes(m, kk, nn, bits, g)
+            per_shape["%dx%d" % (kk, nn)] = {"launches_per_step": count, "us": round(us, 3), "bytes": by,
+                                             "GBps": round(by / us / 1e3, 1), "frac": round(by / us / 1e3 / HBM_PEAK_GBPS, 4)}
+            del gr
+
     result = {
         "metric": "W4A16 g128 dequant-GEMM: decode HBM GB/s (% peak); prefill TFLOP/s",
         "value": round(gbps, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f16", "data": "synthetic",
         "config": {"workload": "Llama-2-7B decoder-layer linears (q/k/v/o 4096x4096, gate/up 4096->11008, down "
-                               "11008->4096), 4-bit g128 RTN, fp16 activations, decode M=%d; one step = the 7 fused "
-                               "forwards of one layer, %d layers' weights rotated" % (m, args.layers),
-                   "M": m, "bits": bits, "group_size": g, "layers_rotated": args.layers,
+                               "11008->4096), 4-bit g128 RTN, fp16 activations, decode M=%d; one step = one token "
+                               "through the %d linears of %d decoder layers (%d distinct layers' weights, %d MB, "
+                               "run through %d times)" % (m, launches_per_step, passes * args.layers, args.layers,
+                                                          layer_bytes * args.layers // 1000000, passes),
+                   "M": m, "bits": bits, "group_size": g, "layers_rotated": args.layers, "launches_per_step": launches_per_step,
                    "bytes_per_step": step_bytes, "launch": "eager" if args.no_graph else "hip_graph"},
         "pct_hbm_peak": round(100 * gbps / HBM_PEAK_GBPS, 2),
         "wall_ms_total": round(wall_ms, 3),
@@ -608,16 +725,19 @@ def main():
                      "frac": round(bytes_per_launch / (us_per_launch * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4),
                      # HBM bytes per launch from rocprofv3 FETCH_SIZE / WRITE_SIZE, scaled by the same counters on
                      # a plain copy (profiles/qgemv_w4g128_llama7b_decode_M1_hbm_traffic.txt); not measurable live
-                     "traffic": 15531000 if m == 1 else None, "kernel": "qgemv_w4_kernel<128>" if m <= 2 else "qgemv_kernel<4,128>", "avg_launch_us": round(us_per_launch, 3),
-                     "bytes_per_launch": round(bytes_per_launch)},
+                     "traffic": 15531000 if m == 1 else None, "kernel": "qgemv_w4_kernel<128>" if m <= 2 else "qgemv_tiles_kernel<4,128>", "avg_launch_us": round(us_per_launch, 3),
+                     "bytes_per_launch": round(bytes_per_launch),
+                     "per_shape": per_shape,
+                     # what this board's memory system delivers to a plain device-to-device copy of 1 GiB (read + write)
+                     "copy_gbps": copy_probe(torch)},
     }
 
     if not args.no_extras:
-        del per_layer_graphs
+        del one_step
         result["extras"] = {name: fn(torch, hip, QuantizedLinear, layers) for name, fn in EXTRAS.items()}
 
     if not args.no_cpu:
-        result["cpu_baseline"] = cpu_baseline(bits, g)
+        result["cpu_baseline"] = cpu_baseline()
     print(json.dumps(result))
 
 

@@ -116,3 +116,54 @@ def test_llama_mixed_precision_map():
         got = qmodel(input_ids=ids).logits.float()
         want = twin(input_ids=ids).logits.float()
     assert (got - want).abs().max().item() <= 3e-2 * want.abs().max().item()
+
+
+def test_decoder_step_under_graph_capture_equals_the_eager_step():
+    """bench_decoder.Decoder (the end-to-end configuration of bench.py) on a 2-layer model with the mixed recipe:
+    a decode step captured in a HIP graph and replayed gives the logits and the tokens of the eager step, token
+    after token; and the quantised model agrees with a float16 twin built from the oracle's W16."""
+    import bench_decoder as bd
+    from bitween_amd import Bitween, QuantizedLinear
+    torch.manual_seed(0)
+    with torch.device("cuda"):
+        model = bd.Decoder(layers=2, hidden=256, heads=4, inter=512, vocab=1000, max_len=96).half()
+    model.init_weights(seed=3)
+    recipe = {"layers.0.self_attn": (8, 128), "layers.1.self_attn": (8, 128), "layers.0.mlp": (4, 128),
+              "layers.1.mlp": (4, 128), "layers.1.mlp.down_proj": (2, 32)}
+    q = Bitween(model, bits=4, group_size=128).quantize(rtn=True, ignore_layers=["lm_head", "embed_tokens"],
+                                                        layer_config=recipe, verbose=False)
+    kinds = {name: (m.bits, m.group_size) for name, m in q.named_modules() if isinstance(m, QuantizedLinear)}
+    assert len(kinds) == 14 and kinds["layers.1.mlp.down_proj"] == (2, 32) and kinds["layers.0.self_attn.k_proj"] == (8, 128)
+    assert isinstance(q.lm_head, torch.nn.Linear)
+    q.alloc_state()
+    ids = torch.randint(0, 1000, (40,), device="cuda", generator=torch.Generator(device="cuda").manual_seed(1))
+    _, _, toks_eager = bd.generate(q, ids, 24)
+    # logits of the first decode step, eagerly
+    q.prefill(ids)
+    logits_eager = q.step().clone()
+    graph = bd.capture_step(q)
+    q.prefill(ids)
+    # capture ran one warm-up step: find the captured step's output tensor by replaying
+    graph.replay()
+    torch.cuda.synchronize()
+    assert int(q.pos) == 41
+    assert torch.equal(q.out[40:41], toks_eager[1:2])
+    _, _, toks_graph = bd.generate(q, ids, 24, graph)
+    assert torch.equal(toks_graph, toks_eager)
+    # the float16 twin: same decoder, every quantised linear replaced by nn.Linear holding W16
+    from bitween_amd.kernels import hip_loader as hip
+    twin = copy.deepcopy(q)
+    for name, m in list(twin.named_modules()):
+        if isinstance(m, QuantizedLinear):
+            lin = torch.nn.Linear(m.in_features, m.out_features, bias=False, device="cuda", dtype=torch.float16)
+            lin.weight.data = hip.dequantize(m.qweight, m.scale, m.zero_point, m.group_size, m.bits, torch.float16)
+            parent = twin
+            *path, leaf = name.split(".")
+            for part in path:
+                parent = getattr(parent, part)
+            setattr(parent, leaf, lin)
+    twin.alloc_state()
+    twin.prefill(ids)
+    logits_twin = twin.step()
+    rel = (logits_eager.float() - logits_twin.float()).abs().max() / logits_twin.float().abs().max()
+    assert rel < 2e-2

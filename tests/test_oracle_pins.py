@@ -256,3 +256,37 @@ def test_backward_is_the_adjoint_of_the_forward_and_matches_brute_force():
     lhs = (go.astype(np.float64) * y64).sum()
     rhs = (got * x.astype(np.float64)).sum()
     assert abs(lhs - rhs) <= 1e-9 * max(1.0, abs(lhs))
+
+
+@pytest.mark.parametrize("name", CASES)
+def test_torch_cpu_path_matches_exact_vectors(name):
+    """oracle/torch_cpu_path.py (the eager-torch restatement that bench.py times as the CPU baseline) against the
+    exact-rational vectors, in every dtype the vectors cover: packed words, scale, zero point, the module's
+    float16 buffers, both dequantisations bit for bit; the matmul against the exactly evaluated products."""
+    import torch
+    from oracle import torch_cpu_path as tcp
+    key, fmt, bits, g, _ = _case(name)
+    dt = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}[fmt]
+    w = torch.from_numpy(GOLD[key + "_w"]).to(dt)
+    valid = GOLD[key + "_valid"]
+    qw, scale, zp, _ = tcp.quantize_rtn(w, bits, g)
+    assert scale.dtype == dt and zp.dtype == torch.int32 and qw.dtype == torch.int32
+    assert np.array_equal(zp.numpy()[valid], GOLD[key + "_zp"][valid])
+    assert np.array_equal(scale.float().numpy().view(np.uint32)[valid], GOLD[key + "_scale"].view(np.uint32)[valid])
+    vq = np.repeat(valid, g, axis=1)
+    assert np.array_equal(orc.unpack_words(qw.numpy(), bits)[vq], GOLD[key + "_q"][vq])
+    if fmt != "f32" or not valid.all():
+        return
+    assert np.array_equal(qw.numpy(), GOLD[key + "_qweight"])
+    qw2, s16, z16 = tcp.module_buffers(w.half() if np.array_equal(w.half().float().numpy(), w.numpy()) else w, bits, g)
+    assert np.array_equal(qw2.numpy(), GOLD[key + "_qweight"])
+    assert np.array_equal(s16.numpy().view(np.uint16), GOLD[key + "_scale16"].view(np.uint16))
+    w16 = tcp.dequantize_rtn(qw, s16, z16, g, bits).half()
+    assert np.array_equal(w16.numpy().view(np.uint16), GOLD[key + "_w16"].view(np.uint16))
+    w32 = tcp.dequantize_rtn(qw, scale, zp, g, bits)
+    assert np.array_equal(w32.numpy().view(np.uint32), GOLD[key + "_w32"].view(np.uint32))
+    y = tcp.forward(torch.from_numpy(GOLD[key + "_x"]), qw, s16, z16, None, bits, g).float().numpy()
+    ref = GOLD[key + "_y64"]
+    with np.errstate(over="ignore", invalid="ignore"):
+        finite = np.isfinite(ref.astype(np.float32).astype(np.float16))
+    assert np.abs(y - ref)[finite].max() <= 1e-2 * max(np.abs(ref[finite]).max(), 1e-30)
