@@ -318,6 +318,8 @@ def quantized_input_grad(grad_y, qweight, scale, zero_point, bits, group_size):
         return None
     if grad_y.stride(1) != 1 or grad_y.stride(0) % 8 or grad_y.data_ptr() % 16:
         grad_y = grad_y.contiguous()
+        if grad_y.data_ptr() % 16:                         # contiguous already, but at an odd offset of its storage
+            grad_y = grad_y.clone()
         if grad_y.stride(0) % 8:
             return None
     qweight, scale, zero_point = qweight.contiguous(), scale.contiguous(), zero_point.contiguous()
@@ -329,7 +331,7 @@ def quantized_input_grad(grad_y, qweight, scale, zero_point, bits, group_size):
         st = lib.bw_qdgrad(grad_y.data_ptr(), BW_F16, m, n, grad_y.stride(0), qweight.data_ptr(), scale.data_ptr(),
                            zero_point.data_ptr(), k, bits, group_size, grad_x.data_ptr(), k,
                            None if ws is None else ws.data_ptr(), nbytes, _raw_stream(index))
-    if st == -2:                                           # BW_EUNSUPPORTED: shape outside the fused kernel
+    if st in (-2, -3):                                     # BW_EUNSUPPORTED / BW_EALIGN: the caller's unfused path
         return None
     _check(st, "bw_qdgrad")
     return grad_x

@@ -184,9 +184,10 @@ class _SiblingGroup:
         self.size = len(members)
         self.wasted = 0                                   # launches in a row that served a single member
         row = 0
-        for m in members:
+        for index, m in enumerate(members):
             a, b = row, row + m.out_features
             m.__dict__["_sibling_rows"] = (a, b)
+            m.__dict__["_sibling_index"] = index
             m._buffers["qweight"] = self.qweight[a:b]
             m._buffers["scale"] = self.scale[a:b]
             m._buffers["zero_point"] = self.zero_point[a:b]
@@ -198,10 +199,11 @@ class _SiblingGroup:
         self._version = -1
         self._y = None
         self._served = 0
+        self._served_mask = 0
 
     def __getstate__(self):                                # copies and pickles drop the one-call cache
         state = dict(self.__dict__)
-        state["_x"], state["_version"], state["_y"], state["_served"] = None, -1, None, 0
+        state["_x"], state["_version"], state["_y"], state["_served"], state["_served_mask"] = None, -1, None, 0, 0
         return state
 
     def forward(self, member, x):
@@ -211,7 +213,10 @@ class _SiblingGroup:
         if self.wasted >= 4:
             return None                                    # the members do not share inputs after all: stop grouping
         seen = self._x() if self._x is not None else None
-        if seen is not x or self._version != x._version or self._y is None:
+        bit = 1 << member.__dict__["_sibling_index"]
+        # The cached result serves each member once: a member that comes back with the very same tensor object and
+        # version (an input rewritten in place through .data or by a kernel writing to its address) gets a new launch.
+        if seen is not x or self._version != x._version or self._y is None or self._served_mask & bit:
             self.wasted = self.wasted + 1 if self._served == 1 else 0
             shape = x.shape
             x2 = x.reshape(-1, shape[-1])
@@ -222,8 +227,10 @@ class _SiblingGroup:
             self._x = weakref.ref(x)
             self._version = x._version
             self._served = 0
+            self._served_mask = 0
         out = self._y[..., rng[0]:rng[1]]
         self._served += 1
+        self._served_mask |= bit
         if self._served == self.size:
             self._y = None                                 # everyone has its slice: do not keep the result alive
         return out
@@ -234,7 +241,12 @@ def fuse_sibling_linears(model, sibling_names=(("q_proj", "k_proj", "v_proj"), (
     per launch before a byte moves).  For every module of `model` that has all the children named in one
     tuple of `sibling_names` as QuantizedLinear layers of equal in_features / bits / group_size, those
     children are grouped.  The model's code is unchanged: it still calls each child.  Returns the number of
-    groups formed.  Not part of the reference's interface."""
+    groups formed.  Not part of the reference's interface.
+    A group computes all its members' outputs when the first of them is called with a tensor and hands the others
+    their slices when they are called with that same tensor (same object, same version counter); a member that
+    asks twice gets a new launch.  An input that is rewritten in place without a version bump (through .data, or
+    by a kernel writing to its address) between the calls of two different members is not noticed: change inputs
+    through ordinary torch ops."""
     formed = 0
     for parent in list(model.modules()):
         for names in sibling_names:

@@ -11,8 +11,12 @@
  *     owned by the caller; nothing is allocated, freed or retained.
  *   - `stream` is a hipStream_t passed as void* (NULL = the null stream).
  *     Work is enqueued on it; no entry point synchronises.
- *   - returns BW_OK (0) or a negative bw_status; never throws.  A non-zero
- *     status means nothing was launched.
+ *   - returns BW_OK (0) or a negative bw_status; never throws.  Arguments are
+ *     checked before anything is enqueued: BW_EINVAL, BW_EUNSUPPORTED, BW_EALIGN
+ *     and BW_EWORKSPACE mean nothing was launched.  BW_ELAUNCH (the HIP runtime
+ *     refused a launch) can come from the second launch of a call that makes
+ *     two (bw_qlinear beyond 16 rows, split-K with its reduction): the output
+ *     is then undefined.
  *   - weight layout is the reference's: W is [N][K] (N = out_features,
  *     K = in_features); qweight is int32 [N][K*bits/32], value k of a row in
  *     word k / (32/bits) at bit offset (k % (32/bits)) * bits

@@ -161,24 +161,20 @@ def dequantize_bf16(qweight, scale16, zp16, group_size, bits):
     return _round_to(w32, "bf16")
 
 
-def qlinear_forward(x16, qweight, scale16, zp16, bias16, bits, group_size, act="f16"):
+def qlinear_forward(x16, qweight, scale16, zp16, bias16, bits, group_size):
     """bitween/modules.py:62-106 and main.py:444-466: y = x16 @ W16.T (+ bias),
     float16 out.  The dot product is taken in float64 here; the reference's
     BLAS accumulates in float32, so agreement is to tolerance (1e-2 relative,
-    main.py:471-477), not bit-exact.  Returns (y as float16-or-bf16-valued
-    float32, y64 before any output rounding)."""
-    if act == "f16":
-        w = dequantize_f16(qweight, scale16, zp16, group_size, bits).astype(np.float64)
-        xa = np.asarray(x16, np.float16).astype(np.float64)
-    else:
-        w = dequantize_bf16(qweight, scale16, zp16, group_size, bits).astype(np.float64)
-        xa = _round_to(np.asarray(x16, np.float32), "bf16").astype(np.float64)
+    main.py:471-477), not bit-exact.  Returns (y as float16-valued float32,
+    y64 before any output rounding)."""
+    w = dequantize_f16(qweight, scale16, zp16, group_size, bits).astype(np.float64)
+    xa = np.asarray(x16, np.float16).astype(np.float64)
     y64 = xa @ w.T
-    y = _round_to(y64.astype(np.float32), act)
+    y = _round_to(y64.astype(np.float32), "f16")
     if bias16 is not None:
         b = np.asarray(bias16).astype(np.float32)
         y64 = y64 + b.astype(np.float64)
-        y = _round_to(y + b, act)                      # second rounding, modules.py:100-101
+        y = _round_to(y + b, "f16")                    # second rounding, modules.py:100-101
     return y, y64
 
 

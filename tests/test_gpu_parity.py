@@ -781,3 +781,26 @@ def test_prefill_llama3_8b_mlp_shapes_at_full_size(k, n, m, xdtype):
         for r, c in hot.items():
             assert torch.equal(y[r], w16[:, c])
         check_matmul(y[:, rows], x_np, qw_o, s16, z16, None, bits, g)
+
+
+def test_sibling_group_does_not_serve_a_member_twice_from_its_cache():
+    """An input rewritten in place without a version bump (.data) and handed to the same member again gets a new
+    launch, not the cached slice."""
+    import bitween_amd
+    torch.manual_seed(0)
+    blk = torch.nn.Module()
+    for name in ("q_proj", "k_proj", "v_proj"):
+        lin = torch.nn.Linear(256, 128, bias=False, device="cuda", dtype=torch.float16)
+        setattr(blk, name, bitween_amd.QuantizedLinear.from_float(lin, 4, 128))
+    assert bitween_amd.fuse_sibling_linears(blk) == 1
+    x = torch.randn(1, 256, device="cuda", dtype=torch.float16)
+    with torch.no_grad():
+        y1 = blk.q_proj(x).clone()
+        version = x._version
+        x.data.mul_(2.0)
+        assert x._version == version                      # the rewrite is invisible to the version counter
+        y2 = blk.q_proj(x)
+        k2 = blk.k_proj(x)
+    assert torch.allclose(y2.float(), 2 * y1.float(), rtol=2e-3, atol=1e-3)
+    ref_k = bitween_amd.kernels.hip_loader.quantized_matmul_hip(x, blk.k_proj.qweight, blk.k_proj.scale, blk.k_proj.zero_point, None, 4, 128)
+    assert torch.equal(k2, ref_k)

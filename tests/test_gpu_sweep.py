@@ -2,11 +2,14 @@
 every kernel switch (1, 2, 16, 32 / 48, split-K or not), bias on and off, float16 and bfloat16 activations.
 
 The expected value is a float64 matmul on the GPU over the library's own bit-exact dequantisation (which
-tests/test_gpu_parity.py pins against the oracle and the exact vectors), so hundreds of cases run in seconds; the
+tests/test_gpu_parity.py pins against the oracle and the exact vectors, and every tenth case here compares with
+the oracle's again), so hundreds of cases run in seconds; the
 bound is elementwise: one float16 rounding of the result plus float32 accumulation error on sum |x| |w|."""
 import numpy as np
 import pytest
 import torch
+
+from oracle import rtn_oracle as orc
 
 pytestmark = pytest.mark.gpu
 
@@ -30,7 +33,14 @@ def _run(seed, cases, max_groups, max_n):
         dt = torch.bfloat16 if rng.integers(0, 4) == 0 else torch.float16
         x = torch.randn(m, k, device="cuda").to(dt)
         y = hip.quantized_matmul_hip(x, qw, s, z, bias, bits, g)
-        w16 = hip.dequantize(qw, s, z, g, bits, torch.float16).double()
+        w16 = hip.dequantize(qw, s, z, g, bits, torch.float16)
+        if it % 10 == 0:
+            # every tenth case: the expected weights straight from the oracle, so the sweep does not rest on the
+            # library's own dequantisation alone
+            w16_o = orc.dequantize_f16(qw.cpu().numpy(), s.cpu().numpy(), z.cpu().numpy(), g, bits)
+            assert np.array_equal(w16.cpu().numpy().view(np.uint16) & 0x7FFF | ((w16.cpu().numpy() != 0) * (w16.cpu().numpy().view(np.uint16) & 0x8000)),
+                                  w16_o.view(np.uint16) & 0x7FFF | ((w16_o != 0) * (w16_o.view(np.uint16) & 0x8000)))
+        w16 = w16.double()
         x64 = x.to(torch.float16).double()
         ref = x64 @ w16.T
         if bias is not None:
