@@ -628,6 +628,9 @@ def main():
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--only", choices=sorted(EXTRAS), default=None,
                     help="run just this section of the extras and print it (used for profiling one kernel)")
+    ap.add_argument("--probe", default=None, metavar="K,N,M,BITS,GROUP",
+                    help="run only eager decode launches of this one shape over 12 rotating layer copies (one dispatch per "
+                         "launch, for rocprofv3 counter runs) and print their device time")
     ap.add_argument("--copy-probe", action="store_true",
                     help="run only a plain 256 MiB device copy a few times (calibrates rocprof FETCH_SIZE/WRITE_SIZE)")
     args = ap.parse_args()
@@ -650,6 +653,15 @@ def main():
             dst.copy_(src)
         torch.cuda.synchronize()
         print(json.dumps({"copy_probe_bytes": 256 << 20, "launches": 5, "copy_gbps_1GiB": copy_probe(torch)}))
+        return
+
+    if args.probe:
+        pk, pn, pm, pb, pg = (int(v) for v in args.probe.split(","))
+        qs = [make_layer(torch, QuantizedLinear, pk, pn, pb, pg, seed=i, outliers=True) for i in range(12)]
+        x = torch.randn(pm, pk, device="cuda", dtype=torch.float16)
+        us = time_calls(torch, lambda: [hip.quantized_matmul_hip(x, q.qweight, q.scale, q.zero_point, None, pb, pg) for q in qs], 3, 1) / 12
+        print(json.dumps({"probe": args.probe, "launches": 48, "eager_us_per_launch": round(us, 2),
+                          "bytes": decode_bytes(pm, pk, pn, pb, pg)}))
         return
 
     layers = [[make_layer(torch, QuantizedLinear, k, n, bits, g, seed=100 * li + i)
