@@ -505,8 +505,9 @@ def extras_llama7b_decoder_graph(torch, hip, QuantizedLinear, layers):
     heads, MLP 11008, vocab 32000, random weights), Bitween(...).quantize(rtn=True, ignore_layers=[lm_head,
     embed_tokens], layer_config = attention 8-bit g128, MLP 4-bit g128, down_proj of layers 0, 1, 30, 31 2-bit g32),
     then a 512-token random prompt and 256 greedy tokens at batch 1 with one decode step captured in a HIP graph
-    and replayed.  The glue (RMSNorm, rotary, cache update, attention, SwiGLU) is plain torch: about 20 small
-    launches per layer next to the 4-7 of the linears."""
+    and replayed.  The glue (RMSNorm, rotary, cache update, attention, SwiGLU) is plain torch - about 17 small
+    launches per layer next to the 4-7 of the linears - or, in the *_hip_glue entries, the five fused kernels of
+    bench_decoder_glue.hip (6 launches per layer)."""
     import bitween_amd
     import bench_decoder as bd
     nlayers, prompt, new_tokens = 32, 512, 256
@@ -529,9 +530,16 @@ def extras_llama7b_decoder_graph(torch, hip, QuantizedLinear, layers):
     res["bytes_per_token_quantized_linears"] = by
     res["byte_ceiling_tokens_per_s"] = round(HBM_PEAK_GBPS * 1e9 / by_all, 1)
     qmodel.alloc_state()
-    for label, fuse in (("per_module_launches", False), ("fused_siblings", True)):
-        if fuse:
+    fused = False
+    for label, fuse, hip_glue in (("per_module_launches", False, False), ("per_module_launches_hip_glue", False, True),
+                                  ("fused_siblings", True, False), ("fused_siblings_hip_glue", True, True)):
+        if fuse and not fused:
             bitween_amd.fuse_sibling_linears(qmodel)
+            fused = True
+        if hip_glue:
+            qmodel.use_hip_glue(splits=12)
+        else:
+            qmodel.glue = None
         bd.generate(qmodel, ids, 4)                                   # warm every kernel and the allocator
         graph = bd.capture_step(qmodel)
         pre_ms, dec_s, toks = bd.generate(qmodel, ids, new_tokens, graph)

@@ -12,14 +12,91 @@ captured in a HIP graph and replayed without the Python interpreter in the way:
   * the position, the current token and the generated tokens live in device tensors that the step itself
     advances, so replaying the captured step N times generates N tokens with no host round trip.
 
+With use_hip_glue() the decode step runs the same arithmetic through five small HIP kernels of this benchmark
+(bench_decoder_glue.hip: residual add + RMSNorm, rotary + cache write, split attention + combine, SwiGLU) instead
+of about seventeen torch kernels per layer; the prompt always goes through the torch ops.
+
 Random weights N(0, 0.02) from a seed (no checkpoint can be fetched); the numbers say how fast the path runs,
 not what it generates.
 """
+import ctypes
+import os
+import subprocess
 import time
 
 import torch
 import torch.nn as nn
 import torch.nn.functional as F
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+GLUE_SRC = os.path.join(HERE, "bench_decoder_glue.hip")
+GLUE_LIB = os.path.join(HERE, "bench_decoder_glue.so")
+
+
+def build_glue():
+    """hipcc the glue kernels for gfx950 into bench_decoder_glue.so next to this file (works without a GPU)."""
+    cmd = [os.environ.get("HIPCC", "/opt/rocm/bin/hipcc"), "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
+           "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-o", GLUE_LIB, GLUE_SRC]
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError("hipcc failed:\n" + proc.stderr)
+    return GLUE_LIB
+
+
+class HipGlue:
+    """ctypes front of bench_decoder_glue.so for one Decoder: every call launches on torch's current stream."""
+
+    def __init__(self, model, splits=12):
+        if not os.path.exists(GLUE_LIB):
+            raise RuntimeError(f"{GLUE_LIB} is not built: run bench_decoder.build_glue() (or __graft_entry__.build()) first")
+        lib = ctypes.CDLL(GLUE_LIB)
+        vp, i32, f32 = ctypes.c_void_p, ctypes.c_int32, ctypes.c_float
+        lib.glue_add_rmsnorm.argtypes = [vp, vp, vp, vp, vp, i32, f32, vp]
+        lib.glue_rope_kv.argtypes = [vp] * 9 + [i32, i32, i32, vp]
+        lib.glue_attention.argtypes = [vp] * 6 + [i32, i32, i32, i32, f32, vp]
+        lib.glue_silu_mul.argtypes = [vp, vp, vp, i32, vp]
+        for f in (lib.glue_add_rmsnorm, lib.glue_rope_kv, lib.glue_attention, lib.glue_silu_mul):
+            f.restype = i32
+        self.lib, self.m, self.splits = lib, model, splits
+        dev = model.lm_head.weight.device
+        self.index = dev.index if dev.index is not None else torch.cuda.current_device()
+        self.part = torch.empty(model.heads * splits * (model.head_dim + 2), dtype=torch.float32, device=dev)
+
+    def _stream(self):
+        return torch._C._cuda_getCurrentRawStream(self.index)
+
+    @staticmethod
+    def _ok(st, what):
+        if st:
+            raise RuntimeError(f"{what} refused its arguments or failed to launch (status {st})")
+
+    def add_rmsnorm(self, x, delta, gamma):
+        m = self.m
+        x_out, h = torch.empty_like(x), torch.empty_like(x)
+        self._ok(self.lib.glue_add_rmsnorm(x.data_ptr(), None if delta is None else delta.data_ptr(), gamma.data_ptr(), x_out.data_ptr(),
+                                           h.data_ptr(), m.hidden, m.eps, self._stream()), "glue_add_rmsnorm")
+        return x_out, h
+
+    def rope_kv(self, q, k, v, layer):
+        m = self.m
+        q_out = torch.empty(1, m.hidden, dtype=torch.float16, device=q.device)
+        self._ok(self.lib.glue_rope_kv(q.data_ptr(), k.data_ptr(), v.data_ptr(), m.cos.data_ptr(), m.sin.data_ptr(), m.pos.data_ptr(),
+                                       q_out.data_ptr(), m.kv[layer, 0].data_ptr(), m.kv[layer, 1].data_ptr(), m.heads, m.head_dim,
+                                       m.max_len, self._stream()), "glue_rope_kv")
+        return q_out
+
+    def attention(self, q, layer):
+        m = self.m
+        o = torch.empty(1, m.hidden, dtype=torch.float16, device=q.device)
+        self._ok(self.lib.glue_attention(q.data_ptr(), m.kv[layer, 0].data_ptr(), m.kv[layer, 1].data_ptr(), m.pos.data_ptr(),
+                                         self.part.data_ptr(), o.data_ptr(), m.heads, m.head_dim, m.max_len, self.splits,
+                                         m.head_dim ** -0.5, self._stream()), "glue_attention")
+        return o
+
+    def silu_mul(self, gate, up):
+        out = torch.empty_like(gate)
+        self._ok(self.lib.glue_silu_mul(gate.data_ptr(), up.data_ptr(), out.data_ptr(), gate.numel(), self._stream()), "glue_silu_mul")
+        return out
 
 
 class Attention(nn.Module):
@@ -60,6 +137,11 @@ class Decoder(nn.Module):
         self.layers = nn.ModuleList([Layer(hidden, heads, inter) for _ in range(layers)])
         self.norm = nn.Parameter(torch.ones(hidden))
         self.lm_head = nn.Linear(hidden, vocab, bias=False)
+        self.glue = None
+
+    def use_hip_glue(self, splits=12):
+        """Run step() through the HIP glue kernels (head dimension 128, float16 parameters; call after alloc_state)."""
+        self.glue = HipGlue(self, splits)
 
     @torch.no_grad()
     def init_weights(self, seed):
@@ -137,10 +219,32 @@ class Decoder(nn.Module):
         self.out.index_copy_(0, self.pos - 1, self.tok[0])
         return logits
 
+    def _step_hip(self):
+        """step() with the glue of a layer in five launches: the residual add of a block is folded into the RMSNorm
+        that follows it."""
+        g = self.glue
+        x = self.embed_tokens(self.tok[0])
+        delta = None
+        for i, layer in enumerate(self.layers):
+            att, mlp = layer.self_attn, layer.mlp
+            x, h = g.add_rmsnorm(x, delta, layer.input_layernorm)
+            q = g.rope_kv(att.q_proj(h), att.k_proj(h), att.v_proj(h), i)
+            delta = att.o_proj(g.attention(q, i))
+            x, h = g.add_rmsnorm(x, delta, layer.post_attention_layernorm)
+            delta = mlp.down_proj(g.silu_mul(mlp.gate_proj(h), mlp.up_proj(h)))
+        _, h = g.add_rmsnorm(x, delta, self.norm)
+        return self.lm_head(h)
+
     @torch.no_grad()
     def step(self):
         """Feed tok at position pos, choose the next token greedily, advance: every tensor it touches is static, so
         the call can be captured once and replayed."""
+        if self.glue is not None:
+            logits = self._step_hip()
+            self.tok.copy_(logits.argmax(-1, keepdim=True))
+            self.out.index_copy_(0, self.pos, self.tok[0])
+            self.pos.add_(1)
+            return logits
         x = self.embed_tokens(self.tok[0])
         self._cos, self._sin = self.cos.index_select(0, self.pos)[:, None, :], self.sin.index_select(0, self.pos)[:, None, :]
         # additive attention bias [heads, 1, max_len]: 0 up to the current position, -inf behind it
