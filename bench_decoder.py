@@ -55,7 +55,8 @@ class HipGlue:
         lib.glue_rope_kv.argtypes = [vp] * 9 + [i32, i32, i32, vp]
         lib.glue_attention.argtypes = [vp] * 6 + [i32, i32, i32, i32, f32, vp]
         lib.glue_silu_mul.argtypes = [vp, vp, vp, i32, vp]
-        for f in (lib.glue_add_rmsnorm, lib.glue_rope_kv, lib.glue_attention, lib.glue_silu_mul):
+        lib.glue_rope_attention.argtypes = [vp] * 10 + [i32, i32, i32, i32, f32, vp]
+        for f in (lib.glue_add_rmsnorm, lib.glue_rope_kv, lib.glue_attention, lib.glue_rope_attention, lib.glue_silu_mul):
             f.restype = i32
         self.lib, self.m, self.splits = lib, model, splits
         dev = model.lm_head.weight.device
@@ -91,6 +92,16 @@ class HipGlue:
         self._ok(self.lib.glue_attention(q.data_ptr(), m.kv[layer, 0].data_ptr(), m.kv[layer, 1].data_ptr(), m.pos.data_ptr(),
                                          self.part.data_ptr(), o.data_ptr(), m.heads, m.head_dim, m.max_len, self.splits,
                                          m.head_dim ** -0.5, self._stream()), "glue_attention")
+        return o
+
+    def rope_attention(self, q, k, v, layer):
+        """rope_kv and attention in one call (two launches)."""
+        m = self.m
+        o = torch.empty(1, m.hidden, dtype=torch.float16, device=q.device)
+        self._ok(self.lib.glue_rope_attention(q.data_ptr(), k.data_ptr(), v.data_ptr(), m.cos.data_ptr(), m.sin.data_ptr(), m.pos.data_ptr(),
+                                              m.kv[layer, 0].data_ptr(), m.kv[layer, 1].data_ptr(), self.part.data_ptr(), o.data_ptr(),
+                                              m.heads, m.head_dim, m.max_len, self.splits, m.head_dim ** -0.5, self._stream()),
+                 "glue_rope_attention")
         return o
 
     def silu_mul(self, gate, up):
@@ -221,15 +232,14 @@ class Decoder(nn.Module):
 
     def _step_hip(self):
         """step() with the glue of a layer in five launches: the residual add of a block is folded into the RMSNorm
-        that follows it."""
+        that follows it, the rotary embedding and the cache write into the attention."""
         g = self.glue
         x = self.embed_tokens(self.tok[0])
         delta = None
         for i, layer in enumerate(self.layers):
             att, mlp = layer.self_attn, layer.mlp
             x, h = g.add_rmsnorm(x, delta, layer.input_layernorm)
-            q = g.rope_kv(att.q_proj(h), att.k_proj(h), att.v_proj(h), i)
-            delta = att.o_proj(g.attention(q, i))
+            delta = att.o_proj(g.rope_attention(att.q_proj(h), att.k_proj(h), att.v_proj(h), i))
             x, h = g.add_rmsnorm(x, delta, layer.post_attention_layernorm)
             delta = mlp.down_proj(g.silu_mul(mlp.gate_proj(h), mlp.up_proj(h)))
         _, h = g.add_rmsnorm(x, delta, self.norm)

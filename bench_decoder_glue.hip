@@ -2,13 +2,15 @@
 // Llama-shaped layer when ONE token is decoded.  Not part of the quantized-linear library and not in its ABI: the
 // benchmark measures that library inside a whole decode step, and with one torch kernel per elementwise operation
 // (about seventeen small launches per layer) the step spends three quarters of its time between the linears.
-// Five kernels, each a single launch, all float16 in memory with float32 arithmetic:
+// All float16 in memory with float32 arithmetic:
 //
 //   glue_add_rmsnorm     x_out = x + delta (rounded to float16); h = x_out * rsqrt(mean(x_out^2) + eps) * gamma
 //   glue_rope_kv         rotate q and k of the new token by the angle of its position; q -> q_out, k and v -> the
 //                        KV cache row of that position
-//   glue_attn_partial    one query row against a slice of the cache: scores, softmax numerators, weighted sum of v
-//   glue_attn_combine    the slices of a head -> the attention output
+//   glue_attention       one query row against the cache, in two launches: per slice of the cache the scores, softmax
+//                        numerators and weighted sum of v; then the slices of a head -> the attention output
+//   glue_rope_attention  the three above in two launches: the attention workgroups rotate q themselves and the one
+//                        whose slice holds the new position rotates k and writes k and v into the cache first
 //   glue_silu_mul        silu(gate) * up
 //
 // The position is read from device memory by the kernels, so a captured step can be replayed while the position
@@ -90,15 +92,22 @@ __global__ __launch_bounds__(256) void rope_kv_kernel(const _Float16* q, const _
 // grid (heads, splits), 256 threads; head dimension 128.  Slice s of the n = pos + 1 cached positions is
 // [s * chunk, min(n, (s + 1) * chunk)) with chunk = ceil(n / splits) <= 256 (checked on the host against max_len).
 // part[(head * splits + s) * 130]: 128 unnormalised output values, the slice's score maximum, its sum of numerators.
+// ROPE: q is the unrotated query and k_new / v_new the new token's key and value; every workgroup rotates its head's
+// query itself, and the one whose slice holds position pos rotates the key, writes key and value into the cache
+// and reads them back like any other row (a workgroup sees its own writes after a barrier).
 constexpr int kD = 128, kMaxChunk = 256;
-__global__ __launch_bounds__(256) void attn_partial_kernel(const _Float16* q, const _Float16* kcache, const _Float16* vcache,
-                                                           const int64_t* pos_ptr, float* part, int max_len, int splits, float scale) {
+template <bool ROPE>
+__global__ __launch_bounds__(256) void attn_partial_kernel(const _Float16* q, const _Float16* k_new, const _Float16* v_new,
+                                                           const _Float16* cos_t, const _Float16* sin_t, _Float16* kcache,
+                                                           _Float16* vcache, const int64_t* pos_ptr, float* part, int max_len,
+                                                           int splits, float scale) {
     __shared__ float qs[kD];
     __shared__ float sc[kMaxChunk];
     __shared__ float red[8];
     __shared__ float oacc[16][kD];
     const int tid = threadIdx.x, head = blockIdx.x, split = blockIdx.y;
-    int64_t n = *pos_ptr + 1;                                   // the new token's k and v are already in the cache
+    const int64_t pos = *pos_ptr;
+    int64_t n = pos + 1;                                        // the new token's position is part of the cache
     if (n > max_len) n = max_len;
     if (n < 0) n = 0;
     const int chunk = (int)((n + splits - 1) / splits);
@@ -108,6 +117,31 @@ __global__ __launch_bounds__(256) void attn_partial_kernel(const _Float16* q, co
         if (tid < kD) out[tid] = 0.f;
         if (tid == 0) { out[kD] = -INFINITY; out[kD + 1] = 0.f; }
         return;
+    }
+    if constexpr (ROPE) {
+        constexpr int half = kD / 2;
+        const bool owner = pos >= p0 && pos < p1;               // then 0 <= pos < max_len
+        const int64_t pc = pos < 0 ? 0 : (pos < max_len ? pos : max_len - 1);
+        if (tid < half || (owner && tid < 2 * half)) {
+            const int i = tid & (half - 1);
+            const _Float16* src = (tid < half ? q : k_new) + head * kD;
+            const float x1 = (float)src[i], x2 = (float)src[i + half];
+            const float c = (float)cos_t[pc * half + i], sn = (float)sin_t[pc * half + i];
+            const _Float16 o1 = (_Float16)(x1 * c - x2 * sn), o2 = (_Float16)(x2 * c + x1 * sn);
+            if (tid < half) {
+                qs[i] = (float)o1;
+                qs[i + half] = (float)o2;
+            } else {
+                _Float16* dst = kcache + ((int64_t)head * max_len + pos) * kD;
+                dst[i] = o1;
+                dst[i + half] = o2;
+            }
+        } else if (owner && tid < 3 * half) {
+            const int i = 2 * (tid - 2 * half);
+            *reinterpret_cast<h2*>(vcache + ((int64_t)head * max_len + pos) * kD + i) = *reinterpret_cast<const h2*>(v_new + head * kD + i);
+        }
+        __threadfence_block();
+        __syncthreads();
     }
     // v of the first 64 positions of the slice: requested now, used after the softmax (16 lanes per position, 8 values
     // of the head dimension each, 16 positions per pass, four passes in registers)
@@ -119,8 +153,10 @@ __global__ __launch_bounds__(256) void attn_partial_kernel(const _Float16* q, co
         const int p = 16 * u + ps;
         vv[u] = *reinterpret_cast<const h8*>(vbase + (int64_t)(p < cnt ? p : 0) * kD);
     }
-    if (tid < kD) qs[tid] = (float)q[head * kD + tid];
-    __syncthreads();
+    if constexpr (!ROPE) {
+        if (tid < kD) qs[tid] = (float)q[head * kD + tid];
+        __syncthreads();
+    }
     // scores: 4 lanes per position, 32 values of the head dimension each
     const int part4 = tid & 3;
     for (int pi = tid >> 2; pi < cnt; pi += 64) {
@@ -253,8 +289,25 @@ extern "C" int glue_attention(const void* q, const void* kcache, const void* vca
                               int D, int max_len, int splits, float scale, void* stream) {
     if (!q || !kcache || !vcache || !pos || !part || !o || heads < 1 || D != kD || max_len < 1 || splits < 1 || splits > kMaxSplits) return -1;
     if ((max_len + splits - 1) / splits > kMaxChunk || !aligned16(kcache) || !aligned16(vcache)) return -1;
-    hipLaunchKernelGGL(attn_partial_kernel, dim3(heads, splits), dim3(256), 0, (hipStream_t)stream, (const _Float16*)q,
-                       (const _Float16*)kcache, (const _Float16*)vcache, (const int64_t*)pos, (float*)part, max_len, splits, scale);
+    hipLaunchKernelGGL(attn_partial_kernel<false>, dim3(heads, splits), dim3(256), 0, (hipStream_t)stream, (const _Float16*)q,
+                       (const _Float16*)nullptr, (const _Float16*)nullptr, (const _Float16*)nullptr, (const _Float16*)nullptr,
+                       (_Float16*)const_cast<void*>(kcache), (_Float16*)const_cast<void*>(vcache), (const int64_t*)pos, (float*)part,
+                       max_len, splits, scale);
+    if (hipGetLastError() != hipSuccess) return -2;
+    hipLaunchKernelGGL(attn_combine_kernel, dim3(heads), dim3(kD), 0, (hipStream_t)stream, (const float*)part, (_Float16*)o, splits);
+    return launched();
+}
+
+// glue_rope_kv and glue_attention in one: q, k, v are the new token's unrotated projections
+extern "C" int glue_rope_attention(const void* q, const void* k, const void* v, const void* cos_t, const void* sin_t, const void* pos,
+                                   void* kcache, void* vcache, void* part, void* o, int heads, int D, int max_len, int splits,
+                                   float scale, void* stream) {
+    if (!q || !k || !v || !cos_t || !sin_t || !pos || !kcache || !vcache || !part || !o) return -1;
+    if (heads < 1 || D != kD || max_len < 1 || splits < 1 || splits > kMaxSplits || (max_len + splits - 1) / splits > kMaxChunk) return -1;
+    if (!aligned16(kcache) || !aligned16(vcache) || (reinterpret_cast<uintptr_t>(v) & 3)) return -1;
+    hipLaunchKernelGGL(attn_partial_kernel<true>, dim3(heads, splits), dim3(256), 0, (hipStream_t)stream, (const _Float16*)q,
+                       (const _Float16*)k, (const _Float16*)v, (const _Float16*)cos_t, (const _Float16*)sin_t, (_Float16*)kcache,
+                       (_Float16*)vcache, (const int64_t*)pos, (float*)part, max_len, splits, scale);
     if (hipGetLastError() != hipSuccess) return -2;
     hipLaunchKernelGGL(attn_combine_kernel, dim3(heads), dim3(kD), 0, (hipStream_t)stream, (const float*)part, (_Float16*)o, splits);
     return launched();

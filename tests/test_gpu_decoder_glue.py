@@ -69,6 +69,12 @@ def test_rope_cache_write_and_attention(small, pos):
     scores = torch.einsum("hd,hnd->hn", q_rot.view(32, 128).float(), kc) * 128 ** -0.5
     want = torch.einsum("hn,hnd->hd", torch.softmax(scores, dim=-1), vc)
     assert rel(o.view(32, 128), want) < 2e-3
+    # the same in one call: rotary, cache write and attention (from the caches as they were before)
+    kv_split = m.kv.clone()
+    m.kv.copy_(kv_before)
+    o_fused = m.glue.rope_attention(q, k, v, 0)
+    assert torch.equal(m.kv, kv_split)
+    assert rel(o_fused, o) < 1e-3
 
 
 def test_silu_mul(small):
