@@ -641,6 +641,9 @@ def main():
                          "launch, for rocprofv3 counter runs) and print their device time")
     ap.add_argument("--copy-probe", action="store_true",
                     help="run only a plain 256 MiB device copy a few times (calibrates rocprof FETCH_SIZE/WRITE_SIZE)")
+    ap.add_argument("--decoder-probe", action="store_true",
+                    help="run only the end-to-end decoder (sibling launches fused, HIP glue): quantize, 512-token prompt, then "
+                         "64 replays of the captured decode step (for rocprofv3 kernel traces of a whole token)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one GPU: this path is a single-device operator and every box here has one GPU; "
@@ -661,6 +664,24 @@ def main():
             dst.copy_(src)
         torch.cuda.synchronize()
         print(json.dumps({"copy_probe_bytes": 256 << 20, "launches": 5, "copy_gbps_1GiB": copy_probe(torch)}))
+        return
+
+    if args.decoder_probe:
+        import bitween_amd
+        import bench_decoder as bd
+        with torch.device("cuda"):
+            model = bd.Decoder(layers=32, max_len=768).half()
+        model.init_weights(seed=0)
+        qmodel = bitween_amd.Bitween(model, bits=4, group_size=128).quantize(
+            rtn=True, ignore_layers=["lm_head", "embed_tokens"], layer_config=bd.mixed_recipe(32), verbose=False)
+        qmodel.alloc_state()
+        bitween_amd.fuse_sibling_linears(qmodel)
+        qmodel.use_hip_glue()
+        ids = torch.randint(0, 32000, (512,), device="cuda", generator=torch.Generator(device="cuda").manual_seed(0))
+        bd.generate(qmodel, ids, 4)
+        graph = bd.capture_step(qmodel)
+        _, dec_s, _ = bd.generate(qmodel, ids, 65, graph)
+        print(json.dumps({"decoder_probe": "32 layers, fused siblings, HIP glue", "replays": 64, "decode_ms_per_token": round(dec_s / 64 * 1e3, 3)}))
         return
 
     if args.probe:
