@@ -207,6 +207,71 @@ __global__ __launch_bounds__(256) void quantize_pack_generic_kernel(const void* 
     qweight[idx] = (int32_t)word;
 }
 
+// float64 weights (functional.py:3-45 is dtype-agnostic: a float64 tensor is quantised in float64 arithmetic and
+// returns a float64 scale).  Rare, so the simple layout: one thread per packed word scanning the group(s) of its
+// values; every operation is the IEEE double operation the reference's eager ops perform.
+__global__ __launch_bounds__(256) void quantize_pack_f64_kernel(const double* __restrict__ w, const double* __restrict__ delta,
+                                                                int64_t N, int K, int64_t ldw, int64_t ldd, int bits, int group,
+                                                                int32_t* __restrict__ qweight, double* __restrict__ scale,
+                                                                int32_t* __restrict__ zp, int recip) {
+    const int vpi = 32 / bits, words = K / vpi, groups = K / group;
+    const double qmax = (double)((1 << bits) - 1);
+    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= N * (int64_t)words) return;
+    const int64_t row = idx / words;
+    const int wcol = (int)(idx - row * words);
+    uint32_t word = 0;
+    int gprev = -1;
+    double s = 0.0, zf = 0.0;
+    auto value = [&](int k) {
+        double x = w[row * ldw + k];
+        if (delta) x = __dadd_rn(x, delta[row * ldd + k]);
+        return x;
+    };
+    for (int i = 0; i < vpi; i++) {
+        const int k = wcol * vpi + i, g = k / group;
+        if (g != gprev) {
+            double lo = value(g * group), hi = lo;
+            for (int e = 1; e < group; e++) {
+                const double x = value(g * group + e);
+                lo = fmin(lo, x);
+                hi = fmax(hi, x);
+            }
+            const double range = __dsub_rn(hi, lo);
+            s = recip ? __dmul_rn(range, __ddiv_rn(1.0, qmax)) : __ddiv_rn(range, qmax);
+            s = fmax(s, 1e-8);
+            zf = fmin(fmax(rint(__ddiv_rn(-lo, s)), 0.0), qmax);
+            gprev = g;
+            if (k == g * group) {
+                scale[row * groups + g] = s;
+                zp[row * groups + g] = (int32_t)zf;
+            }
+        }
+        const double t = rint(__dadd_rn(__ddiv_rn(value(k), s), zf));
+        word |= (uint32_t)(int)fmin(fmax(t, 0.0), qmax) << (i * bits);
+    }
+    qweight[idx] = (int32_t)word;
+}
+
+// functional.py:70 with a float64 scale: scale * (q.float() - zp.float()) promotes to float64; q - zp is exact.
+__global__ __launch_bounds__(256) void dequantize_f64_kernel(const uint32_t* __restrict__ qweight, const double* __restrict__ scale,
+                                                             const void* __restrict__ zp, int zp_dtype, int64_t N, int K, int bits,
+                                                             int group, double* __restrict__ out, int64_t ldo) {
+    const int vpi = 32 / bits, words = K / vpi, groups = K / group;
+    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= N * (int64_t)words) return;
+    const int64_t row = idx / words;
+    const int wcol = (int)(idx - row * words);
+    const uint32_t word = qweight[idx], mask = (1u << bits) - 1;
+    for (int i = 0; i < vpi; i++) {
+        const int k = wcol * vpi + i;
+        const int64_t gi = row * groups + k / group;
+        const float z = zp_dtype == BW_I32 ? (float)((const int32_t*)zp)[gi] : (float)((const _Float16*)zp)[gi];
+        const float d = __fsub_rn((float)((word >> (i * bits)) & mask), z);
+        out[row * ldo + k] = __dmul_rn(scale[gi], (double)d);
+    }
+}
+
 // out[n][k] = scale * (q - zp): float32 product, rounded once to the output type.  A thread owns one packed word
 // (32 / BITS weights); grid.x runs along the row, grid.y over rows.  VEC: the row pitch and base of `out` allow
 // 16-byte stores (8-byte for the 8 bytes an 8-bit word becomes in a 16-bit type).
@@ -397,6 +462,17 @@ extern "C" int bw_quantize_pack_add(const void* w, const void* delta, int w_dtyp
     const int recip = (math_dtype & BW_SCALE_RECIPROCAL) != 0;
     math_dtype &= ~BW_SCALE_RECIPROCAL;
     if (!bw_shape_ok(N, K, bits, group) || ldw < K || (delta && ldd < K)) return BW_EINVAL;
+    if (w_dtype == BW_F64) {
+        // float64 in, float64 arithmetic, float64 scale, int32 zero point: what the reference returns for such a tensor
+        if (math_dtype != BW_F64 || scale_dtype != BW_F64 || zp_dtype != BW_I32) return BW_EINVAL;
+        if (!bw_aligned(w, 8) || !bw_aligned(qweight, 4) || !bw_aligned(scale, 8) || !bw_aligned(zp, 4) || (delta && !bw_aligned(delta, 8)))
+            return BW_EALIGN;
+        const int64_t total = N * (K / (32 / bits));
+        hipLaunchKernelGGL(quantize_pack_f64_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
+                           (const double*)w, (const double*)delta, N, (int)K, ldw, ldd, bits, group, qweight, (double*)scale,
+                           (int32_t*)zp, recip);
+        return hipGetLastError() == hipSuccess ? BW_OK : BW_ELAUNCH;
+    }
     if (w_dtype != BW_F16 && w_dtype != BW_BF16 && w_dtype != BW_F32) return BW_EINVAL;
     if (scale_dtype != BW_F32 && scale_dtype != BW_F16 && scale_dtype != BW_BF16) return BW_EINVAL;
     if (zp_dtype != BW_I32 && zp_dtype != BW_F16 && zp_dtype != BW_BF16) return BW_EINVAL;
@@ -426,6 +502,14 @@ extern "C" int bw_dequantize(const int32_t* qweight, const void* scale, int scal
                              void* stream) {
     if (!qweight || !scale || !zp || !w_out) return BW_EINVAL;
     if (!bw_shape_ok(N, K, bits, group) || ldo < K) return BW_EINVAL;
+    if (scale_dtype == BW_F64 || out_dtype == BW_F64) {
+        if (scale_dtype != BW_F64 || out_dtype != BW_F64 || (zp_dtype != BW_I32 && zp_dtype != BW_F16)) return BW_EINVAL;
+        if (!bw_aligned(scale, 8) || !bw_aligned(w_out, 8)) return BW_EALIGN;
+        const int64_t total = N * (K / (32 / bits));
+        hipLaunchKernelGGL(dequantize_f64_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
+                           (const uint32_t*)qweight, (const double*)scale, zp, zp_dtype, N, (int)K, bits, group, (double*)w_out, ldo);
+        return hipGetLastError() == hipSuccess ? BW_OK : BW_ELAUNCH;
+    }
     if (scale_dtype != BW_F32 && scale_dtype != BW_F16) return BW_EINVAL;
     if (zp_dtype != BW_I32 && zp_dtype != BW_F16) return BW_EINVAL;
     if (out_dtype != BW_F32 && out_dtype != BW_F16 && out_dtype != BW_BF16) return BW_EINVAL;
@@ -467,7 +551,7 @@ extern "C" int bw_dequantize(const int32_t* qweight, const void* scale, int scal
     return BW_EINVAL;
 }
 
-extern "C" int bw_abi_version(void) { return 6; }
+extern "C" int bw_abi_version(void) { return 7; }
 
 extern "C" const char* bw_strerror(int status) {
     switch (status) {

@@ -73,7 +73,7 @@ def _quantize(weight, bits, group_size, value):
         raise ValueError(f"Padding {pad} columns to {in_features} to make it a multiple of {group_size}")
     if in_features % (32 // bits):
         raise ValueError(f"in_features={in_features} does not fill whole int32 words at {bits} bits")
-    if weight.dtype not in (torch.float32, torch.float16, torch.bfloat16):
+    if weight.dtype not in (torch.float32, torch.float16, torch.bfloat16, torch.float64):
         raise NotImplementedError(f"quantize_rtn: weight dtype {weight.dtype} is not supported")
     dev = _gpu_for(weight)
     w = weight.to(dev)
@@ -88,7 +88,8 @@ def _quantize(weight, bits, group_size, value):
 @torch.no_grad()
 def dequantize_rtn(q_packed: torch.Tensor, scale: torch.Tensor, zero_point: torch.Tensor, group_size: int,
                    bits: int = 8):
-    """scale * (q - zero_point) as float32 [N, K] (bitween/functional.py:47-71)."""
+    """scale * (q - zero_point) as float32 [N, K] (bitween/functional.py:47-71); float64 for a float64 scale, as
+    the reference's product promotes."""
     assert bits in [2, 4, 8], "Only 2, 4, or 8-bit quantization supported."
     dev = _gpu_for(q_packed)
     s = scale.to(dev)
@@ -98,5 +99,6 @@ def dequantize_rtn(q_packed: torch.Tensor, scale: torch.Tensor, zero_point: torc
     if z.dtype not in (torch.int32, torch.float16):
         z = z.to(torch.int32) if not z.is_floating_point() else z.float().to(torch.int32)
     n = q_packed.shape[0]
-    out = _hip.dequantize(q_packed.to(dev), s.reshape(n, -1), z.reshape(n, -1), group_size, bits, torch.float32)
+    out_dtype = torch.float64 if s.dtype == torch.float64 else torch.float32
+    out = _hip.dequantize(q_packed.to(dev), s.reshape(n, -1), z.reshape(n, -1), group_size, bits, out_dtype)
     return out if q_packed.is_cuda else out.to(q_packed.device)

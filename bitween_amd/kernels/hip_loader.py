@@ -16,11 +16,11 @@ _LIB_PATH = os.environ.get("BITWEEN_HIP_LIB") or os.path.join(
     os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "csrc", "libbitween_hip.so")
 _lib = None
 
-BW_F16, BW_BF16, BW_F32, BW_I32 = 0, 1, 2, 3
+BW_F16, BW_BF16, BW_F32, BW_I32, BW_F64 = 0, 1, 2, 3, 4
 BW_SCALE_RECIPROCAL = 0x100   # flag for math_dtype: scale = (max - min) * fl32(1 / Qmax), as eager torch computes it on a GPU
-_DTYPE_CODE = {torch.float16: BW_F16, torch.bfloat16: BW_BF16, torch.float32: BW_F32, torch.int32: BW_I32}
+_DTYPE_CODE = {torch.float16: BW_F16, torch.bfloat16: BW_BF16, torch.float32: BW_F32, torch.int32: BW_I32, torch.float64: BW_F64}
 
-ABI_VERSION = 6            # what bw_abi_version() of a matching library returns
+ABI_VERSION = 7            # what bw_abi_version() of a matching library returns
 ENTRY_POINTS = ("bw_abi_version", "bw_strerror", "bw_quantize_pack", "bw_quantize_pack_add", "bw_dequantize", "bw_qgemv", "bw_qgemm",
                 "bw_qgemm_ws", "bw_qgemm_static", "bw_qgemm_workspace_bytes", "bw_qlinear", "bw_qdgrad", "bw_qdgrad_workspace_bytes", "bw_cast_bf16_f16", "bw_qlinear_decode_rows")
 
@@ -98,7 +98,7 @@ def _stream(device):
 
 
 def quantize_pack(weight, bits, group_size, math_dtype, scale_dtype, zp_dtype, delta=None, scale_reciprocal=False):
-    """weight [N,K] on GPU (f16/bf16/f32) -> (qweight int32, scale, zero_point) per bw_quantize_pack; with
+    """weight [N,K] on GPU (f16/bf16/f32, or f64 with f64 math and scale) -> (qweight int32, scale, zero_point) per bw_quantize_pack; with
     `delta` (same shape and dtype) the kernel quantises weight + delta (bw_quantize_pack_add).
     `scale_reciprocal`: the scale as eager torch forms it on a GPU (BW_SCALE_RECIPROCAL)."""
     require_gpu(weight, "quantize_pack")
@@ -127,7 +127,8 @@ def quantize_pack(weight, bits, group_size, math_dtype, scale_dtype, zp_dtype, d
 
 
 def dequantize(qweight, scale, zero_point, group_size, bits, out_dtype):
-    """(qweight, scale f32|f16, zero_point i32|f16) on GPU -> weight [N,K] of out_dtype per bw_dequantize."""
+    """(qweight, scale f32|f16, zero_point i32|f16) on GPU -> weight [N,K] of out_dtype per bw_dequantize; a float64
+    scale goes with out_dtype float64."""
     require_gpu(qweight, "dequantize")
     qweight, scale, zero_point = qweight.contiguous(), scale.contiguous(), zero_point.contiguous()
     n, words = qweight.shape

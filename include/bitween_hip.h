@@ -33,7 +33,7 @@
 extern "C" {
 #endif
 
-typedef enum bw_dtype { BW_F16 = 0, BW_BF16 = 1, BW_F32 = 2, BW_I32 = 3 } bw_dtype;
+typedef enum bw_dtype { BW_F16 = 0, BW_BF16 = 1, BW_F32 = 2, BW_I32 = 3, BW_F64 = 4 } bw_dtype;
 
 /* Flag for the math_dtype argument of bw_quantize_pack / bw_quantize_pack_add (OR it in): form the scale as
  * (max - min) * fl32(1 / Qmax) instead of (max - min) / Qmax.  bitween/functional.py:25 divides a tensor by the
@@ -69,6 +69,8 @@ const char* bw_strerror(int status);
  *   scale      [N][K/group] of scale_dtype (BW_F32 | BW_F16 | BW_BF16); a 16-bit
  *              type applies the module's round-to-nearest-even store
  *   zp         [N][K/group] of zp_dtype (BW_I32 | BW_F16 | BW_BF16)
+ * A float64 tensor (functional.py is dtype-agnostic): w_dtype = math_dtype = scale_dtype = BW_F64, zp_dtype BW_I32 -
+ * float64 arithmetic throughout, a float64 scale, as the reference returns for such a tensor.
  * Bit-exact against the reference arithmetic for finite inputs. */
 int bw_quantize_pack(const void* w, int w_dtype, int math_dtype, int64_t N, int64_t K, int64_t ldw,
                      int bits, int group, int32_t* qweight, void* scale, int scale_dtype,
@@ -87,7 +89,8 @@ int bw_quantize_pack_add(const void* w, const void* delta, int w_dtype, int math
  * dequantize kernel bitween/modules.py:10-58 (out_dtype BW_F16: one rounding
  * of the float32 product).  BW_BF16 output is an extension.
  *   scale [N][K/group] of scale_dtype (BW_F32 | BW_F16), zp of zp_dtype
- *   (BW_I32 | BW_F16); w_out [N][ldo] of out_dtype.  Bit-exact. */
+ *   (BW_I32 | BW_F16); w_out [N][ldo] of out_dtype.  A BW_F64 scale goes with a BW_F64 output (the float64
+ *   product functional.py:70 promotes to).  Bit-exact. */
 int bw_dequantize(const int32_t* qweight, const void* scale, int scale_dtype, const void* zp, int zp_dtype,
                   int64_t N, int64_t K, int bits, int group, void* w_out, int out_dtype, int64_t ldo,
                   void* stream);

@@ -19,6 +19,7 @@ How each function is pinned (see tests/test_oracle_pins.py):
                               rounding after every operation; groups whose
                               scale rounds to zero are "parity unpinned"
                               (the reference divides by zero there)
+  quantize_rtn_f64 / dequantize_rtn_f64   exact-rational evaluation with 53-bit rounding per operation
   store_module_buffers        numpy float16 cast is RNE (library routine)
   dequantize_f16              closed form RNE_f16(s16*(q-z)); product exact
   dequantize_rtn_f32          single binary32 multiply
@@ -123,6 +124,41 @@ def quantize_rtn(weight, bits=8, group_size=32, math="f32", scale_div="ieee"):
         q = np.clip(np.rint(t), np.float32(0), qmax).astype(np.int32)
     q = q.reshape(n, k)
     return pack_words(q, bits), scale.reshape(n, groups), zero_point.reshape(n, groups), q
+
+
+def quantize_rtn_f64(weight, bits=8, group_size=32, scale_div="ieee"):
+    """bitween/functional.py:3-45 on a float64 tensor: the same sequence in IEEE double arithmetic (numpy float64
+    operations are correctly rounded), a float64 scale.  "reciprocal": the scalar division as a multiplication by
+    1.0 / Qmax in double, what eager torch does on a GPU.  Pinned by exact-rational vectors with 53-bit rounding."""
+    assert bits in SUPPORTED_BITS, "Only 2, 4, or 8-bit quantization supported."
+    w = np.asarray(weight, dtype=np.float64)
+    n, k = w.shape
+    if k % group_size:
+        pad = group_size - k % group_size
+        raise ValueError(f"Padding {pad} columns to {k} to make it a multiple of {group_size}")
+    qmax = np.float64((1 << bits) - 1)
+    groups = k // group_size
+    wg = w.reshape(n, groups, group_size)
+    w_min = wg.min(axis=-1, keepdims=True)
+    w_max = wg.max(axis=-1, keepdims=True)
+    with np.errstate(all="ignore"):
+        rng = w_max - w_min
+        scale = rng / qmax if scale_div == "ieee" else rng * (np.float64(1.0) / qmax)
+        scale = np.maximum(scale, np.float64(1e-8))
+        zp_f = np.clip(np.rint((-w_min) / scale), 0.0, qmax)
+        q = np.clip(np.rint(wg / scale + zp_f), 0.0, qmax).astype(np.int32)
+    q = q.reshape(n, k)
+    return pack_words(q, bits), scale.reshape(n, groups), zp_f.astype(np.int32).reshape(n, groups), q
+
+
+def dequantize_rtn_f64(qweight, scale64, zero_point, group_size, bits=8):
+    """bitween/functional.py:70 with a float64 scale: scale * (q.float() - zp.float()) promotes to float64; the
+    difference is an exact small integer."""
+    q = unpack_words(qweight, bits)
+    n, k = q.shape
+    groups = k // group_size
+    d = q.reshape(n, groups, group_size).astype(np.float32) - np.asarray(zero_point).astype(np.float32).reshape(n, groups, 1)
+    return (np.asarray(scale64, np.float64).reshape(n, groups, 1) * d.astype(np.float64)).reshape(n, k)
 
 
 def store_module_buffers(scale, zero_point):

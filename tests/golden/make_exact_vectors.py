@@ -156,5 +156,50 @@ def main():
     print(f"wrote {path}: {idx} cases, {os.path.getsize(path) / 1024:.0f} KiB")
 
 
+def main_f64():
+    """float64 tensors (functional.py is dtype-agnostic): every operation rounded to 53 bits; a file of its own."""
+    out, names, idx = {}, [], 0
+    for scale_div in ("ieee", "reciprocal"):
+        for bits in (2, 4, 8):
+            for g in (32, 128):
+                for kind in ("normal_f64", "ties_f64"):
+                    rng = np.random.default_rng(91000 + 1000 * bits + g + len(kind) + (7 if scale_div == "ieee" else 0))
+                    n, k = 3, 2 * g
+                    w = rng.standard_normal((n, k)) * 0.02
+                    if kind == "ties_f64":
+                        # values on a grid of the group's range: many exact x.5 ties after w / scale + zp
+                        qmax = (1 << bits) - 1
+                        step = 2.0 ** -10
+                        w = rng.integers(0, 2 * qmax + 1, size=(n, k)).astype(np.float64) * (step / 2)
+                        w[:, ::g] = 0.0
+                        w[:, 1::g] = qmax * step
+                    groups = k // g
+                    q = np.zeros((n, k), np.int32)
+                    scale = np.zeros((n, groups), np.float64)
+                    zp = np.zeros((n, groups), np.int32)
+                    w64 = np.zeros((n, k), np.float64)
+                    for r in range(n):
+                        for gi in range(groups):
+                            s, z, qq = quantize_group_exact([float(v) for v in w[r, gi * g:(gi + 1) * g]], bits, "f64", scale_div)
+                            scale[r, gi], zp[r, gi] = float(s), z
+                            q[r, gi * g:(gi + 1) * g] = qq
+                            for i, qi in enumerate(qq):
+                                w64[r, gi * g + i] = float(rn(s * (qi - z), "f64")) or (-0.0 if qi < z else 0.0)
+                    words = np.array([pack_exact(list(q[r]), bits) for r in range(n)], np.int64).astype(np.int32)
+                    key = f"d{idx:03d}"
+                    names.append(f"{key}:f64:{bits}:{g}:{kind}:{scale_div}")
+                    for name, arr in dict(w=w, q=q, qweight=words, scale=scale, zp=zp, w64=w64).items():
+                        out[f"{key}_{name}"] = arr
+                    idx += 1
+    out["names"] = np.array(names)
+    path = os.path.join(HERE, "rtn_exact_vectors_f64.npz")
+    np.savez_compressed(path, **out)
+    print(f"wrote {path}: {idx} cases, {os.path.getsize(path) / 1024:.0f} KiB")
+
+
 if __name__ == "__main__":
-    main()
+    import sys
+    if "--f64" in sys.argv:
+        main_f64()
+    else:
+        main()

@@ -14,6 +14,7 @@ FORMATS = {           # precision (bits incl. hidden), min normal exponent, max 
     "f32": (24, -126, 127),
     "f16": (11, -14, 15),
     "bf16": (8, -126, 127),
+    "f64": (53, -1022, 1023),
 }
 
 
@@ -67,10 +68,13 @@ def quantize_group_exact(values, bits, fmt="f32", scale_div="ieee"):
         scale = rn(rn(hi - lo, fmt) / qmax, fmt)
     else:
         assert scale_div == "reciprocal"
-        scale = rn(rn(rn(hi - lo, fmt) * rn(Fraction(1, qmax), "f32"), "f32"), fmt)
+        op = "f64" if fmt == "f64" else "f32"                           # the type the multiplication is carried out in
+        scale = rn(rn(rn(hi - lo, fmt) * rn(Fraction(1, qmax), op), op), fmt)
     import struct
     floor32 = Fraction(struct.unpack("f", struct.pack("f", 1e-8))[0])   # the float32 nearest 1e-8
     floor = rn(floor32, fmt) if fmt != "f32" else floor32               # 0 in f16
+    if fmt == "f64":
+        floor = Fraction(1e-8)                                          # the double nearest 1e-8
     scale = max(scale, floor)
     if scale == 0:
         raise ZeroDivisionError("scale rounds to zero in this format")

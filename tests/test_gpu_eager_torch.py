@@ -33,18 +33,20 @@ def _bits(t):
     t = t.contiguous().cpu()
     if t.dtype in (torch.float16, torch.bfloat16):
         return t.view(torch.int16).numpy().view(np.uint16)
+    if t.dtype is torch.float64:
+        return t.view(torch.int64).numpy().view(np.uint64)
     return t.view(torch.int32).numpy().view(np.uint32)
 
 
 def _weights(dtype, outliers, seed):
     g = torch.Generator().manual_seed(seed)
-    w = torch.randn(384, 1024, generator=g) * 0.02
+    w = torch.randn(384, 1024, generator=g, dtype=torch.float64 if dtype is torch.float64 else torch.float32) * 0.02
     if outliers:
         w = torch.where(torch.rand(384, 1024, generator=g) < 0.001, w * 10, w)
     return w.to(dtype)
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16, torch.float64])
 @pytest.mark.parametrize("bits,group", [(2, 32), (4, 128), (4, 64), (8, 128)])
 @pytest.mark.parametrize("where,mode", [("cpu", "ieee"), ("cuda", "torch_device")])
 def test_kernel_matches_eager_torch(dtype, bits, group, where, mode):

@@ -64,6 +64,36 @@ def test_quantize_matches_exact_vectors(name):
         assert np.array_equal(qw.cpu().numpy(), GOLD[key + "_qweight"])
 
 
+GOLD64 = np.load(os.path.join(os.path.dirname(__file__), "golden", "rtn_exact_vectors_f64.npz"))
+
+
+@pytest.mark.parametrize("name", [str(n) for n in GOLD64["names"]])
+def test_quantize_float64_tensor_matches_exact_vectors(name):
+    """functional.py:3-71 is dtype-agnostic: a float64 weight is quantised in float64 arithmetic, returns a float64
+    scale, and dequantises to float64 - bit for bit, in both scale-division modes."""
+    import bitween_amd
+    key, _, bits, g, _, scale_div = name.split(":")
+    bits, g = int(bits), int(g)
+    w = torch.from_numpy(GOLD64[key + "_w"]).cuda()
+    previous = bitween_amd.set_scale_division("ieee" if scale_div == "ieee" else "torch_device")
+    try:
+        qw, scale, zp, group = bitween_amd.quantize_rtn(w, bits, g)
+    finally:
+        bitween_amd.set_scale_division(previous)
+    assert group == g and scale.dtype == torch.float64 and zp.dtype == torch.int32 and qw.dtype == torch.int32
+    assert np.array_equal(qw.cpu().numpy(), GOLD64[key + "_qweight"])
+    assert np.array_equal(zp.cpu().numpy(), GOLD64[key + "_zp"])
+    assert np.array_equal(scale.cpu().numpy().view(np.uint64), GOLD64[key + "_scale"].view(np.uint64))
+    w64 = bitween_amd.dequantize_rtn(qw, scale, zp, g, bits)
+    assert w64.dtype == torch.float64
+    assert np.array_equal(w64.cpu().numpy().view(np.uint64), GOLD64[key + "_w64"].view(np.uint64))
+    # the perturbed form: w = a + b with the sum rounded once to float64
+    a = w * 0.75
+    qw2, s2, z2, _ = bitween_amd.quantize_rtn_perturbed(a, w - a, bits, g)
+    qw3, s3, z3, _ = bitween_amd.quantize_rtn(a + (w - a), bits, g)
+    assert torch.equal(qw2, qw3) and torch.equal(s2, s3) and torch.equal(z2, z3)
+
+
 @pytest.mark.parametrize("name", RECIP_CASES)
 def test_quantize_with_reciprocal_scale_matches_exact_vectors(name):
     """set_scale_division("torch_device"): the scale as eager torch forms it on a GPU, (max - min) * fl32(1 / Qmax)."""

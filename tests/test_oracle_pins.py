@@ -290,3 +290,30 @@ def test_torch_cpu_path_matches_exact_vectors(name):
     with np.errstate(over="ignore", invalid="ignore"):
         finite = np.isfinite(ref.astype(np.float32).astype(np.float16))
     assert np.abs(y - ref)[finite].max() <= 1e-2 * max(np.abs(ref[finite]).max(), 1e-30)
+
+
+GOLD64 = np.load(os.path.join(os.path.dirname(__file__), "golden", "rtn_exact_vectors_f64.npz"))
+
+
+@pytest.mark.parametrize("name", [str(n) for n in GOLD64["names"]])
+def test_f64_oracle_matches_exact_vectors(name):
+    """quantize_rtn on a float64 tensor (the reference is dtype-agnostic): 53-bit rounding per operation, both
+    roundings of the scale division; the torch restatement run on a float64 tensor agrees in the IEEE mode."""
+    key, _, bits, g, _, scale_div = name.split(":")
+    bits, g = int(bits), int(g)
+    w = GOLD64[key + "_w"]
+    qw, scale, zp, q = orc.quantize_rtn_f64(w, bits, g, scale_div)
+    assert np.array_equal(q, GOLD64[key + "_q"])
+    assert np.array_equal(qw, GOLD64[key + "_qweight"])
+    assert np.array_equal(zp, GOLD64[key + "_zp"])
+    assert np.array_equal(scale.view(np.uint64), GOLD64[key + "_scale"].view(np.uint64))
+    w64 = orc.dequantize_rtn_f64(qw, scale, zp, g, bits)
+    assert np.array_equal(w64.view(np.uint64), GOLD64[key + "_w64"].view(np.uint64))
+    if scale_div == "ieee":
+        import torch
+        from oracle import torch_cpu_path as tcp
+        qw_t, s_t, z_t, _ = tcp.quantize_rtn(torch.from_numpy(w), bits, g)
+        assert s_t.dtype == torch.float64
+        assert np.array_equal(qw_t.numpy(), qw) and np.array_equal(s_t.numpy(), scale) and np.array_equal(z_t.numpy(), zp)
+        w_t = tcp.dequantize_rtn(qw_t, s_t, z_t, g, bits)
+        assert w_t.dtype == torch.float64 and np.array_equal(w_t.numpy().view(np.uint64), w64.view(np.uint64))
