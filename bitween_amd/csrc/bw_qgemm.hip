@@ -36,10 +36,11 @@ struct GemmCfg {
     static constexpr int CHUNK_BYTES = 64 * WL;                  // of a packed weight row
     static constexpr int NG = (VPL > GROUP) ? VPL / GROUP : 1;   // groups inside a lane's values
     static constexpr int WPG = 4 * WL / NG;                      // words of a lane's values per group
-    // One K step = one group: the scales (zero points) of four consecutive steps are 8 adjacent bytes and can
-    // come in one request per tile instead of four (kernel parameter META4; needs rows of scales that
-    // start on 4-byte boundaries, i.e. an even number of groups).
-    static constexpr bool CAN_META4 = CHUNK_K == GROUP;
+    // One K step = one group, or two: the scales (zero points) of four (two) consecutive steps are 8 adjacent bytes
+    // and can come in one request per tile instead of one per step and lane group (kernel parameter META4; needs rows
+    // of scales that start on 4-byte boundaries, i.e. an even number of groups).  SPR = steps per request.
+    static constexpr bool CAN_META4 = (CHUNK_K == GROUP || CHUNK_K == 2 * GROUP) && VPL <= GROUP;
+    static constexpr int SPR = 4 * GROUP / CHUNK_K, GPS = CHUNK_K / GROUP;   // groups per step (1 or 2)
     // Where the per-step side work sits (each placement measured per format, M = 512 and 2048):
     // EARLY_W: the first weight fragments of a K step are unpacked under the last MFMA step of the step
     // before (else at the start of the step, with the matrix pipe idle);
@@ -210,7 +211,7 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
     // the buffer); no step that runs ever uses those: a META4 launch has an even group count and even slices, so
     // the K loop below never pads with a zero step, and what the last step prepares for its successor is dropped.
     auto issue_meta4 = [&](int j, int which, int c, u2 (*m)[2]) {
-        m[j][which] = __builtin_amdgcn_raw_buffer_load_b64(which == 0 ? rs : rz, m_off[j] + c * 2, 0, 0);
+        m[j][which] = __builtin_amdgcn_raw_buffer_load_b64(which == 0 ? rs : rz, m_off[j] + c * (2 * C::GPS), 0, 0);
     };
     // Weight fragment of MFMA step t: values [8 t, 8 t + 8) of the lane's VPL, from lane load t / SPL.
     auto unpack = [&](const WSet& ws, int j, int t, const GroupConst<BITS>* gcj) {
@@ -234,9 +235,12 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
     auto set_consts = [&](GC* gj, int j, const WSet& from, const u2 (*m)[2], int half) {
 #pragma unroll
         for (int g = 0; g < C::NG; g++) {
-            if constexpr (META4)
+            if constexpr (META4 && C::GPS == 1)
                 gj[g].set(__builtin_bit_cast(_Float16, (uint16_t)(m[j][0][half >> 1] >> (16 * (half & 1)))),
                           __builtin_bit_cast(_Float16, (uint16_t)(m[j][1][half >> 1] >> (16 * (half & 1)))));
+            else if constexpr (META4)                            // two groups per step: lanes kq >= 2 take the second
+                gj[g].set(__builtin_bit_cast(_Float16, (uint16_t)(m[j][0][half] >> (16 * (kq >> 1)))),
+                          __builtin_bit_cast(_Float16, (uint16_t)(m[j][1][half] >> (16 * (kq >> 1)))));
             else
                 gj[g].set(__builtin_bit_cast(_Float16, (uint16_t)from.s[j][g]), __builtin_bit_cast(_Float16, (uint16_t)from.z[j][g]));
         }
@@ -265,7 +269,7 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
         auto slot_requests = [&](int t, int i) {
             static_assert(C::MF >= 4, "second and last MFMA step are distinct");
             if constexpr (META4) {
-                if (t == 1 && ph == 0) issue_meta4(i / 2, i & 1, c + 4, m_next);
+                if (t == 1 && ph == 0) issue_meta4(i / 2, i & 1, c + C::SPR, m_next);
             } else {
                 if (t == 1) issue_meta(i / 2, i & 1, c + 2, ws);
             }
@@ -277,7 +281,7 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
             asm volatile("" ::: "memory");
         };
         auto next_consts = [&](int j) {
-            if constexpr (META4) set_consts(gn[j], j, wsn, ph < 3 ? m_cur : m_next, ph < 3 ? ph + 1 : 0);
+            if constexpr (META4) set_consts(gn[j], j, wsn, ph < C::SPR - 1 ? m_cur : m_next, ph < C::SPR - 1 ? ph + 1 : 0);
             else set_consts(gn[j], j, wsn, m_cur, 0);
         };
 #pragma unroll
@@ -418,7 +422,14 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
         for (int e = 0; e < 4; e++) wf[0][j][e] = h2{f[2 * e], f[2 * e + 1]};
     }
     __syncthreads();
-    if constexpr (META4) {
+    if constexpr (META4 && C::SPR == 2) {
+        for (int c = c_begin; c < c_end; c += 2) {   // runs of two steps = one request; an odd count runs one step on zeros
+            step(c, buf0, buf1, set0, set1, gc0, gc1, 0);
+            step(c + 1, buf1, buf0, set1, set0, gc1, gc0, 1);
+#pragma unroll
+            for (int j = 0; j < NT; j++) { m_cur[j][0] = m_next[j][0]; m_cur[j][1] = m_next[j][1]; }
+        }
+    } else if constexpr (META4) {
         int c = c_begin;
         for (; c + 2 < c_end; c += 4) {          // runs of four steps; the last may run one step on zeros
             step(c, buf0, buf1, set0, set1, gc0, gc1, 0);
@@ -567,7 +578,9 @@ int launch_gemm(GemmArgs a, void* workspace, size_t workspace_bytes, hipStream_t
     static uint64_t big_lds_devices[2] = {0, 0};           // per kernel
     int which = 0;
     if constexpr (C::CAN_META4) {
-        if (a.groups % 2 == 0 && bw_aligned(a.scale, 4) && bw_aligned(a.zp, 4)) {
+        // an even number of K steps (so that the loop never pads with a step that would read past the row's scales)
+        // and rows of scales on 4-byte boundaries
+        if (a.groups % (2 * C::GPS) == 0 && bw_aligned(a.scale, 4) && bw_aligned(a.zp, 4)) {
             kern = qgemm_kernel<BITS, GROUP, true>;
             which = 1;
         }

@@ -813,6 +813,38 @@ def test_prefill_llama3_8b_mlp_shapes_at_full_size(k, n, m, xdtype):
         check_matmul(y[:, rows], x_np, qw_o, s16, z16, None, bits, g)
 
 
+@pytest.mark.parametrize("bits,g", [(4, 64), (8, 64), (2, 128)])
+@pytest.mark.parametrize("groups", [8, 10, 12, 20])
+@pytest.mark.parametrize("m", [40, 200])
+def test_prefill_formats_with_two_groups_per_k_step(bits, g, groups, m):
+    """Formats whose K step spans two groups (4 and 8 bits at g64, 2 bits at g128): with a multiple of four groups the
+    prefill kernel fetches the scales of two steps in one 8-byte request per tile, else per step and lane - both
+    against the oracle, split and unsplit, one-hot rows bit for bit, and the two plans on shapes that differ only in
+    taking one or the other."""
+    import ctypes
+    hip = _hip()
+    lib = hip.load()
+    k, n = g * groups, 300
+    _, qw, s16, z16, b16 = quantized_layer(n, k, bits, g, seed=bits * 1000 + groups, outliers=True)
+    rng = np.random.default_rng(groups + m)
+    x = rng.standard_normal((m, k)).astype(np.float16)
+    hot = {0: 0, 3: k - 1, m - 1: k // 2 + 1}
+    for r, c in hot.items():
+        x[r] = 0
+        x[r, c] = 1
+    d = [to_gpu(a) for a in (x, qw, s16, z16, b16)]
+    w16 = orc.dequantize_f16(qw, s16, z16, g, bits)
+    y_ws = hip.quantized_gemm_hip(d[0], d[1], d[2], d[3], None, bits, g)
+    y_plain = torch.empty((m, n), dtype=torch.float16, device="cuda")
+    assert lib.bw_qgemm(d[0].data_ptr(), 0, m, k, k, d[1].data_ptr(), d[2].data_ptr(), d[3].data_ptr(), d[4].data_ptr(), n, bits, g,
+                        y_plain.data_ptr(), n, ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)) == 0
+    torch.cuda.synchronize()
+    check_matmul(y_ws, x, qw, s16, z16, None, bits, g)
+    check_matmul(y_plain, x, qw, s16, z16, b16, bits, g)
+    for r, c in hot.items():
+        assert np.array_equal(y_ws[r].cpu().numpy().view(np.uint16), w16[:, c].view(np.uint16))
+
+
 def test_sibling_group_does_not_serve_a_member_twice_from_its_cache():
     """An input rewritten in place without a version bump (.data) and handed to the same member again gets a new
     launch, not the cached slice."""
