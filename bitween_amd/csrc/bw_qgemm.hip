@@ -129,9 +129,12 @@ BW_DEV __amdgpu_buffer_rsrc_t make_rsrc(const void* p, uint32_t bytes) {
 //   the activations of chunk c+1 were requested one step earlier and are written to buffer (c+1)&1 during
 //   step c, then re-requested for chunk c+2; the weights of chunk c+2 are requested into step c's own set
 //   once its last fragment is unpacked.  Every global load has a full K step (~2000 MFMA cycles) to land.
-template <int BITS, int GROUP, bool META4>
+template <int BITS, int GROUP, bool WIDE_META>
 __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
     using C = GemmCfg<BITS, GROUP>;
+    // WIDE_META (rows of scales on 4-byte boundaries): META4 = 8-byte requests over runs of K steps; PAIR = a lane whose
+    // values span two groups fetches both scales (zero points) with one 4-byte request instead of two 2-byte ones
+    constexpr bool META4 = WIDE_META && C::CAN_META4, PAIR = WIDE_META && !C::CAN_META4 && C::NG == 2;
     constexpr uint32_t kOob = 0x80000000u;
     extern __shared__ __attribute__((aligned(16))) char smem[];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -201,6 +204,11 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
     };
     auto issue_meta = [&](int j, int which, int c, WSet& ws) {   // which: 0 = scales, 1 = zero points
         const int g0 = min((c * C::CHUNK_K + kq * C::VPL) / GROUP, groups - C::NG);
+        if constexpr (PAIR) {                                       // g0 is even: both entries in one aligned word
+            if (which == 0) ws.s[j][0] = __builtin_amdgcn_raw_buffer_load_b32(rs, m_off[j] + g0 * 2, 0, 0);
+            else ws.z[j][0] = __builtin_amdgcn_raw_buffer_load_b32(rz, m_off[j] + g0 * 2, 0, 0);
+            return;
+        }
 #pragma unroll
         for (int g = 0; g < C::NG; g++) {
             if (which == 0) ws.s[j][g] = __builtin_amdgcn_raw_buffer_load_b16(rs, m_off[j] + (g0 + g) * 2, 0, 0);
@@ -241,6 +249,8 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
             else if constexpr (META4)                            // two groups per step: lanes kq >= 2 take the second
                 gj[g].set(__builtin_bit_cast(_Float16, (uint16_t)(m[j][0][half] >> (16 * (kq >> 1)))),
                           __builtin_bit_cast(_Float16, (uint16_t)(m[j][1][half] >> (16 * (kq >> 1)))));
+            else if constexpr (PAIR)
+                gj[g].set(__builtin_bit_cast(_Float16, (uint16_t)(from.s[j][0] >> (16 * g))), __builtin_bit_cast(_Float16, (uint16_t)(from.z[j][0] >> (16 * g))));
             else
                 gj[g].set(__builtin_bit_cast(_Float16, (uint16_t)from.s[j][g]), __builtin_bit_cast(_Float16, (uint16_t)from.z[j][g]));
         }
@@ -577,10 +587,10 @@ int launch_gemm(GemmArgs a, void* workspace, size_t workspace_bytes, hipStream_t
     void (*kern)(const GemmArgs) = qgemm_kernel<BITS, GROUP, false>;
     static uint64_t big_lds_devices[2] = {0, 0};           // per kernel
     int which = 0;
-    if constexpr (C::CAN_META4) {
+    if constexpr (C::CAN_META4 || C::NG == 2) {
         // an even number of K steps (so that the loop never pads with a step that would read past the row's scales)
         // and rows of scales on 4-byte boundaries
-        if (a.groups % (2 * C::GPS) == 0 && bw_aligned(a.scale, 4) && bw_aligned(a.zp, 4)) {
+        if (a.groups % (C::CAN_META4 ? 2 * C::GPS : 2) == 0 && bw_aligned(a.scale, 4) && bw_aligned(a.zp, 4)) {
             kern = qgemm_kernel<BITS, GROUP, true>;
             which = 1;
         }

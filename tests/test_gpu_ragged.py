@@ -74,6 +74,31 @@ def test_prefill_scale_rows_at_every_alignment(bits, groups, offset):
     check_matmul(y, x, qw, s16, z16, None, bits, g)
 
 
+@pytest.mark.parametrize("bits,g,groups", [(4, 64, 24), (8, 64, 12), (2, 128, 8), (2, 32, 16), (2, 32, 24)])
+@pytest.mark.parametrize("offset", [0, 1, 2, 3])
+def test_prefill_wide_scale_requests_at_every_alignment(bits, g, groups, offset):
+    """The other formats with wide scale requests - one 8-byte request per two K steps (4 and 8 bits at g64, 2 bits at
+    g128), one 4-byte request for a lane's two groups (2 bits at g32): a base address off by one element must take
+    the 2-byte requests and give the same result."""
+    from bitween_amd.kernels import hip_loader
+    lib = hip_loader.load()
+    n, m = 300, 192
+    k = g * groups
+    _, qw, s16, z16, _ = quantized_layer(n, k, bits, g, seed=177 + groups, outliers=True)
+    x = np.random.default_rng(groups + offset).standard_normal((m, k)).astype(np.float16)
+    sbuf = torch.zeros(n * groups + offset, dtype=torch.float16, device="cuda")
+    zbuf = torch.zeros(n * groups + offset, dtype=torch.float16, device="cuda")
+    sbuf[offset:] = to_gpu(s16).reshape(-1)
+    zbuf[offset:] = to_gpu(z16).reshape(-1)
+    xg, qg = to_gpu(x), to_gpu(qw)
+    y = torch.empty((m, n), dtype=torch.float16, device="cuda")
+    st = lib.bw_qgemm(xg.data_ptr(), 0, m, k, k, qg.data_ptr(), sbuf.data_ptr() + 2 * offset, zbuf.data_ptr() + 2 * offset,
+                      None, n, bits, g, y.data_ptr(), n, ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    assert st == 0
+    torch.cuda.synchronize()
+    check_matmul(y, x, qw, s16, z16, None, bits, g)
+
+
 @pytest.mark.parametrize("m", [1, 2, 16, 130])
 @pytest.mark.parametrize("bits", [2, 4, 8])
 @pytest.mark.parametrize("groups", [13, 14, 15, 16])
