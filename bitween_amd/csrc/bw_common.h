@@ -64,13 +64,16 @@ template <> struct GroupConst<2> {
 
 constexpr uint32_t kMagic = 0x64006400u;   // two float16 1024.0
 
-// (a & mask) | orv in one VALU op.  The VOP3 encoding of gfx950 takes no 32-bit literals, so the
-// compiler emits v_and + v_or for literal operands; with the mask in an SGPR and the magic in a VGPR the
-// fused form is encodable.
+// (a & mask) | orv in one VALU op.  The VOP3 encoding of gfx950 takes no 32-bit literals, so for literal operands the
+// compiler emits v_and + v_or; with the mask in an SGPR and the magic in a VGPR the fused v_and_or_b32 is
+// encodable.  The two empty statements only hide the constants from folding (they emit nothing, and being
+// non-volatile they are hoisted and shared like any other pure computation).  The instruction itself stays one the
+// compiler knows: after an inline-assembly and-or it pads every consumer with a wait state, which the MFMA-bound
+// loops notice.
 BW_DEV uint32_t and_or(uint32_t a, uint32_t mask, uint32_t orv) {
-    uint32_t d;
-    asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(d) : "v"(a), "s"(mask), "v"(orv));
-    return d;
+    asm("" : "+s"(mask));
+    asm("" : "+v"(orv));
+    return (a & mask) | orv;
 }
 
 // SCALE = true: out = fp16(s * (q - z)) (the reference's W16).  SCALE = false: out = q - z exactly
