@@ -553,6 +553,49 @@ def extras_llama7b_decoder_graph(torch, hip, QuantizedLinear, layers):
     return res
 
 
+def build_probes():
+    """hipcc bench_probes.hip for gfx950 into bench_probes.so next to this file (works without a GPU)."""
+    import subprocess
+    here = os.path.dirname(os.path.abspath(__file__))
+    lib = os.path.join(here, "bench_probes.so")
+    cmd = [os.environ.get("HIPCC", "/opt/rocm/bin/hipcc"), "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
+           "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-o", lib, os.path.join(here, "bench_probes.hip")]
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError("hipcc failed:\n" + proc.stderr)
+    return lib
+
+
+def extras_board_probes(torch, hip, QuantizedLinear, layers):
+    """The constants of this board that the decode and prefill ceilings are derived from (bench_probes.hip): device
+    time per launch of an empty kernel under graph replay, the rate of a kernel that only reads, and how many
+    instructions a single wave can issue per MFMA."""
+    import ctypes
+    lib_path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "bench_probes.so")
+    if not os.path.exists(lib_path):
+        return {"skipped": "bench_probes.so is not built (run __graft_entry__.build())"}
+    lib = ctypes.CDLL(lib_path)
+    vp, i32, dbl = ctypes.c_void_p, ctypes.c_int32, ctypes.c_double
+    lib.probe_launch_floor.argtypes, lib.probe_launch_floor.restype = [i32, i32, i32, i32], dbl
+    lib.probe_read_rate.argtypes, lib.probe_read_rate.restype = [vp, ctypes.c_size_t, vp, i32, i32], dbl
+    lib.probe_mfma_issue.argtypes, lib.probe_mfma_issue.restype = [i32, i32, vp], dbl
+    torch.cuda.synchronize()
+    out = {"empty_kernel_us_per_launch_graph_replay": {
+        "grid256_block512": round(lib.probe_launch_floor(200, 256, 512, 10), 3),
+        "grid688_block1024": round(lib.probe_launch_floor(200, 688, 1024, 10), 3)}}
+    src = torch.empty(1 << 30, dtype=torch.uint8, device="cuda").fill_(1)
+    scratch = torch.zeros(4, dtype=torch.float32, device="cuda")
+    torch.cuda.synchronize()
+    out["read_only_kernel_GBps_1GiB"] = round(lib.probe_read_rate(src.data_ptr(), src.numel(), scratch.data_ptr(), 4096, 4), 1)
+    del src
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    ns = [lib.probe_mfma_issue(v, cus, scratch.data_ptr()) for v in range(4)]
+    out["mfma_16x16x32_f16_ns_per_wave"] = {"mfma_only": round(ns[0], 2), "plus_1_valu": round(ns[1], 2), "plus_2_valu": round(ns[2], 2),
+                                            "plus_3_valu": round(ns[3], 2)}
+    out["mfma_only_TFLOPs"] = round(cus * 4 * 16384 / ns[0] / 1e3, 1)
+    return out
+
+
 def extras_backward(torch, hip, QuantizedLinear, layers):
     """grad_input of QuantizedLinearFunction.backward, 4096 -> 14336 W4 g128: the fused kernel (bw_qdgrad), the
     path it replaces (HIP dequantise to float16 + library GEMM) and that GEMM alone on resident fp16 weights."""
@@ -618,7 +661,7 @@ def extras_opt125m_fc1(torch, hip, QuantizedLinear, layers):
 EXTRAS = {"opt125m_fc1": extras_opt125m_fc1, "decode": extras_decode, "decode_infinity_cache_hot": extras_decode_hot,
           "decode_other_formats": extras_decode_other_formats, "hipblaslt_fp16_decode": extras_hipblaslt_decode,
           "prefill": extras_prefill, "prefill_other_formats": extras_prefill_other_formats, "quantize": extras_quantize, "mixed_precision_model": extras_mixed_precision_model, "eager_call": extras_eager_call,
-          "decode_fused_siblings": extras_decode_fused_siblings,
+          "decode_fused_siblings": extras_decode_fused_siblings, "board_probes": extras_board_probes,
           # the heavy sections last: the GEMMs and the 7B model leave the board warm, which shows in the decode timings
           "backward": extras_backward, "llama7b_decoder_graph": extras_llama7b_decoder_graph,
           "transformers_drop_in_check": extras_llama7b_end_to_end}

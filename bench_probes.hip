@@ -1,0 +1,135 @@
+// Board probes of bench.py (extras.board_probes): the three constants the kernel ceilings are derived from.  Not part
+// of the quantized-linear library.
+//   probe_launch_floor   device time per launch of an empty kernel when `launches` dependent launches are replayed
+//                        from one HIP graph (what separates two kernels of a decode step)
+//   probe_read_rate      a kernel that only reads `bytes` of device memory: GB/s
+//   probe_mfma_issue     v_mfma_f32_16x16x32_f16 back to back, one wave per SIMD, 32 independent accumulator tiles, with
+//                        0..3 independent VALU instructions after every MFMA: ns per MFMA and wave (how many issue
+//                        slots a single wave has per MFMA)
+// Every entry point returns a negative value on a HIP error.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace {
+
+typedef unsigned int u4v __attribute__((ext_vector_type(4)));
+typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+typedef float f4 __attribute__((ext_vector_type(4)));
+
+__global__ void empty_kernel(int* p) {
+    if (p && threadIdx.x == 0x7fffffff) p[0] = 1;
+}
+
+__global__ __launch_bounds__(256) void read_kernel(const u4v* __restrict__ s, int* out, size_t n) {
+    size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    const size_t st = (size_t)gridDim.x * 256;
+    unsigned acc = 0;
+    for (; i + 3 * st < n; i += 4 * st) {
+        const u4v a = s[i], b = s[i + st], c = s[i + 2 * st], e = s[i + 3 * st];
+        acc ^= a.x ^ b.y ^ c.z ^ e.w;
+    }
+    for (; i < n; i += st) acc ^= s[i].x;
+    if (acc == 0x12345u) out[0] = 1;                          // keeps the loads alive; practically never true
+}
+
+template <int VPM>
+__global__ __launch_bounds__(256) void mfma_kernel(float* out, int iters, float seed) {
+    constexpr int NACC = 32;
+    f4 acc[NACC];
+#pragma unroll
+    for (int i = 0; i < NACC; i++) acc[i] = f4{0.f, 0.f, 0.f, 0.f};
+    h8 a, b;
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+        a[e] = (_Float16)(seed + threadIdx.x * 1e-3f + e);
+        b[e] = (_Float16)(seed * 0.5f + e);
+    }
+    float v0 = seed, v1 = seed + 1.f, v2 = seed + 2.f;
+    for (int it = 0; it < iters; it++) {
+#pragma unroll
+        for (int i = 0; i < NACC; i++) {
+            asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc[i]) : "v"(a), "v"(b));
+            if (VPM >= 1) asm volatile("v_fma_f32 %0, %0, %1, %1" : "+v"(v0) : "v"(v1));
+            if (VPM >= 2) asm volatile("v_fma_f32 %0, %0, %1, %1" : "+v"(v1) : "v"(v2));
+            if (VPM >= 3) asm volatile("v_fma_f32 %0, %0, %1, %1" : "+v"(v2) : "v"(v0));
+        }
+    }
+    float s = v0 + v1 + v2;
+#pragma unroll
+    for (int i = 0; i < NACC; i++) s += acc[i][0] + acc[i][1] + acc[i][2] + acc[i][3];
+    if (s == 12345.678f) out[0] = s;
+}
+
+struct Timer {
+    hipEvent_t a = nullptr, b = nullptr;
+    bool ok = false;
+    Timer() { ok = hipEventCreate(&a) == hipSuccess && hipEventCreate(&b) == hipSuccess; }
+    ~Timer() {
+        if (a) (void)hipEventDestroy(a);
+        if (b) (void)hipEventDestroy(b);
+    }
+};
+
+}  // namespace
+
+extern "C" double probe_launch_floor(int launches, int grid, int block, int replays) {
+    if (launches < 1 || grid < 1 || block < 1 || block > 1024 || replays < 1) return -1.0;
+    hipStream_t st;
+    if (hipStreamCreate(&st) != hipSuccess) return -2.0;
+    hipGraph_t g = nullptr;
+    hipGraphExec_t ge = nullptr;
+    Timer t;
+    double us = -2.0;
+    if (t.ok && hipStreamBeginCapture(st, hipStreamCaptureModeThreadLocal) == hipSuccess) {
+        for (int i = 0; i < launches; i++) hipLaunchKernelGGL(empty_kernel, dim3(grid), dim3(block), 0, st, (int*)nullptr);
+        if (hipStreamEndCapture(st, &g) == hipSuccess && hipGraphInstantiate(&ge, g, nullptr, nullptr, 0) == hipSuccess) {
+            bool ok = true;
+            for (int i = 0; i < 3 && ok; i++) ok = hipGraphLaunch(ge, st) == hipSuccess;
+            ok = ok && hipStreamSynchronize(st) == hipSuccess && hipEventRecord(t.a, st) == hipSuccess;
+            for (int i = 0; i < replays && ok; i++) ok = hipGraphLaunch(ge, st) == hipSuccess;
+            ok = ok && hipEventRecord(t.b, st) == hipSuccess && hipStreamSynchronize(st) == hipSuccess;
+            float ms = 0.f;
+            if (ok && hipEventElapsedTime(&ms, t.a, t.b) == hipSuccess) us = (double)ms * 1e3 / ((double)replays * launches);
+        }
+    }
+    if (ge) (void)hipGraphExecDestroy(ge);
+    if (g) (void)hipGraphDestroy(g);
+    (void)hipStreamDestroy(st);
+    return us;
+}
+
+// `src`: `bytes` of device memory (16-byte aligned, a multiple of 16), `scratch`: 4 bytes of device memory
+extern "C" double probe_read_rate(const void* src, size_t bytes, void* scratch, int grid, int runs) {
+    if (!src || !scratch || bytes < 16 || bytes % 16 || grid < 1 || runs < 1 || ((uintptr_t)src & 15)) return -1.0;
+    Timer t;
+    if (!t.ok) return -2.0;
+    hipLaunchKernelGGL(read_kernel, dim3(grid), dim3(256), 0, 0, (const u4v*)src, (int*)scratch, bytes / 16);
+    if (hipDeviceSynchronize() != hipSuccess || hipEventRecord(t.a, 0) != hipSuccess) return -2.0;
+    for (int i = 0; i < runs; i++) hipLaunchKernelGGL(read_kernel, dim3(grid), dim3(256), 0, 0, (const u4v*)src, (int*)scratch, bytes / 16);
+    float ms = 0.f;
+    if (hipEventRecord(t.b, 0) != hipSuccess || hipDeviceSynchronize() != hipSuccess || hipEventElapsedTime(&ms, t.a, t.b) != hipSuccess)
+        return -2.0;
+    return (double)bytes * runs / ((double)ms * 1e-3) / 1e9;
+}
+
+// ns per MFMA and wave with `valu_per_mfma` (0..3) independent VALU instructions after every MFMA; `scratch`: 4 bytes
+extern "C" double probe_mfma_issue(int valu_per_mfma, int workgroups, void* scratch) {
+    if (valu_per_mfma < 0 || valu_per_mfma > 3 || workgroups < 1 || !scratch) return -1.0;
+    const int iters = 2000;
+    Timer t;
+    if (!t.ok) return -2.0;
+    auto launch = [&](int n) {
+        float* out = (float*)scratch;
+        if (valu_per_mfma == 0) hipLaunchKernelGGL(mfma_kernel<0>, dim3(workgroups), dim3(256), 0, 0, out, n, 1.0f);
+        else if (valu_per_mfma == 1) hipLaunchKernelGGL(mfma_kernel<1>, dim3(workgroups), dim3(256), 0, 0, out, n, 1.0f);
+        else if (valu_per_mfma == 2) hipLaunchKernelGGL(mfma_kernel<2>, dim3(workgroups), dim3(256), 0, 0, out, n, 1.0f);
+        else hipLaunchKernelGGL(mfma_kernel<3>, dim3(workgroups), dim3(256), 0, 0, out, n, 1.0f);
+    };
+    launch(50);
+    if (hipDeviceSynchronize() != hipSuccess || hipEventRecord(t.a, 0) != hipSuccess) return -2.0;
+    launch(iters);
+    float ms = 0.f;
+    if (hipEventRecord(t.b, 0) != hipSuccess || hipDeviceSynchronize() != hipSuccess || hipEventElapsedTime(&ms, t.a, t.b) != hipSuccess)
+        return -2.0;
+    return (double)ms * 1e6 / ((double)iters * 32);
+}
