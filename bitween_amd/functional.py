@@ -13,17 +13,19 @@ from .kernels import hip_loader as _hip
 
 # How `(w_max - w_min) / Qmax` (bitween/functional.py:25) is rounded.  Eager torch divides a tensor by a Python
 # scalar exactly on the CPU and multiplies by the float32 reciprocal on a GPU; the two differ in the last bit of
-# most float32 scales.  "ieee" (default) is the CPU arithmetic, the source as written; "torch_device" reproduces
-# what the reference computes when it quantises on a GPU.  BITWEEN_SCALE_DIVISION sets the initial choice.
-_SCALE_DIVISIONS = ("ieee", "torch_device")
-_scale_division = os.environ.get("BITWEEN_SCALE_DIVISION", "ieee")
+# most float32 scales.  "auto" (default) follows the device of the tensor being quantised, which is what the
+# reference's own call yields: a CPU tensor gets the true division, a GPU tensor the reciprocal.  "ieee" forces
+# the CPU arithmetic (the source as written), "torch_device" the GPU's, wherever the tensor lives.
+# BITWEEN_SCALE_DIVISION sets the initial choice.
+_SCALE_DIVISIONS = ("auto", "ieee", "torch_device")
+_scale_division = os.environ.get("BITWEEN_SCALE_DIVISION", "auto")
 if _scale_division not in _SCALE_DIVISIONS:
     raise ValueError(f"BITWEEN_SCALE_DIVISION must be one of {_SCALE_DIVISIONS}, got {_scale_division!r}")
 
 
 def set_scale_division(mode: str) -> str:
-    """Choose the rounding of the scale division for quantize_rtn and QuantizedLinear.from_float: "ieee" or
-    "torch_device".  Returns the previous choice."""
+    """Choose the rounding of the scale division for quantize_rtn and QuantizedLinear.from_float: "auto" (follow the
+    tensor's device), "ieee" or "torch_device".  Returns the previous choice."""
     global _scale_division
     if mode not in _SCALE_DIVISIONS:
         raise ValueError(f"scale division must be one of {_SCALE_DIVISIONS}, got {mode!r}")
@@ -33,6 +35,16 @@ def set_scale_division(mode: str) -> str:
 
 def get_scale_division() -> str:
     return _scale_division
+
+
+def scale_reciprocal_for(tensor, mode=None) -> bool:
+    """True when the scale of `tensor` is to be formed as (max - min) * fl(1 / Qmax): the current mode (or `mode`)
+    says "torch_device", or it says "auto" and the tensor lives on a GPU - where the reference's eager division by
+    a Python scalar is that multiplication."""
+    mode = _scale_division if mode is None else mode
+    if mode not in _SCALE_DIVISIONS:
+        raise ValueError(f"scale division must be one of {_SCALE_DIVISIONS}, got {mode!r}")
+    return mode == "torch_device" or (mode == "auto" and tensor.is_cuda)
 
 
 def _gpu_for(t):
@@ -79,7 +91,7 @@ def _quantize(weight, bits, group_size, value):
     w = weight.to(dev)
     qweight, scale, zp = _hip.quantize_pack(w, bits, group_size, math_dtype=weight.dtype, scale_dtype=weight.dtype,
                                             zp_dtype=torch.int32, delta=None if value is None else value.to(dev),
-                                            scale_reciprocal=_scale_division == "torch_device")
+                                            scale_reciprocal=scale_reciprocal_for(weight))
     if not weight.is_cuda:
         qweight, scale, zp = qweight.to(weight.device), scale.to(weight.device), zp.to(weight.device)
     return qweight, scale, zp, group_size

@@ -101,7 +101,9 @@ class QuantizedLinear(nn.Module):
             plan = self.__dict__.get("_decode_plan")
             b = self._buffers
             if plan is None or plan[0] is not b["qweight"] or plan[1] is not b["scale"] or \
-                    plan[2] is not b["zero_point"] or plan[3] is not b.get("bias") or plan[4] != plan[0].data_ptr():
+                    plan[2] is not b["zero_point"] or plan[3] is not b.get("bias") or plan[4] != plan[0].data_ptr() or \
+                    plan[5] != plan[1].data_ptr() or plan[6] != plan[2].data_ptr() or \
+                    (plan[3] is not None and plan[7] != plan[3].data_ptr()):
                 plan = _hip.make_decode_plan(b["qweight"], b["scale"], b["zero_point"], b.get("bias"), self.bits,
                                              self.group_size) if b["qweight"].is_cuda else None
                 self.__dict__["_decode_plan"] = plan
@@ -139,7 +141,7 @@ class QuantizedLinear(nn.Module):
             weight = weight.to("cuda")
         qweight, scale, zero_point = _hip.quantize_pack(weight, bits, group_size, math_dtype=torch.float32,
                                                         scale_dtype=torch.float16, zp_dtype=torch.float16,
-                                                        scale_reciprocal=_functional.get_scale_division() == "torch_device")
+                                                        scale_reciprocal=_functional.scale_reciprocal_for(float_layer.weight))
         # the constructor's zero buffers are built on the meta device (no memory, no host-to-device copy) and
         # replaced by the kernel's outputs, which already have the buffers' shapes and dtypes
         with torch.device("meta"):
@@ -206,9 +208,22 @@ class _SiblingGroup:
         state["_x"], state["_version"], state["_y"], state["_served"], state["_served_mask"] = None, -1, None, 0, 0
         return state
 
+    def _views_fused_buffers(self, member, row):
+        """Every buffer of `member` still starts at its row of the concatenated tensors (a buffer replaced through
+        `.data = ...` or `.set_()` keeps its Python object but not its address)."""
+        b = member._buffers
+        if b["qweight"].data_ptr() != self.qweight.data_ptr() + row * self.qweight.stride(0) * 4 or \
+                b["scale"].data_ptr() != self.scale.data_ptr() + row * self.scale.stride(0) * 2 or \
+                b["zero_point"].data_ptr() != self.zero_point.data_ptr() + row * self.zero_point.stride(0) * 2:
+            return False
+        bias = b.get("bias")
+        if (bias is None) != (self.bias is None):
+            return False
+        return bias is None or bias.data_ptr() == self.bias.data_ptr() + row * 2
+
     def forward(self, member, x):
         rng = member.__dict__.get("_sibling_rows")
-        if rng is None or member.qweight.data_ptr() != self.qweight.data_ptr() + rng[0] * self.qweight.stride(0) * 4:
+        if rng is None or not self._views_fused_buffers(member, rng[0]):
             return None                                    # the member no longer views the fused buffers
         if self.wasted >= 4:
             return None                                    # the members do not share inputs after all: stop grouping

@@ -166,3 +166,28 @@ def test_precision_map_lookup():
     assert _precision_for("model.layers.01.mlp.up_proj", cfg, None) is None           # prefix of a name is not a block
     assert _precision_for("lm_head", cfg, (4, 128)) == (4, 128)
     assert _precision_for("lm", cfg, None) == (4, 64)
+
+
+@pytest.mark.default_scale_division
+def test_scale_division_default_follows_the_tensor_device():
+    """The default mode is "auto": the reference's `(max - min) / Qmax` is a true division for a CPU tensor and a
+    multiplication by the float32 reciprocal for a GPU tensor (bitween/functional.py:25 under eager torch)."""
+    import bitween_amd
+    from bitween_amd import functional as F
+
+    class OnGpu:                                              # stands in for a GPU tensor: only the device is asked
+        is_cuda = True
+
+    if "BITWEEN_SCALE_DIVISION" not in os.environ:
+        assert bitween_amd.get_scale_division() == "auto"
+    cpu = torch.zeros(1)
+    assert F.scale_reciprocal_for(cpu, "auto") is False and F.scale_reciprocal_for(OnGpu(), "auto") is True
+    assert F.scale_reciprocal_for(cpu, "ieee") is False and F.scale_reciprocal_for(OnGpu(), "ieee") is False
+    assert F.scale_reciprocal_for(cpu, "torch_device") is True and F.scale_reciprocal_for(OnGpu(), "torch_device") is True
+    previous = bitween_amd.set_scale_division("torch_device")
+    try:
+        assert bitween_amd.get_scale_division() == "torch_device" and F.scale_reciprocal_for(cpu) is True
+        with pytest.raises(ValueError):
+            bitween_amd.set_scale_division("fast")
+    finally:
+        bitween_amd.set_scale_division(previous)

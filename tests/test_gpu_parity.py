@@ -671,6 +671,31 @@ def test_validated_buffer_cache_follows_replaced_buffers():
     assert torch.equal(qf(x.to(torch.bfloat16)), qf(x.to(torch.bfloat16).to(torch.float16)))
     xs = torch.randn(3, 2 * k, device="cuda", dtype=torch.float16)[:, ::2]     # strided x falls back to the general path
     assert torch.equal(qf(xs), qf(xs.contiguous()))
+    # same Python objects, new storage: `.data = ...` and `.set_()` on scale, zero_point and bias
+    qg = bitween_amd.QuantizedLinear.from_float(lin_a, 4, 64)
+    assert torch.equal(qg(x), ya)
+    keep = [qg.scale.data, qg.zero_point.data, qg.bias.data]  # the old blocks stay allocated: the test must not depend on reuse
+    scale_obj, zp_obj, bias_obj = qg.scale, qg.zero_point, qg.bias
+    qg.scale.data = qb.scale.clone()
+    assert qg.scale is scale_obj and torch.equal(qg(x), direct(qg)) and not torch.equal(qg(x), ya)
+    qg.zero_point.set_(qb.zero_point.clone())
+    assert qg.zero_point is zp_obj and torch.equal(qg(x), direct(qg))
+    qg.bias.data = torch.zeros_like(qg.bias)
+    assert qg.bias is bias_obj and torch.equal(qg(x), direct(qg))
+    qg.qweight.data = qb.qweight.clone()
+    assert torch.equal(qg(x), hip.quantized_matmul_hip(x, qb.qweight, qb.scale, qb.zero_point, None, 4, 64))
+    del keep
+    # and in a sibling group: a member whose scale was re-pointed leaves the group and answers for itself
+    blk = torch.nn.Module()
+    blk.gate_proj = bitween_amd.QuantizedLinear.from_float(lin_a, 4, 64)
+    blk.up_proj = bitween_amd.QuantizedLinear.from_float(lin_b, 4, 64)
+    assert bitween_amd.fuse_sibling_linears(blk) == 1
+    with torch.no_grad():
+        assert torch.equal(blk.gate_proj(x), ya) and torch.equal(blk.up_proj(x), yb)
+        blk.up_proj.scale.data = qa.scale.clone()
+        x2 = x.clone()
+        assert torch.equal(blk.gate_proj(x2), ya)
+        assert torch.equal(blk.up_proj(x2), hip.quantized_matmul_hip(x, qb.qweight, qa.scale, qb.zero_point, qb.bias, 4, 64))
 
 
 def test_bf16_cast_matches_tensor_cast_bit_for_bit():
