@@ -175,15 +175,17 @@ static inline bool bw_shape_ok(int64_t N, int64_t K, int bits, int group) {
 }
 static inline bool bw_aligned(const void* p, size_t a) { return ((uintptr_t)p & (a - 1)) == 0; }
 
-// Compute units of the current device (256 on MI355X); asked once.
+// Compute units of the current device (256 on MI355X); asked once per device.
 static inline int bw_device_cus() {
-    static const int cus = [] {
-        int dev = 0, n = 0;
-        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess)
-            n = 0;
-        return n > 0 ? n : 256;
-    }();
-    return cus;
+    static int cus[64] = {0};                                 // per device ordinal; a race writes the same value twice
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return 256;
+    int& slot = cus[dev & 63];
+    if (slot > 0) return slot;
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    slot = n;
+    return n;
 }
 
 // A kernel that wants more than 64 KiB of dynamic LDS has to be told so once per device.  `done` is the caller's

@@ -26,6 +26,7 @@
 #include "bw_common.h"
 
 #include <cstdlib>
+#include <type_traits>
 
 namespace {
 
@@ -77,6 +78,9 @@ struct GemvArgs {
     int x_bf16;                              // x holds bfloat16: every value is rounded to float16 as it is staged
     int ntiles, nsteps;                      // qgemv_tiles_kernel / qgemv_rounds_kernel: 16-row tiles of N; tiles or rounds per workgroup
     int meta_lds_off;                        // qgemv_tiles_kernel: where the scale blocks start in LDS
+#ifdef BW_TUNE
+    int tune;
+#endif
 };
 
 // two bfloat16 -> two float16, round to nearest even (what torch's .to(float16) does)
@@ -633,6 +637,70 @@ __global__ __launch_bounds__(1024) void qgemv_rounds_kernel(const GemvArgs a) {
     }
 }
 
+// ---- packed weights, memory -> LDS -> MFMA operand layout ---------------------------------------------------------
+//
+// The B operand of v_mfma_f32_16x16x32_f16 wants lane l to hold row (l & 15), 16-byte piece (l >> 4) of a chunk: loaded
+// that way straight from memory, neighbouring lanes touch 16 different rows and every 128-byte line of weights is
+// asked for by eight separate quarter-line requests.  Measured on MI355X (weights only, graph replay): 3.5 / 6.0 us
+// for the 8.4 / 22.5 MB of a Llama-7B projection that way, 2.8 / 4.8 us when eight neighbouring lanes ask for one
+// whole line and the loads carry the non-temporal hint (a weight byte is read once; the hint alone, without whole
+// lines, gains nothing).  So the weights take the coalesced route: a load instruction covers eight rows x 128 bytes
+// (two chunks), lands in LDS without passing through registers (16 bytes per lane at lane * 16), and the lane that
+// feeds the matrix core reads its 16 bytes back from there.  The piece a lane loads is XOR-swizzled with its row
+// (lane (a, s) of an instruction loads piece s ^ a of row a), so that the sixteen rows a read instruction touches
+// fall into different LDS banks; the second instruction of a pair (rows 8-15) sits 128 bytes further for the same reason.
+struct WeightTile {
+    static constexpr int kHalf = 1024 + 128;              // rows 0-7 | rows 8-15 of a pair of chunks
+    static constexpr int kPair = 2 * kHalf;               // LDS bytes per pair of chunks (16 rows x 128 bytes + padding)
+    static constexpr int kAuxNt = 2;                      // cache-policy bits of the buffer load: non-temporal
+
+    // request pair q of a wave's batch: chunks c, c + 1 of rows n0 .. n0 + 15 (rows past N and chunks past the row's end
+    // are range-checked to zero by the buffer resource)
+    static BW_DEV void request(const __amdgpu_buffer_rsrc_t& rw, char* tile, int q, uint32_t n0, int c, int row_bytes, int lane) {
+        const int a = lane >> 3, p = (lane & 7) ^ a;
+        const int cc = c + (p >> 2);
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+            uint32_t off = (n0 + 8 * i + a) * (uint32_t)row_bytes + cc * 64 + (p & 3) * 16;
+            asm volatile("" : "+v"(off));                     // a value of its own: the select below stays a select
+            off = cc * 64 < row_bytes ? off : 0x80000000u;
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, (__attribute__((address_space(3))) void*)(tile + q * kPair + i * kHalf),
+                                                     16, off, 0, 0, kAuxNt);
+        }
+    }
+    // the 16 bytes lane (n = lane & 15, j = lane >> 4) feeds the matrix core with for chunk b of the batch
+    static BW_DEV u4 fetch(const char* tile, int b, int lane) {
+        const int n = lane & 15, j = lane >> 4, a = n & 7, p = (b & 1) * 4 + j;
+        return *reinterpret_cast<const u4*>(tile + (b >> 1) * kPair + (n >> 3) * kHalf + (a * 8 + (p ^ a)) * 16);
+    }
+};
+
+// Workgroup barrier for LDS data that ordinary stores of this wave wrote: waits for the wave's own LDS operations and
+// then for the other waves, without the memory fence of __syncthreads() - a fence would also wait for every weight
+// request in flight, since those land in LDS too.
+BW_DEV void lds_barrier() {
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_waitcnt(0xC07F);                   // lgkmcnt(0)
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+}
+
+// f(integral_constant<int, 0>{}), ..., f(integral_constant<int, N - 1>{}): a loop whose index is a constant expression
+template <int I, int N, class F>
+BW_DEV void static_for(F&& f) {
+    if constexpr (I < N) {
+        f(std::integral_constant<int, I>{});
+        static_for<I + 1, N>(f);
+    }
+}
+
+// wait until at most `n` of this wave's memory loads are outstanding (loads return in order)
+template <int N>
+BW_DEV void wait_loads() {
+    static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
+    __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | 0x0F70);   // expcnt and lgkmcnt left alone
+}
+
 // ---- 4-bit, M <= 2: integer operands, scale and zero point taken out of the inner loop -------------------
 //
 // A masked packed word is already a float16: bits 0-3 of a half are the subnormal q * 2^-24, bits 4-7 the
@@ -662,103 +730,118 @@ BW_DEV float lanes_sum(float v) {
     return v;
 }
 
+// the buffer [p + skip, p + bytes): empty when `skip` lies past the end.  All operands are wave-uniform, so this is
+// scalar arithmetic; it lets the per-wave and per-round part of an address live in the descriptor (range-checked)
+// instead of in a per-lane add.
+BW_DEV __amdgpu_buffer_rsrc_t make_rsrc_at(const void* p, uint32_t bytes, uint32_t skip) {
+    // (readfirstlane: the saturating subtraction is a vector instruction even for uniform operands, and a descriptor
+    // the compiler cannot see to be uniform costs a loop around every load)
+    const uint32_t left = __builtin_amdgcn_readfirstlane(skip < bytes ? bytes - skip : 0u);
+    return make_rsrc(static_cast<const char*>(p) + skip, left);
+}
+
 template <int GROUP, int MT, int KB>
 __global__ __launch_bounds__(1024) void qgemv_w4_kernel(const GemvArgs a) {
     constexpr int NGC = 128 / GROUP;                      // groups per chunk
     constexpr int ROWS = MT * NGC;                        // MFMA rows in use: (m, group of the chunk)
     static_assert(ROWS <= 4, "the outputs must fit the four rows the lanes with kq == 0 hold");
+    static_assert(KB % 2 == 0, "weights are requested in pairs of chunks");
     constexpr int GL = GROUP / 8;                         // staging lanes per group (8 halves each)
+    constexpr int P = KB / 2;                             // pairs of chunks per wave and round
     constexpr int UPR = KB * 16;                          // 8-half units per activation row and round
     constexpr int XL = (MT * UPR + 63) / 64;              // unit loads per lane and round
     constexpr int ROW_BYTES = KB * 256 + 16, X_BYTES = ROWS * ROW_BYTES;
+    constexpr int KBG = KB * NGC, MP = KBG | 1;           // groups a wave covers per round; odd row pitch of its (scale, zp) block
+    constexpr int ML = (KBG + 3) / 4;                     // 2-byte requests per lane, array and round
+    constexpr int META_BYTES = (16 * MP * 4 + 15) & ~15;
+    constexpr int WAVE_BYTES = X_BYTES + META_BYTES + P * WeightTile::kPair;
     constexpr uint32_t kOob = 0x80000000u;
     extern __shared__ __attribute__((aligned(16))) char smem[];
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nwaves = blockDim.x >> 6;
+    const int tid = threadIdx.x, lane = tid & 63, nwaves = blockDim.x >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int nl = lane & 15, kq = lane >> 4;
-    const int n0 = blockIdx.x * 16;
-    // LDS: [(scale, zero point) pairs, 16 rows x GP][x tile of wave 0] ... [x tile of wave n-1][partial sums]
-    const int gcols = (a.groups + 31) & ~31, GP = gcols + 1;     // odd pitch: the 16 rows hit different banks
-    uint32_t* meta = reinterpret_cast<uint32_t*>(smem);
-    char* after_meta = smem + ((16 * GP * 4 + 15) & ~15);
-    char* xs = after_meta + wave * X_BYTES;
-    float* red = reinterpret_cast<float*>(after_meta + nwaves * X_BYTES);
-    const __amdgpu_buffer_rsrc_t rw = make_rsrc(a.qweight, a.w_bytes), rx = make_rsrc(a.x, a.x_bytes),
-                                 rs = make_rsrc(a.scale, a.meta_bytes), rz = make_rsrc(a.zp, a.meta_bytes);
+    const uint32_t n0 = blockIdx.x * 16;
+    // LDS, everything a wave touches before the final sum is its own (no workgroup barrier until then):
+    // [wave 0: x tile | (scale, zero point) pairs of its groups, 16 rows x MP | weight batch] ... [partial sums]
+    char* xs = smem + wave * WAVE_BYTES;
+    uint32_t* meta = reinterpret_cast<uint32_t*>(xs + X_BYTES);
+    char* wt = xs + X_BYTES + META_BYTES;
+    float* red = reinterpret_cast<float*>(smem + nwaves * WAVE_BYTES);
 
-    // Scales / zero points of the 16 rows: entry e = tid + j * blockDim is row (e / 32) % 16, column
-    // e % 32 + 32 * (e / 512).  The first ME entries of a thread are requested ahead of x and the weights
-    // (loads return in order: a request made later only comes back after the whole weight batch); shapes
-    // with more entries than that finish in a loop behind them.
-    constexpr int ME = 128 / GROUP;
-    const uint32_t meta_base = (uint32_t)n0 * a.groups * 2;
-    const int meta_entries = 16 * gcols;
-    auto meta_off = [&](int e) {
-        const int r = (e >> 5) & 15, c = (e & 31) + 32 * (e >> 9);
-        return c < a.groups ? meta_base + (r * a.groups + c) * 2 : kOob;
-    };
-    auto meta_slot = [&](int e) { return ((e >> 5) & 15) * GP + (e & 31) + 32 * (e >> 9); };
-    uint32_t ms[ME], mz[ME];
-#pragma unroll
-    for (int j = 0; j < ME; j++) {
-        ms[j] = mz[j] = 0;
-        if ((wave + j * nwaves) * 64 < meta_entries) {          // wave-uniform
-            const uint32_t off = meta_off(tid + j * (int)blockDim.x);
-            ms[j] = __builtin_amdgcn_raw_buffer_load_b16(rs, off, 0, 0);
-            mz[j] = __builtin_amdgcn_raw_buffer_load_b16(rz, off, 0, 0);
-        }
-    }
+    // the bias of the outputs the first MT waves will store, requested before anything else
+    uint32_t bias_v = 0;
+    if (wave < MT && a.bias)
+        bias_v = __builtin_amdgcn_raw_buffer_load_b16(make_rsrc(a.bias, (uint32_t)a.N * 2), (n0 + nl) * 2, 0, 0);
 
-    const uint32_t w_lane = (uint32_t)(n0 + nl) * a.row_bytes + kq * 16;
-    // where this lane's unit u = lane + 64 i of the round goes: activation row u / UPR, unit ku = u % UPR
+    // ---- per-lane parts of the addresses (the per-wave and per-round parts go into the descriptors)
+    // scales / zero points: lane (row lane / 4, column lane % 4 + 4 t) - four neighbouring lanes ask for 8 adjacent bytes
+    const uint32_t m_off = ((uint32_t)(lane >> 2) * a.groups + (lane & 3)) * 2;
+    uint32_t* m_dst = meta + (lane >> 2) * MP + (lane & 3);
+    // x: unit u = lane + 64 i of the round: activation row u / UPR, unit ku = u % UPR
     uint32_t x_off[XL], x_dst[XL];
 #pragma unroll
     for (int i = 0; i < XL; i++) {
         const int u = lane + 64 * i, m = u / UPR, ku = u % UPR;
-        x_off[i] = m < a.M ? (uint32_t)(m * a.ldx + ku * 8) * 2 : kOob;
+        x_off[i] = (MT == 1 || m < a.M) ? (uint32_t)(m * a.ldx + ku * 8) * 2 : kOob;
         x_dst[i] = m * NGC * ROW_BYTES + (ku >> 2) * 64 + (ku & 3) * 8;
     }
-    u4 xr[XL], wr[KB];
-    // x before the weights: loads return in order and the staging of x should overlap the weight stream
-    auto issue = [&](int c0) {
-#pragma unroll
-        for (int i = 0; i < XL; i++) {
-            const int ku = (lane + 64 * i) % UPR;
-            const uint32_t xo = (x_off[i] != kOob && c0 * 128 + ku * 8 < a.K) ? x_off[i] + c0 * 256 : kOob;
-            xr[i] = __builtin_amdgcn_raw_buffer_load_b128(rx, xo, 0, 0);
-        }
-        asm volatile("" ::: "memory");
-        const uint32_t off = c0 * 64 < a.row_bytes ? w_lane + c0 * 64 : kOob;
-#pragma unroll
-        for (int b = 0; b < KB; b++) wr[b] = __builtin_amdgcn_raw_buffer_load_b128(rw, off + b * 64, 0, 0);
-        asm volatile("" ::: "memory");
-    };
-    int c0 = wave * KB;
-    issue(c0);
-
-#pragma unroll
-    for (int j = 0; j < ME; j++) {
-        const int e = tid + j * (int)blockDim.x;
-        if (e < meta_entries) meta[meta_slot(e)] = ms[j] | (mz[j] << 16);
+    // weights: lane (row lane / 8 (+ 8 for the second instruction of a pair), piece (lane % 8) ^ row)
+    uint32_t w_off[2];
+    {
+        const int r = lane >> 3, p = (lane & 7) ^ r;
+        w_off[0] = (uint32_t)r * a.row_bytes + (p >> 2) * 64 + (p & 3) * 16;
+        w_off[1] = w_off[0] + 8u * a.row_bytes;
     }
-    for (int e = tid + ME * (int)blockDim.x; e < meta_entries; e += blockDim.x) {   // more entries than that
-        const uint32_t off = meta_off(e);
-        const uint32_t s2 = __builtin_amdgcn_raw_buffer_load_b16(rs, off, 0, 0);
-        const uint32_t z2 = __builtin_amdgcn_raw_buffer_load_b16(rz, off, 0, 0);
-        meta[meta_slot(e)] = s2 | (z2 << 16);
-    }
-    __syncthreads();
 
     float acc[MT];
 #pragma unroll
     for (int r = 0; r < MT; r++) acc[r] = 0.f;
     const char* xrow = xs + (nl < ROWS ? nl : ROWS - 1) * ROW_BYTES + kq * 64;
-    const uint32_t* mrow = meta + nl * GP;
+    const uint32_t* mrow = meta + nl * MP;
     const int my_group = ((lane & 15) * 8) / GROUP;       // group of the chunk this lane's staged unit lies in
     constexpr uint32_t kEven = 0x000F000Fu, kOdd = 0x00F000F0u;
+    int c0 = wave * KB;
     while (true) {
-        // stage the round's activations: even-k quartets (x0,x4,x2,x6) and odd-k quartets (x1,x5,x3,x7) of
-        // every 8 values, in the order the masks below emit the nibbles, into the row of their group (zeros
-        // into the rows of the chunk's other groups); and -2^-24 * sum(x) per group
+        // ---- requests, small things first (loads return in order): scales / zero points, x, then the weights
+        const uint32_t g0 = (uint32_t)c0 * NGC;           // first group of the round
+        const __amdgpu_buffer_rsrc_t rs = make_rsrc_at(a.scale, a.meta_bytes, (n0 * a.groups + g0) * 2),
+                                     rz = make_rsrc_at(a.zp, a.meta_bytes, (n0 * a.groups + g0) * 2),
+                                     rx = make_rsrc_at(a.x, a.x_bytes, (uint32_t)c0 * 256),
+                                     rw = make_rsrc_at(a.qweight, a.w_bytes, n0 * (uint32_t)a.row_bytes + (uint32_t)c0 * 64);
+        const int glim = min(KBG, a.groups - (int)g0);    // groups of the round that exist (the others read as zero)
+        uint32_t ms[ML], mz[ML];
+#pragma unroll
+        for (int t = 0; t < ML; t++) {
+            const uint32_t off = (lane & 3) + 4 * t < glim ? m_off : kOob;
+            ms[t] = __builtin_amdgcn_raw_buffer_load_b16(rs, off + 8 * t, 0, 0);
+            mz[t] = __builtin_amdgcn_raw_buffer_load_b16(rz, off + 8 * t, 0, 0);
+        }
+        u4 xr[XL];
+#pragma unroll
+        for (int i = 0; i < XL; i++) {
+            uint32_t xo = x_off[i];
+            if constexpr (MT > 1) {                           // one row: the end of x is the end of the buffer
+                const int ku = (lane + 64 * i) % UPR;
+                xo = c0 * 128 + ku * 8 < a.K ? xo : kOob;
+            }
+            xr[i] = __builtin_amdgcn_raw_buffer_load_b128(rx, xo, 0, 0);
+        }
+        asm volatile("" ::: "memory");
+        static_for<0, KB>([&](auto ic) {
+            constexpr int q = decltype(ic)::value / 2, i = decltype(ic)::value % 2;
+            // (the instruction's immediate offset moves the LDS destination as well as the memory address: taken off again here)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, (__attribute__((address_space(3))) void*)(wt + q * (WeightTile::kPair - 128) + i * WeightTile::kHalf),
+                                                     16, w_off[i], 0, q * 128, WeightTile::kAuxNt);
+        });
+        asm volatile("" ::: "memory");
+
+        // ---- scales / zero points -> this wave's block, as (scale | zero point << 16)
+#pragma unroll
+        for (int t = 0; t < ML; t++)
+            if (4 * t + 3 < KBG || (lane & 3) + 4 * t < KBG) m_dst[4 * t] = ms[t] | (mz[t] << 16);
+        // ---- the round's activations: even-k quartets (x0,x4,x2,x6) and odd-k quartets (x1,x5,x3,x7) of every 8
+        // values, in the order the masks below emit the nibbles, into the row of their group (zeros into the rows
+        // of the chunk's other groups); and -2^-24 * sum(x) per group
         float nsum[XL];
 #pragma unroll
         for (int i = 0; i < XL; i++) {
@@ -791,9 +874,15 @@ __global__ __launch_bounds__(1024) void qgemv_w4_kernel(const GemvArgs a) {
             nsum[i] = lanes_sum<GL>(t) * 0x1p-24f;
         }
         __builtin_amdgcn_wave_barrier();
-#pragma unroll
-        for (int b = 0; b < KB; b++) {
-            const u4 w = wr[b];
+        asm volatile("" ::: "memory");
+        static_for<0, KB>([&](auto bc) {
+            constexpr int b = decltype(bc)::value;
+            if constexpr ((b & 1) == 0) {                     // the pair's two load instructions have landed in LDS
+                wait_loads<KB - 2 - b>();
+                __builtin_amdgcn_wave_barrier();
+                asm volatile("" ::: "memory");                // the reads below stay below
+            }
+            const u4 w = WeightTile::fetch(wt, b, lane);
             u4 e0, e1, o0, o1;                            // B operands: even / odd nibbles of words 0,1 and 2,3
 #pragma unroll
             for (int j = 0; j < 2; j++) {
@@ -811,7 +900,7 @@ __global__ __launch_bounds__(1024) void qgemv_w4_kernel(const GemvArgs a) {
             po = __builtin_amdgcn_mfma_f32_16x16x32_f16(xp[3], __builtin_bit_cast(h8, o1), po, 0, 0, 0);
 #pragma unroll
             for (int g = 0; g < NGC; g++) {
-                const uint32_t sz = mrow[(c0 + b) * NGC + g];
+                const uint32_t sz = mrow[b * NGC + g];
                 const float sf = half_of(sz, 0), zf = half_of(sz, 1);
 #pragma unroll
                 for (int m = 0; m < MT; m++) {
@@ -822,11 +911,12 @@ __global__ __launch_bounds__(1024) void qgemv_w4_kernel(const GemvArgs a) {
                     acc[m] = __builtin_fmaf(sf, __builtin_fmaf(zf, ns, t), acc[m]);
                 }
             }
-        }
+        });
         c0 += nwaves * KB;
         if (c0 >= a.nchunks) break;                       // wave-uniform
+        __builtin_amdgcn_s_waitcnt(0xC07F);               // lgkmcnt(0): everything has been read out of LDS, the next round may land
         __builtin_amdgcn_wave_barrier();
-        issue(c0);
+        asm volatile("" ::: "memory");
     }
 
     // acc[m] = 2^-24 * partial y[m][n = nl] in the lanes with kq == 0
@@ -834,43 +924,66 @@ __global__ __launch_bounds__(1024) void qgemv_w4_kernel(const GemvArgs a) {
 #pragma unroll
         for (int r = 0; r < MT; r++) red[(wave * MT + r) * 16 + nl] = acc[r];
     }
-    __syncthreads();
-    // one wave per output row: the four 16-lane quarters each add every fourth partial sum, then fold
-    for (int m = wave; m < MT; m += nwaves) {
-        float v = 0.f;
-        for (int w = kq; w < nwaves; w += 4) v += red[(w * MT + m) * 16 + nl];
+    lds_barrier();
+    // wave m adds up row m: its four 16-lane quarters each take every fourth partial sum (all reads requested at
+    // once), then fold
+    if (wave < MT) {
+        const int m = wave;
+        float part[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+            if (kq + 4 * i < nwaves) part[i] = red[((kq + 4 * i) * MT + m) * 16 + nl];
+        float v = (part[0] + part[1]) + (part[2] + part[3]);
         v += __shfl_xor(v, 16);
         v += __shfl_xor(v, 32);
-        const int n = n0 + nl;
-        if (kq == 0 && m < a.M && n < a.N) {
-            v *= 0x1p24f;
-            if (a.bias) v += (float)a.bias[n];
+        const uint32_t n = n0 + nl;
+        asm volatile("" : "+v"(bias_v));                      // the wait for the bias belongs here, not behind its request
+        if (kq == 0 && m < a.M && n < (uint32_t)a.N) {
+            v = __builtin_fmaf(v, 0x1p24f, half_of(bias_v, 0));
             a.y[(int64_t)m * a.ldy + n] = (_Float16)v;
         }
     }
+}
+
+// LDS a workgroup of qgemv_w4_kernel<GROUP, MT, KB> needs with `nwaves` waves
+template <int GROUP, int MT, int KB>
+constexpr size_t w4_lds_bytes(int nwaves) {
+    constexpr int NGC = 128 / GROUP, MP = (KB * NGC) | 1;
+    constexpr int WAVE_BYTES = MT * NGC * (KB * 256 + 16) + ((16 * MP * 4 + 15) & ~15) + (KB / 2) * WeightTile::kPair;
+    return (size_t)nwaves * (WAVE_BYTES + MT * 64);
 }
 
 template <int GROUP, int MT, int KB>
 int launch_w4_kb(const GemvArgs& a, hipStream_t stream) {
     int nwaves = (a.nchunks + KB - 1) / KB;
     if (nwaves > 16) nwaves = 16;
-    const int gcols = (a.groups + 31) & ~31;
-    const size_t lds = (size_t)((16 * (gcols + 1) * 4 + 15) & ~15) +
-                       (size_t)nwaves * (MT * (128 / GROUP) * (KB * 256 + 16) + MT * 64);
+    while (nwaves > 1 && w4_lds_bytes<GROUP, MT, KB>(nwaves) > (size_t)160 * 1024) nwaves--;
+    const size_t lds = w4_lds_bytes<GROUP, MT, KB>(nwaves);
+    if (lds > (size_t)160 * 1024 || nwaves < MT) return BW_EUNSUPPORTED;
     auto kern = qgemv_w4_kernel<GROUP, MT, KB>;
     static uint64_t big_lds_devices = 0;                   // per instantiation
-    if (lds > 150 * 1024) return BW_EUNSUPPORTED;
     if (lds > 64 * 1024 && !bw_allow_big_lds(reinterpret_cast<const void*>(kern), big_lds_devices)) return BW_ELAUNCH;
     hipLaunchKernelGGL(kern, dim3((unsigned)((a.N + 15) / 16)), dim3(nwaves * 64), lds, stream, a);
     return hipGetLastError() == hipSuccess ? BW_OK : BW_ELAUNCH;
 }
 
-// BW_EUNSUPPORTED = the scale / zero-point block does not fit LDS; the caller falls back
+// BW_EUNSUPPORTED = nothing fits LDS; the caller falls back
 template <int GROUP, int MT>
 int launch_w4(const GemvArgs& a, hipStream_t stream) {
-    // chunks a wave has in flight per round: 2 for the small square projections (more, shorter waves), else 4
-    if (a.nchunks <= 32 && a.N <= 4096) return launch_w4_kb<GROUP, MT, 2>(a, stream);
-    return launch_w4_kb<GROUP, MT, 4>(a, stream);
+    // Chunks a wave requests per round (pairs, each landing in LDS), from timing the Llama-7B shapes on MI355X at
+    // M = 1 (us: 4096 x 4096 / 4096 -> 11008 / 11008 -> 4096): 2 chunks 4.00 / 7.02 / 6.20, 4 chunks 3.98 / 6.22 / 6.45,
+    // 8 chunks 4.24 / 6.45 / 6.95 - rows that fit one round of up to 16 waves take 4, longer rows many short rounds
+#ifdef BW_TUNE
+    if (const char* e = getenv("BW_W4_KB")) {
+        switch (atoi(e)) {
+            case 2: return launch_w4_kb<GROUP, MT, 2>(a, stream);
+            case 4: return launch_w4_kb<GROUP, MT, 4>(a, stream);
+            case 8: return launch_w4_kb<GROUP, MT, 8>(a, stream);
+        }
+    }
+#endif
+    if (a.nchunks <= 64) return launch_w4_kb<GROUP, MT, 4>(a, stream);
+    return launch_w4_kb<GROUP, MT, 2>(a, stream);
 }
 
 // ---- 2-bit, M <= 2: the same integer-operand scheme ---------------------------------------------------------
@@ -1158,6 +1271,10 @@ int launch_tiles(GemvArgs a, hipStream_t stream) {
     if (nwaves * 64 < 16 * MT) return BW_EUNSUPPORTED;
     a.ntiles = (a.N + 15) / 16;
     if (rounds == 1) {
+        // one 4-byte request per thread brings in a tile's scale block, and the waves wait on a counter for the
+        // ceil(8 groups / 64) waves that hold those requests: both need 8 groups <= threads.  (K <= 256 per wave
+        // and group >= 32 give exactly that today; a launch that breaks it must fall back, not hang.)
+        if (8 * a.groups > nwaves * 64) return BW_EUNSUPPORTED;
         // every workgroup resident at once (a CU holds 16 waves of this kernel: up to 128 registers each), each
         // running up to NTMAX tiles
         constexpr int NTMAX = BITS == 8 ? (MT == 16 ? 2 : 3) : 4;
@@ -1315,6 +1432,9 @@ extern "C" int bw_qgemv(const void* x, int act_dtype, int64_t M, int64_t K, int6
     a.w_bytes = (uint32_t)(N * a.row_bytes);
     a.meta_bytes = (uint32_t)(N * a.groups * 2);
     hipStream_t st = (hipStream_t)stream;
+#ifdef BW_TUNE
+    a.tune = getenv("BW_TUNE_FLAGS") ? atoi(getenv("BW_TUNE_FLAGS")) : 0;
+#endif
 #define BW_CASE(B, G) \
     if (bits == B && group == G) return launch_gemv<B, G>(a, st);
     BW_CASE(4, 128) BW_CASE(4, 64) BW_CASE(4, 32)
