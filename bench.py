@@ -207,9 +207,10 @@ def extras_decode_hot(torch, hip, QuantizedLinear, layers):
 
 
 def extras_decode_other_formats(torch, hip, QuantizedLinear, layers):
-    """K=4096 -> N=11008 at 8-bit g128, 4-bit g64, 2-bit g32 (weights with 0.1 % outliers x10), M = 1 and 16."""
-    k, n, out = 4096, 11008, {}
-    for bits, g in ((8, 128), (4, 64), (2, 32)):
+    """K=4096 -> N=11008 at 8-bit g128, 4-bit g64, 2-bit g32 (weights with 0.1 % outliers x10), M = 1 and 16; and the
+    8-bit attention linears of the mixed recipe: 4096 x 4096 and the fused q/k/v launch (N = 12288)."""
+    out = {}
+    for bits, g, k, n in ((8, 128, 4096, 11008), (4, 64, 4096, 11008), (2, 32, 4096, 11008), (8, 128, 4096, 4096), (8, 128, 4096, 12288)):
         copies = (320 << 20) // (n * k * bits // 8) + 1          # > 256 MiB of packed weights in rotation
         qs = [make_layer(torch, QuantizedLinear, k, n, bits, g, seed=31 * bits + i, outliers=True) for i in range(copies)]
         for mm in (1, 16):

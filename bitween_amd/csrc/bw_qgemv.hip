@@ -986,6 +986,251 @@ int launch_w4(const GemvArgs& a, hipStream_t stream) {
     return launch_w4_kb<GROUP, MT, 2>(a, stream);
 }
 
+// ---- 8-bit, M <= 4: the same integer-operand scheme ---------------------------------------------------------
+//
+// A byte in bits 0-7 of a half is the subnormal q * 2^-24, so a packed word becomes two operand dwords with two byte
+// permutes (bytes 0, 1 and bytes 2, 3, each byte zero-extended to a half): in natural k order, with a single
+// accumulator class - sum x q = 2^24 P - and x staged as it lies in memory, no permutation.  A chunk is 64 weights
+// of a row (two MFMAs); with groups of 128 two chunks accumulate into one group sum, with groups of 32 the two groups
+// of a chunk take the MFMA rows (m, group) as in the 4-bit kernel.  Weights arrive as in qgemv_w4_kernel (whole
+// cache lines, non-temporal, through LDS); everything before the final sum is private to a wave.
+template <int GROUP, int MT, int KB>
+__global__ __launch_bounds__(1024) void qgemv_w8_kernel(const GemvArgs a) {
+    constexpr int GPC = GROUP >= 64 ? 1 : 64 / GROUP;     // groups per chunk
+    constexpr int CPG = GROUP >= 64 ? GROUP / 64 : 1;     // chunks per group
+    constexpr int ROWS = MT * GPC;                        // MFMA rows in use: (m, group of the chunk)
+    static_assert(ROWS <= 4, "the outputs must fit the four rows the lanes with kq == 0 hold");
+    static_assert(KB % 2 == 0, "weights are requested in pairs of chunks");
+    constexpr int GL = GROUP / 8;                         // staging lanes per group (8 halves each)
+    constexpr int P = KB / 2;                             // pairs of chunks per wave and round
+    constexpr int UPR = KB * 8;                           // 8-half units per activation row and round
+    constexpr int XL = (MT * UPR + 63) / 64;              // unit loads per lane and round
+    constexpr int ROW_BYTES = KB * 128 + 16, X_BYTES = ROWS * ROW_BYTES;
+    constexpr int KBG = KB * 64 / GROUP, MP = KBG | 1;    // groups a wave covers per round; odd row pitch of its (scale, zp) block
+    constexpr int ML = (KBG + 3) / 4;                     // 2-byte requests per lane, array and round
+    constexpr int META_BYTES = (16 * MP * 4 + 15) & ~15;
+    constexpr int WAVE_BYTES = X_BYTES + META_BYTES + P * WeightTile::kPair;
+    constexpr uint32_t kOob = 0x80000000u;
+    static_assert(UPR % GL == 0, "a group's staging lanes must not straddle activation rows");
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    const int tid = threadIdx.x, lane = tid & 63, nwaves = blockDim.x >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int nl = lane & 15, kq = lane >> 4;
+    const uint32_t n0 = blockIdx.x * 16;
+    // LDS: [wave 0: x tile | (scale, zero point) pairs of its groups, 16 rows x MP | weight batch] ... [partial sums]
+    char* xs = smem + wave * WAVE_BYTES;
+    uint32_t* meta = reinterpret_cast<uint32_t*>(xs + X_BYTES);
+    char* wt = xs + X_BYTES + META_BYTES;
+    float* red = reinterpret_cast<float*>(smem + nwaves * WAVE_BYTES);
+
+    // the bias of the outputs the first MT waves will store, requested before anything else
+    uint32_t bias_v = 0;
+    if (wave < MT && a.bias)
+        bias_v = __builtin_amdgcn_raw_buffer_load_b16(make_rsrc(a.bias, (uint32_t)a.N * 2), (n0 + nl) * 2, 0, 0);
+
+    // ---- per-lane parts of the addresses (the per-wave and per-round parts go into the descriptors)
+    const uint32_t m_off = ((uint32_t)(lane >> 2) * a.groups + (lane & 3)) * 2;
+    uint32_t* m_dst = meta + (lane >> 2) * MP + (lane & 3);
+    // x: unit u = lane + 64 i of the round: activation row u / UPR, unit ku = u % UPR, kept in memory order
+    uint32_t x_off[XL], x_dst[XL];
+#pragma unroll
+    for (int i = 0; i < XL; i++) {
+        const int u = lane + 64 * i, m = u / UPR, ku = u % UPR;
+        x_off[i] = (MT == 1 || m < a.M) ? (uint32_t)(m * a.ldx + ku * 8) * 2 : kOob;
+        x_dst[i] = m * GPC * ROW_BYTES + ku * 16;
+    }
+    uint32_t w_off[2];
+    {
+        const int r = lane >> 3, p = (lane & 7) ^ r;
+        w_off[0] = (uint32_t)r * a.row_bytes + (p >> 2) * 64 + (p & 3) * 16;
+        w_off[1] = w_off[0] + 8u * a.row_bytes;
+    }
+
+    float acc[MT];
+#pragma unroll
+    for (int r = 0; r < MT; r++) acc[r] = 0.f;
+    const char* xrow = xs + (nl < ROWS ? nl : ROWS - 1) * ROW_BYTES + kq * 32;
+    const uint32_t* mrow = meta + nl * MP;
+    int c0 = wave * KB;
+    while (true) {
+        // ---- requests, small things first (loads return in order): scales / zero points, x, then the weights
+        const uint32_t g0 = (uint32_t)c0 * 64 / GROUP;    // first group of the round
+        const __amdgpu_buffer_rsrc_t rs = make_rsrc_at(a.scale, a.meta_bytes, (n0 * a.groups + g0) * 2),
+                                     rz = make_rsrc_at(a.zp, a.meta_bytes, (n0 * a.groups + g0) * 2),
+                                     rx = make_rsrc_at(a.x, a.x_bytes, (uint32_t)c0 * 128),
+                                     rw = make_rsrc_at(a.qweight, a.w_bytes, n0 * (uint32_t)a.row_bytes + (uint32_t)c0 * 64);
+        const int glim = min(KBG, a.groups - (int)g0);    // groups of the round that exist (the others read as zero)
+        uint32_t ms[ML], mz[ML];
+#pragma unroll
+        for (int t = 0; t < ML; t++) {
+            const uint32_t off = (lane & 3) + 4 * t < glim ? m_off : kOob;
+            ms[t] = __builtin_amdgcn_raw_buffer_load_b16(rs, off + 8 * t, 0, 0);
+            mz[t] = __builtin_amdgcn_raw_buffer_load_b16(rz, off + 8 * t, 0, 0);
+        }
+        u4 xr[XL];
+#pragma unroll
+        for (int i = 0; i < XL; i++) {
+            uint32_t xo = x_off[i];
+            if constexpr (MT > 1) {                           // one row: the end of x is the end of the buffer
+                const int ku = (lane + 64 * i) % UPR;
+                xo = c0 * 64 + ku * 8 < a.K ? xo : kOob;
+            }
+            xr[i] = __builtin_amdgcn_raw_buffer_load_b128(rx, xo, 0, 0);
+        }
+        asm volatile("" ::: "memory");
+        static_for<0, KB>([&](auto ic) {
+            constexpr int q = decltype(ic)::value / 2, i = decltype(ic)::value % 2;
+            // (the instruction's immediate offset moves the LDS destination as well as the memory address: taken off again here)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, (__attribute__((address_space(3))) void*)(wt + q * (WeightTile::kPair - 128) + i * WeightTile::kHalf),
+                                                     16, w_off[i], 0, q * 128, WeightTile::kAuxNt);
+        });
+        asm volatile("" ::: "memory");
+
+        // ---- scales / zero points -> this wave's block, as (scale | zero point << 16)
+#pragma unroll
+        for (int t = 0; t < ML; t++)
+            if (4 * t + 3 < KBG || (lane & 3) + 4 * t < KBG) m_dst[4 * t] = ms[t] | (mz[t] << 16);
+        // ---- the round's activations, as they lie in memory (into the row of their group where a chunk holds two
+        // groups, zeros into the other's row); and -2^-24 * sum(x) per group
+        float nsum[XL];
+#pragma unroll
+        for (int i = 0; i < XL; i++) {
+            u4 v = xr[i];
+            if (a.x_bf16) {
+#pragma unroll
+                for (int j = 0; j < 4; j++) v[j] = bf16x2_to_f16x2(v[j]);
+            }
+            if (MT * UPR >= 64 * (i + 1) || lane + 64 * i < MT * UPR) {
+                const int my_group = (((lane + 64 * i) % UPR) * 8 % 64) / (GROUP >= 64 ? 64 : GROUP);   // group of its chunk this unit lies in
+#pragma unroll
+                for (int g = 0; g < GPC; g++) {
+                    const bool mine = GPC == 1 || g == my_group;
+                    *reinterpret_cast<u4*>(xs + x_dst[i] + g * ROW_BYTES) = mine ? v : u4{0u, 0u, 0u, 0u};
+                }
+            }
+            float t = 0.f;
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const h2 p = __builtin_bit_cast(h2, (uint32_t)v[j]);
+                t -= (float)p[0];
+                t -= (float)p[1];
+            }
+            nsum[i] = lanes_sum<GL>(t) * 0x1p-24f;
+        }
+        __builtin_amdgcn_wave_barrier();
+        asm volatile("" ::: "memory");
+        f4 p = {0.f, 0.f, 0.f, 0.f};
+        static_for<0, KB>([&](auto bc) {
+            constexpr int b = decltype(bc)::value;
+            if constexpr ((b & 1) == 0) {                     // the pair's two load instructions have landed in LDS
+                wait_loads<KB - 2 - b>();
+                __builtin_amdgcn_wave_barrier();
+                asm volatile("" ::: "memory");                // the reads below stay below
+            }
+            const u4 w = WeightTile::fetch(wt, b, lane);
+            u4 b0, b1;                                    // B operands: the bytes of words 0, 1 and of words 2, 3 as halves
+#pragma unroll
+            for (int j = 0; j < 2; j++) {
+                b0[2 * j] = __builtin_amdgcn_perm(0u, w[j], 0x0C010C00u);
+                b0[2 * j + 1] = __builtin_amdgcn_perm(0u, w[j], 0x0C030C02u);
+                b1[2 * j] = __builtin_amdgcn_perm(0u, w[2 + j], 0x0C010C00u);
+                b1[2 * j + 1] = __builtin_amdgcn_perm(0u, w[2 + j], 0x0C030C02u);
+            }
+            const h8* xp = reinterpret_cast<const h8*>(xrow + b * 128);
+            if constexpr (b % CPG == 0) p = f4{0.f, 0.f, 0.f, 0.f};
+            p = __builtin_amdgcn_mfma_f32_16x16x32_f16(xp[0], __builtin_bit_cast(h8, b0), p, 0, 0, 0);
+            p = __builtin_amdgcn_mfma_f32_16x16x32_f16(xp[1], __builtin_bit_cast(h8, b1), p, 0, 0, 0);
+            if constexpr (b % CPG == CPG - 1) {
+#pragma unroll
+                for (int g = 0; g < GPC; g++) {
+                    constexpr int gbase = (b / CPG) * GPC;    // first group of the round this chunk closes
+                    const uint32_t sz = mrow[gbase + g];
+                    const float sf = half_of(sz, 0), zf = half_of(sz, 1);
+#pragma unroll
+                    for (int m = 0; m < MT; m++) {
+                        // the sum of (row m, group) sits in the lanes that staged it: unit m * UPR + (gbase + g) * GL
+                        const int u = m * UPR + (gbase + g) * GL, r = m * GPC + g;
+                        const float ns = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, nsum[u / 64]), u % 64));
+                        acc[m] = __builtin_fmaf(sf, __builtin_fmaf(zf, ns, p[r]), acc[m]);
+                    }
+                }
+            }
+        });
+        c0 += nwaves * KB;
+        if (c0 >= a.nchunks) break;                       // wave-uniform
+        __builtin_amdgcn_s_waitcnt(0xC07F);               // lgkmcnt(0): everything has been read out of LDS, the next round may land
+        __builtin_amdgcn_wave_barrier();
+        asm volatile("" ::: "memory");
+    }
+
+    // acc[m] = 2^-24 * partial y[m][n = nl] in the lanes with kq == 0
+    if (kq == 0) {
+#pragma unroll
+        for (int r = 0; r < MT; r++) red[(wave * MT + r) * 16 + nl] = acc[r];
+    }
+    lds_barrier();
+    if (wave < MT) {
+        const int m = wave;
+        float part[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+            if (kq + 4 * i < nwaves) part[i] = red[((kq + 4 * i) * MT + m) * 16 + nl];
+        float v = (part[0] + part[1]) + (part[2] + part[3]);
+        v += __shfl_xor(v, 16);
+        v += __shfl_xor(v, 32);
+        const uint32_t n = n0 + nl;
+        asm volatile("" : "+v"(bias_v));                      // the wait for the bias belongs here, not behind its request
+        if (kq == 0 && m < a.M && n < (uint32_t)a.N) {
+            v = __builtin_fmaf(v, 0x1p24f, half_of(bias_v, 0));
+            a.y[(int64_t)m * a.ldy + n] = (_Float16)v;
+        }
+    }
+}
+
+template <int GROUP, int MT, int KB>
+constexpr size_t w8_lds_bytes(int nwaves) {
+    constexpr int GPC = GROUP >= 64 ? 1 : 64 / GROUP, MP = (KB * 64 / GROUP) | 1;
+    constexpr int WAVE_BYTES = MT * GPC * (KB * 128 + 16) + ((16 * MP * 4 + 15) & ~15) + (KB / 2) * WeightTile::kPair;
+    return (size_t)nwaves * (WAVE_BYTES + MT * 64);
+}
+
+template <int GROUP, int MT, int KB>
+int launch_w8_kb(const GemvArgs& a, hipStream_t stream) {
+    int nwaves = (a.nchunks + KB - 1) / KB;
+    if (nwaves > 16) nwaves = 16;
+    while (nwaves > 1 && w8_lds_bytes<GROUP, MT, KB>(nwaves) > (size_t)160 * 1024) nwaves--;
+    const size_t lds = w8_lds_bytes<GROUP, MT, KB>(nwaves);
+    if (lds > (size_t)160 * 1024 || nwaves < MT) return BW_EUNSUPPORTED;
+    auto kern = qgemv_w8_kernel<GROUP, MT, KB>;
+    static uint64_t big_lds_devices = 0;                   // per instantiation
+    if (lds > 64 * 1024 && !bw_allow_big_lds(reinterpret_cast<const void*>(kern), big_lds_devices)) return BW_ELAUNCH;
+    hipLaunchKernelGGL(kern, dim3((unsigned)((a.N + 15) / 16)), dim3(nwaves * 64), lds, stream, a);
+    return hipGetLastError() == hipSuccess ? BW_OK : BW_ELAUNCH;
+}
+
+template <int GROUP, int MT>
+int launch_w8(const GemvArgs& a, hipStream_t stream) {
+#ifdef BW_TUNE
+    if (const char* e = getenv("BW_W8_KB")) {
+        switch (atoi(e)) {
+            case 2: return launch_w8_kb<GROUP, MT, 2>(a, stream);
+            case 4: return launch_w8_kb<GROUP, MT, 4>(a, stream);
+            case 8: return launch_w8_kb<GROUP, MT, 8>(a, stream);
+        }
+    }
+#endif
+    // Chunks a wave requests per round: the largest batch whose workgroups still all fit the chip at once (a grid of
+    // 688 tiles wants three workgroups per compute unit, and the weight batches are what fills LDS).  Measured, M = 1,
+    // groups of 128 (us: 4096 x 4096 / 4096 -> 11008 / 11008 -> 4096): 2 chunks 5.59 / 10.40 / 11.81, 4 chunks
+    // 5.59 / 12.45 / 11.42, 8 chunks 5.36 / 11.90 / 11.39.
+    const int cus = bw_device_cus(), tiles = (a.N + 15) / 16;
+    const size_t per_wg = (size_t)160 * 1024 / (size_t)(tiles <= cus ? 1 : (tiles + cus - 1) / cus > 4 ? 4 : (tiles + cus - 1) / cus);
+    auto waves = [&](int kb) { const int w = (a.nchunks + kb - 1) / kb; return w > 16 ? 16 : w; };
+    if (w8_lds_bytes<GROUP, MT, 8>(waves(8)) <= per_wg) return launch_w8_kb<GROUP, MT, 8>(a, stream);
+    if (w8_lds_bytes<GROUP, MT, 4>(waves(4)) <= per_wg) return launch_w8_kb<GROUP, MT, 4>(a, stream);
+    return launch_w8_kb<GROUP, MT, 2>(a, stream);
+}
+
 // ---- 2-bit, M <= 2: the same integer-operand scheme ---------------------------------------------------------
 //
 // A masked 2-bit field at bits 2c..2c+1 (c = 0..3) of a half is the subnormal q * 4^c * 2^-24; the fields at bits
@@ -1373,19 +1618,46 @@ int tiles_min_rows(int nchunks) {
 
 template <int BITS, int GROUP>
 int launch_gemv(const GemvArgs& a, hipStream_t stream) {
+    constexpr int KBW = BITS == 4 ? 2 : (BITS == 8 ? 4 : 1);
+    const bool one_round = a.nchunks <= 16 * KBW;         // K fits one round of qgemv_tiles_kernel
+    const bool many_tiles = (a.N + 15) / 16 > bw_device_cus();
+    // The subnormal-operand kernels first, where they win (timed on the Llama-7B shapes, MI355X).
+    if constexpr (BITS == 8) {
+        // rows of the MFMA tile in use = M * groups per chunk, at most 4: faster than the tile kernels on every shape
+        constexpr int GPC = GROUP >= 64 ? 1 : 64 / GROUP;
+#ifdef BW_TUNE
+        if (!getenv("BW_W8_OFF"))
+#endif
+        if (a.M * GPC <= 4) {
+            const int st = a.M == 1 ? launch_w8<GROUP, 1>(a, stream)
+                         : a.M == 2 ? launch_w8<GROUP, 2>(a, stream)
+                                    : launch_w8<GROUP, (GPC == 1 ? 4 : 2)>(a, stream);
+            if (st != BW_EUNSUPPORTED) return st;
+        }
+    }
+    if constexpr (BITS == 4) {
+        // rows in use = M * groups per chunk, at most 4.  At 3 and 4 rows (groups of 128) the tile kernel is ahead
+        // where a workgroup gets several tiles out of one staging of x (one round of K, more tiles than compute
+        // units: 7.4 against 7.9 us on 4096 -> 11008), this one elsewhere (4.4 against 4.7 us on 4096 x 4096, 7.4
+        // against 8.5 us on 11008 -> 4096).
+        const bool first = a.M <= 2 || !(one_round && many_tiles);
+#ifdef BW_TUNE
+        if (!getenv("BW_W4_OFF"))
+#endif
+        if (a.M * (128 / GROUP) <= 4 && first) {
+            const int st = a.M == 1 ? launch_w4<GROUP, 1>(a, stream)
+                         : a.M == 2 ? launch_w4<GROUP, (GROUP >= 64 ? 2 : 1)>(a, stream)
+                                    : launch_w4<GROUP, (GROUP == 128 ? 4 : 1)>(a, stream);
+            if (st != BW_EUNSUPPORTED) return st;
+        }
+    }
+#ifdef BW_TUNE
+    if (!getenv("BW_TILES_OFF"))
+#endif
     if (a.M >= tiles_min_rows<BITS, GROUP>(a.nchunks)) {
         const int st = a.M <= 4 ? launch_tiles<BITS, GROUP, 4>(a, stream)
                                 : (a.M <= 8 ? launch_tiles<BITS, GROUP, 8>(a, stream) : launch_tiles<BITS, GROUP, 16>(a, stream));
         if (st != BW_EUNSUPPORTED) return st;
-    }
-    if constexpr (BITS == 4) {
-        // rows of the MFMA tile in use = M * groups per chunk, at most 4.  With groups of 64 the doubled
-        // activation rows cost more than the cheaper unpack saves until the weights reach about 16 MiB.
-        const bool pays = GROUP != 64 || (int64_t)a.N * a.K > (int64_t)1 << 25;
-        if (a.M * (128 / GROUP) <= 4 && a.M <= 2 && pays) {
-            const int st = a.M == 1 ? launch_w4<GROUP, 1>(a, stream) : launch_w4<GROUP, (GROUP >= 64 ? 2 : 1)>(a, stream);
-            if (st != BW_EUNSUPPORTED) return st;
-        }
     }
     if constexpr (BITS == 2) {
         if (a.M <= 2) {

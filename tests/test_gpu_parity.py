@@ -517,7 +517,11 @@ def test_error_conventions_on_gpu():
 
 @pytest.mark.parametrize("bits,g,k,n", [(4, 128, 4096, 11008), (4, 128, 11008, 4096), (8, 128, 4096, 11008),
                                         (4, 64, 4096, 11008), (2, 32, 4096, 11008), (4, 128, 4096, 4096),
-                                        (4, 32, 11008, 4096), (4, 64, 11008, 4096), (2, 32, 11008, 4096)])
+                                        (4, 32, 11008, 4096), (4, 64, 11008, 4096), (2, 32, 11008, 4096),
+                                        # the attention linears of the mixed recipe: 8-bit on 4096 x 4096 and on the fused
+                                        # q/k/v launch (N = 12288); 8-bit on a long K and at the smaller groups
+                                        (8, 128, 4096, 4096), (8, 128, 4096, 12288), (8, 128, 11008, 4096),
+                                        (8, 64, 4096, 4096), (8, 32, 4096, 11008)])
 def test_full_size_properties(bits, g, k, n):
     """Full-size layers (Llama-2-7B shapes), checked through size-independent properties:
       * a one-hot activation row returns a column of W16 bit-for-bit (the fused kernels reproduce the
@@ -552,6 +556,14 @@ def test_full_size_properties(bits, g, k, n):
         y1 = hip.quantized_gemv_hip(x[1:], q.qweight, q.scale, q.zero_point, None, bits, g)
         assert torch.equal(y2[0], w16[:, cols[i]]) and torch.equal(y2[1], w16[:, cols[i + 1]])
         assert torch.equal(y1[0], w16[:, cols[i + 1]])
+    # and through the three- and four-row forms (4-bit groups of 128 and 8-bit: still the subnormal-operand kernels)
+    for m in (3, 4):
+        x = torch.zeros(m, k, device="cuda", dtype=torch.float16)
+        for i in range(m):
+            x[i, cols[(i + m) % len(cols)]] = 1.0
+        y = hip.quantized_gemv_hip(x, q.qweight, q.scale, q.zero_point, None, bits, g)
+        for i in range(m):
+            assert torch.equal(y[i], w16[:, cols[(i + m) % len(cols)]])
     # reconstruction bound
     w32 = hip.dequantize(q.qweight, q.scale, q.zero_point, g, bits, torch.float32)
     qmax = (1 << bits) - 1
