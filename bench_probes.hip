@@ -2,7 +2,7 @@
 // of the quantized-linear library.
 //   probe_launch_floor   device time per launch of an empty kernel when `launches` dependent launches are replayed
 //                        from one HIP graph (what separates two kernels of a decode step)
-//   probe_read_rate      a kernel that only reads `bytes` of device memory: GB/s
+//   probe_read_rate      a kernel that only reads `bytes` of device memory, by grid, block, loads in flight and cache hint: GB/s
 //   probe_mfma_issue     v_mfma_f32_16x16x32_f16 back to back, one wave per SIMD, 32 independent accumulator tiles, with
 //                        0..3 independent VALU instructions after every MFMA: ns per MFMA and wave (how many issue
 //                        slots a single wave has per MFMA)
@@ -20,13 +20,18 @@ __global__ void empty_kernel(int* p) {
     if (p && threadIdx.x == 0x7fffffff) p[0] = 1;
 }
 
-__global__ __launch_bounds__(256) void read_kernel(const u4v* __restrict__ s, int* out, size_t n) {
-    size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
-    const size_t st = (size_t)gridDim.x * 256;
+// grid-stride read of n 16-byte words with UNROLL loads in flight per lane; NT = the loads carry the non-temporal hint
+template <int UNROLL, bool NT>
+__global__ __launch_bounds__(1024) void read_kernel(const u4v* __restrict__ s, int* out, size_t n) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t st = (size_t)gridDim.x * blockDim.x;
     unsigned acc = 0;
-    for (; i + 3 * st < n; i += 4 * st) {
-        const u4v a = s[i], b = s[i + st], c = s[i + 2 * st], e = s[i + 3 * st];
-        acc ^= a.x ^ b.y ^ c.z ^ e.w;
+    for (; i + (UNROLL - 1) * st < n; i += UNROLL * st) {
+        u4v v[UNROLL];
+#pragma unroll
+        for (int u = 0; u < UNROLL; u++) v[u] = NT ? __builtin_nontemporal_load(&s[i + u * st]) : s[i + u * st];
+#pragma unroll
+        for (int u = 0; u < UNROLL; u++) acc ^= v[u].x ^ v[u].w;
     }
     for (; i < n; i += st) acc ^= s[i].x;
     if (acc == 0x12345u) out[0] = 1;                          // keeps the loads alive; practically never true
@@ -98,14 +103,26 @@ extern "C" double probe_launch_floor(int launches, int grid, int block, int repl
     return us;
 }
 
-// `src`: `bytes` of device memory (16-byte aligned, a multiple of 16), `scratch`: 4 bytes of device memory
-extern "C" double probe_read_rate(const void* src, size_t bytes, void* scratch, int grid, int runs) {
-    if (!src || !scratch || bytes < 16 || bytes % 16 || grid < 1 || runs < 1 || ((uintptr_t)src & 15)) return -1.0;
+// `src`: `bytes` of device memory (16-byte aligned, a multiple of 16), `scratch`: 4 bytes of device memory.
+// `unroll` 4 or 8 loads in flight per lane, `nontemporal` 0 / 1, `grid` workgroups of `block` threads.
+extern "C" double probe_read_rate(const void* src, size_t bytes, void* scratch, int grid, int block, int unroll, int nontemporal, int runs) {
+    if (!src || !scratch || bytes < 16 || bytes % 16 || grid < 1 || block < 64 || block > 1024 || block % 64 || runs < 1 ||
+        (unroll != 4 && unroll != 8) || ((uintptr_t)src & 15))
+        return -1.0;
     Timer t;
     if (!t.ok) return -2.0;
-    hipLaunchKernelGGL(read_kernel, dim3(grid), dim3(256), 0, 0, (const u4v*)src, (int*)scratch, bytes / 16);
+    auto launch = [&]() {
+        const u4v* p = (const u4v*)src;
+        int* o = (int*)scratch;
+        const size_t n = bytes / 16;
+        if (unroll == 4 && !nontemporal) hipLaunchKernelGGL((read_kernel<4, false>), dim3(grid), dim3(block), 0, 0, p, o, n);
+        else if (unroll == 4) hipLaunchKernelGGL((read_kernel<4, true>), dim3(grid), dim3(block), 0, 0, p, o, n);
+        else if (!nontemporal) hipLaunchKernelGGL((read_kernel<8, false>), dim3(grid), dim3(block), 0, 0, p, o, n);
+        else hipLaunchKernelGGL((read_kernel<8, true>), dim3(grid), dim3(block), 0, 0, p, o, n);
+    };
+    launch();
     if (hipDeviceSynchronize() != hipSuccess || hipEventRecord(t.a, 0) != hipSuccess) return -2.0;
-    for (int i = 0; i < runs; i++) hipLaunchKernelGGL(read_kernel, dim3(grid), dim3(256), 0, 0, (const u4v*)src, (int*)scratch, bytes / 16);
+    for (int i = 0; i < runs; i++) launch();
     float ms = 0.f;
     if (hipEventRecord(t.b, 0) != hipSuccess || hipDeviceSynchronize() != hipSuccess || hipEventElapsedTime(&ms, t.a, t.b) != hipSuccess)
         return -2.0;

@@ -28,7 +28,20 @@
 #include <cstdlib>
 #include <type_traits>
 
+#include <string>
+
 namespace {
+
+// Name of the decode kernel this thread launched last (bw_qgemv_last_kernel): lets a benchmark label its numbers
+// with the kernel that actually ran.  The string is built once per kernel instantiation; a launch only stores a pointer.
+thread_local const char* g_last_kernel = "";
+inline const char* kernel_name(const char* base, std::initializer_list<int> params) {
+    std::string s = std::string(base) + "<";
+    bool first = true;
+    for (int v : params) { s += (first ? "" : ", ") + std::to_string(v); first = false; }
+    return (new std::string(s + ">"))->c_str();           // lives as long as the library
+}
+#define BW_NOTE_KERNEL(base, ...) do { static const char* const nm = kernel_name(base, {__VA_ARGS__}); g_last_kernel = nm; } while (0)
 
 template <int BITS, int GROUP, int MT>
 struct GemvCfg {
@@ -961,6 +974,7 @@ int launch_w4_kb(const GemvArgs& a, hipStream_t stream) {
     const size_t lds = w4_lds_bytes<GROUP, MT, KB>(nwaves);
     if (lds > (size_t)160 * 1024 || nwaves < MT) return BW_EUNSUPPORTED;
     auto kern = qgemv_w4_kernel<GROUP, MT, KB>;
+    BW_NOTE_KERNEL("qgemv_w4_kernel", GROUP, MT, KB);
     static uint64_t big_lds_devices = 0;                   // per instantiation
     if (lds > 64 * 1024 && !bw_allow_big_lds(reinterpret_cast<const void*>(kern), big_lds_devices)) return BW_ELAUNCH;
     hipLaunchKernelGGL(kern, dim3((unsigned)((a.N + 15) / 16)), dim3(nwaves * 64), lds, stream, a);
@@ -1202,6 +1216,7 @@ int launch_w8_kb(const GemvArgs& a, hipStream_t stream) {
     const size_t lds = w8_lds_bytes<GROUP, MT, KB>(nwaves);
     if (lds > (size_t)160 * 1024 || nwaves < MT) return BW_EUNSUPPORTED;
     auto kern = qgemv_w8_kernel<GROUP, MT, KB>;
+    BW_NOTE_KERNEL("qgemv_w8_kernel", GROUP, MT, KB);
     static uint64_t big_lds_devices = 0;                   // per instantiation
     if (lds > 64 * 1024 && !bw_allow_big_lds(reinterpret_cast<const void*>(kern), big_lds_devices)) return BW_ELAUNCH;
     hipLaunchKernelGGL(kern, dim3((unsigned)((a.N + 15) / 16)), dim3(nwaves * 64), lds, stream, a);
@@ -1462,6 +1477,7 @@ int launch_w2_kb(const GemvArgs& a, hipStream_t stream) {
     const size_t lds = fixed + (size_t)nwaves * (WAVE_BYTES + MT * 64);
     if (lds > (size_t)150 * 1024) return BW_EUNSUPPORTED;
     auto kern = qgemv_w2_kernel<GROUP, MT, KB>;
+    BW_NOTE_KERNEL("qgemv_w2_kernel", GROUP, MT, KB);
     static uint64_t big_lds_devices = 0;                   // per instantiation
     if (lds > 64 * 1024 && !bw_allow_big_lds(reinterpret_cast<const void*>(kern), big_lds_devices)) return BW_ELAUNCH;
     hipLaunchKernelGGL(kern, dim3((unsigned)((a.N + 15) / 16)), dim3(nwaves * 64), lds, stream, a);
@@ -1481,6 +1497,7 @@ constexpr int kLdsBudget = 150 * 1024;
 template <int BITS, int GROUP, int MT, int NT>
 int launch_tiles_nt(const GemvArgs& a, int grid, int nwaves, size_t lds, hipStream_t stream) {
     auto kern = qgemv_tiles_kernel<BITS, GROUP, MT, NT>;
+    BW_NOTE_KERNEL("qgemv_tiles_kernel", BITS, GROUP, MT, NT);
     static uint64_t big_lds_devices = 0;                   // per instantiation
     if (lds > 64 * 1024 && !bw_allow_big_lds(reinterpret_cast<const void*>(kern), big_lds_devices)) return BW_ELAUNCH;
     hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(nwaves * 64), lds, stream, a);
@@ -1490,6 +1507,7 @@ int launch_tiles_nt(const GemvArgs& a, int grid, int nwaves, size_t lds, hipStre
 template <int BITS, int GROUP, int MT, int DEPTH, bool LOOP>
 int launch_rounds_depth(const GemvArgs& a, int grid, int nwaves, size_t lds, hipStream_t stream) {
     auto kern = qgemv_rounds_kernel<BITS, GROUP, MT, DEPTH, LOOP>;
+    BW_NOTE_KERNEL("qgemv_rounds_kernel", BITS, GROUP, MT, DEPTH, (int)LOOP);
     static uint64_t big_lds_devices = 0;                   // per instantiation
     if (lds > 64 * 1024 && !bw_allow_big_lds(reinterpret_cast<const void*>(kern), big_lds_devices)) return BW_ELAUNCH;
     hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(nwaves * 64), lds, stream, a);
@@ -1578,6 +1596,7 @@ int launch_gemv_kb(const GemvArgs& a, hipStream_t stream) {
     const size_t lds = fixed + (size_t)nwaves * (X_BYTES + MT * 64);
     if (lds > (size_t)kLdsBudget) return BW_EUNSUPPORTED;
     auto kern = qgemv_kernel<BITS, GROUP, MT, KB>;
+    BW_NOTE_KERNEL("qgemv_kernel", BITS, GROUP, MT, KB);
     static uint64_t big_lds_devices = 0;                   // per instantiation
     if (lds > 64 * 1024 && !bw_allow_big_lds(reinterpret_cast<const void*>(kern), big_lds_devices)) return BW_ELAUNCH;
     hipLaunchKernelGGL(kern, dim3((unsigned)((a.N + 15) / 16)), dim3(nwaves * 64), lds, stream, a);
@@ -1685,12 +1704,15 @@ int bw_qgemm_generic(const void* x, int act_dtype, int64_t M, int64_t K, int64_t
                      const void* scale16, const void* zp16, const void* bias, int64_t N, int bits, int group, void* y,
                      int64_t ldy, void* stream);
 
+extern "C" const char* bw_qgemv_last_kernel(void) { return g_last_kernel; }
+
 extern "C" int bw_qgemv(const void* x, int act_dtype, int64_t M, int64_t K, int64_t ldx, const int32_t* qweight,
                         const void* scale16, const void* zp16, const void* bias, int64_t N, int bits, int group,
                         void* y, int64_t ldy, void* stream) {
     if (!x || !qweight || !scale16 || !zp16 || !y) return BW_EINVAL;
     if (!bw_shape_ok(N, K, bits, group) || M < 1 || M > 16 || ldx < K || ldy < N) return BW_EINVAL;
     if (act_dtype != BW_F16 && act_dtype != BW_BF16) return BW_EUNSUPPORTED;
+    g_last_kernel = "";
     if (!bw_fast_shape(M, N, K, ldx, bits, group) || !bw_aligned(x, 16) || (ldx * 2) % 16 || !bw_aligned(qweight, 16))
         return bw_qgemm_generic(x, act_dtype, M, K, ldx, qweight, scale16, zp16, bias, N, bits, group, y, ldy, stream);
     GemvArgs a;

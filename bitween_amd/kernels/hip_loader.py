@@ -20,9 +20,9 @@ BW_F16, BW_BF16, BW_F32, BW_I32, BW_F64 = 0, 1, 2, 3, 4
 BW_SCALE_RECIPROCAL = 0x100   # flag for math_dtype: scale = (max - min) * fl32(1 / Qmax), as eager torch computes it on a GPU
 _DTYPE_CODE = {torch.float16: BW_F16, torch.bfloat16: BW_BF16, torch.float32: BW_F32, torch.int32: BW_I32, torch.float64: BW_F64}
 
-ABI_VERSION = 7            # what bw_abi_version() of a matching library returns
+ABI_VERSION = 8            # what bw_abi_version() of a matching library returns
 ENTRY_POINTS = ("bw_abi_version", "bw_strerror", "bw_quantize_pack", "bw_quantize_pack_add", "bw_dequantize", "bw_qgemv", "bw_qgemm",
-                "bw_qgemm_ws", "bw_qgemm_static", "bw_qgemm_workspace_bytes", "bw_qlinear", "bw_qdgrad", "bw_qdgrad_workspace_bytes", "bw_cast_bf16_f16", "bw_qlinear_decode_rows")
+                "bw_qgemm_ws", "bw_qgemm_static", "bw_qgemm_workspace_bytes", "bw_qlinear", "bw_qdgrad", "bw_qdgrad_workspace_bytes", "bw_cast_bf16_f16", "bw_qlinear_decode_rows", "bw_qgemv_last_kernel")
 
 
 class BitweenHipError(RuntimeError):
@@ -67,6 +67,8 @@ def load():
     lib.bw_cast_bf16_f16.restype = i32
     lib.bw_qlinear_decode_rows.argtypes = [i64, i64, i32]
     lib.bw_qlinear_decode_rows.restype = i32
+    lib.bw_qgemv_last_kernel.argtypes = []
+    lib.bw_qgemv_last_kernel.restype = ctypes.c_char_p
     for name in ("bw_quantize_pack", "bw_quantize_pack_add", "bw_dequantize", "bw_qgemv", "bw_qgemm", "bw_qgemm_ws", "bw_qgemm_static", "bw_qlinear"):
         getattr(lib, name).restype = i32
     for name in ("bw_qgemv", "bw_qgemm", "bw_qlinear"):
@@ -336,6 +338,11 @@ def quantized_input_grad(grad_y, qweight, scale, zero_point, bits, group_size):
         return None
     _check(st, "bw_qdgrad")
     return grad_x
+
+
+def last_decode_kernel():
+    """Name of the decode kernel this thread's last bw_qgemv / bw_qlinear launch ran (a diagnostic for benchmarks)."""
+    return load().bw_qgemv_last_kernel().decode()
 
 
 def quantized_matmul_hip(x, qweight, scale, zero_point, bias, bits, group_size):

@@ -149,6 +149,11 @@ int bw_qgemm_static(const void* x, int act_dtype, int64_t M, int64_t K, int64_t 
 
 int bw_qlinear_decode_rows(int64_t N, int64_t K, int bits);
 
+/* Diagnostic, no counterpart in the reference: the name (with template arguments) of the decode kernel that the
+ * calling thread's last bw_qgemv / bw_qlinear launch ran ("" before the first one, or when the generic kernel ran).
+ * For benchmarks that label a timing with the kernel it belongs to; the string lives as long as the library. */
+const char* bw_qgemv_last_kernel(void);
+
 int bw_qlinear(const void* x, int act_dtype, int64_t M, int64_t K, int64_t ldx,
                const int32_t* qweight, const void* scale16, const void* zp16, const void* bias,
                int64_t N, int bits, int group, void* y, int64_t ldy, void* stream);

@@ -167,3 +167,57 @@ def test_decoder_step_under_graph_capture_equals_the_eager_step():
     logits_twin = twin.step()
     rel = (logits_eager.float() - logits_twin.float()).abs().max() / logits_twin.float().abs().max()
     assert rel < 2e-2
+
+
+def test_full_size_decoder_layer_with_the_mixed_recipe_against_the_oracle():
+    """The end-to-end configuration at its real widths: one decoder layer of bench_decoder.Decoder with hidden 4096,
+    32 heads, MLP 11008, vocab 32000 and the mixed recipe (attention 8-bit g128, gate / up 4-bit g128, down_proj 2-bit
+    g32), quantised by Bitween(...).quantize.  Every quantised linear is checked against the oracle on sampled rows
+    (packed words, float16 scales and zero points, W16 bit for bit); the logits of the first decode step - one launch
+    per module, then with q/k/v and gate/up sharing launches - are compared with a float16 twin that holds W16."""
+    import bench_decoder as bd
+    import bitween_amd
+    from bitween_amd import Bitween, QuantizedLinear
+    from bitween_amd.kernels import hip_loader as hip
+    with torch.device("cuda"):
+        model = bd.Decoder(layers=1, hidden=4096, heads=32, inter=11008, vocab=32000, max_len=64).half()
+    model.init_weights(seed=5)
+    recipe = {"layers.0.self_attn": (8, 128), "layers.0.mlp": (4, 128), "layers.0.mlp.down_proj": (2, 32)}
+    originals = {name: m.weight.data for name, m in model.named_modules() if isinstance(m, torch.nn.Linear)}
+    q = Bitween(model, bits=4, group_size=128).quantize(rtn=True, ignore_layers=["lm_head", "embed_tokens"],
+                                                        layer_config=recipe, verbose=False)
+    qlin = {name: m for name, m in q.named_modules() if isinstance(m, QuantizedLinear)}
+    assert sorted((m.bits, m.group_size) for m in qlin.values()) == [(2, 32)] + [(4, 128)] * 2 + [(8, 128)] * 4
+    twin = copy.deepcopy(q)
+    for name, m in qlin.items():
+        w16 = hip.dequantize(m.qweight, m.scale, m.zero_point, m.group_size, m.bits, torch.float16)
+        rows = np.unique(np.concatenate([np.arange(0, m.out_features, m.out_features // 16), [m.out_features - 1]]))
+        w_rows = originals[name][rows].float().cpu().numpy()
+        qw_o, s_o, z_o, _ = orc.quantize_rtn(w_rows, m.bits, m.group_size)
+        s16, z16 = orc.store_module_buffers(s_o, z_o)
+        assert np.array_equal(m.qweight[rows].cpu().numpy(), qw_o), name
+        assert np.array_equal(m.scale[rows].cpu().numpy().view(np.uint16), s16.view(np.uint16)), name
+        assert np.array_equal(m.zero_point[rows].cpu().numpy(), z16), name
+        w16_o = orc.dequantize_f16(qw_o, s16, z16, m.group_size, m.bits)
+        assert np.array_equal(w16[rows].cpu().numpy().view(np.uint16), w16_o.view(np.uint16)), name
+        lin = torch.nn.Linear(m.in_features, m.out_features, bias=False, device="cuda", dtype=torch.float16)
+        lin.weight.data = w16
+        parent = twin
+        *path, leaf = name.split(".")
+        for part in path:
+            parent = getattr(parent, part)
+        setattr(parent, leaf, lin)
+    ids = torch.randint(0, 32000, (24,), device="cuda", generator=torch.Generator(device="cuda").manual_seed(2))
+    twin.alloc_state()
+    twin.prefill(ids)
+    want = twin.step().float()
+    q.alloc_state()
+    q.prefill(ids)
+    got = q.step().float()
+    assert (got - want).abs().max().item() <= 2e-2 * want.abs().max().item()
+    assert bitween_amd.fuse_sibling_linears(q) == 2
+    q.prefill(ids)
+    fused = q.step().float()
+    assert (fused - want).abs().max().item() <= 2e-2 * want.abs().max().item()
+    # the fused launches run the same arithmetic over concatenated rows (another split of K over waves at most)
+    assert (fused - got).abs().max().item() <= 2e-3 * want.abs().max().item()
