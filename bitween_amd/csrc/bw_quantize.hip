@@ -83,11 +83,16 @@ BW_DEV float quant_exact(float w, float s, float zf) {
 // the shape allows); the lpg = group / VPT threads of a group (a power of two <= 64, aligned inside the
 // wave) agree on min and max with cross-lane shuffles.
 //
-// float32 math takes a short cut that cannot change a result: with r = 1/s refined once (relative error
-// <= 2^-23) t = fma(w, r, zf) differs from the reference's fl(fl(w / s) + zf) by less than 3.5e-4 as long as
-// |w / s| < 1024 (1024 * 2^-23 for r, plus the roundings of the quotient and of the two sums near 1300).  Unless t
-// lies within 2^-11 = 4.9e-4 of a half-integer, round(t) is therefore the reference's value; beyond 1024 both clamp
-// to the same end of the range.  Values near a tie (and infinities, NaN) are redone with the true IEEE divide.
+// float32 math takes a short cut that cannot change a result.  With x = w / s, r = 1/s refined once (relative
+// error <= 2^-23), F = fma(w, r, zf) and the reference's A = fl(fl(x) + zf):
+//     |F - (x + zf)| <= |x| 2^-23 + |F| 2^-24,      |A - (x + zf)| <= |x| 2^-24 + |A| 2^-24,
+// so |F - A| <= 2^-23 (1.5 |x| + max(|F|, |A|)) <= 2.5 * 2^-23 * B with B = max|x| of the group + Qmax + 3 (an upper
+// bound of |x|, |F| and |A|, with room for the rounding of B itself).  Unless F lies within 2^-21 B (> 2.5 * 2^-23 B)
+// of a half-integer, round(F) is therefore the reference's value.  B is formed once per group from its extrema: a
+// group of 4-bit weights that straddles zero has B ~ 20, a window of 1e-5 around the ties instead of a fixed one
+// sized for the worst case - the exact path, which a wave enters when any of its lanes needs it, was what a third
+// of the kernel's arithmetic went into.  Values inside the window (and infinities, NaN, groups so lopsided that the
+// window exceeds 1/2) are redone with the true IEEE divide.
 template <int BITS, int WDT, int MATH, int WPT>
 __global__ __launch_bounds__(256) void quantize_pack_kernel(const void* __restrict__ w, const void* __restrict__ delta,
                                                             int64_t N, int K, int64_t ldw, int64_t ldd,
@@ -125,13 +130,14 @@ __global__ __launch_bounds__(256) void quantize_pack_kernel(const void* __restri
         if constexpr (MATH == BW_F32) {
             const float r0 = __builtin_amdgcn_rcpf(s);
             const float r = __builtin_fmaf(__builtin_fmaf(-s, r0, 1.0f), r0, r0);
+            const float bound = __builtin_fmaf(fmaxf(fabsf(lo), fabsf(hi)), r, QMAX + 3.0f);
+            const float safe = __builtin_fmaf(-0x1p-21f, bound, 0.5f);   // NaN extrema: every comparison below fails
 #pragma unroll
             for (int i = 0; i < VPT; i++) {
                 const float sum = __builtin_fmaf(v[i], r, zf);
                 t[i] = rintf(sum);
-                // far from a tie (a huge |sum| has no fraction and clamps the same either way; NaN fails the test)?
-                // else redo with the true divide: one value in a thousand, so a wave rarely enters any one of these
-                if (!(fabsf(__fsub_rn(sum, t[i])) < 0.5f - 0x1p-11f)) t[i] = quant_exact<MATH>(v[i], s, zf);
+                // far enough from a tie?  (an infinite sum gives NaN here and fails the test.)  Else redo with the true divide.
+                if (!(fabsf(__fsub_rn(sum, t[i])) < safe)) t[i] = quant_exact<MATH>(v[i], s, zf);
             }
         } else {
 #pragma unroll
@@ -150,7 +156,10 @@ __global__ __launch_bounds__(256) void quantize_pack_kernel(const void* __restri
         }
         if (live) {
             uint32_t* dst = reinterpret_cast<uint32_t*>(qweight) + (row * tpr + tcol) * WPT;
-            if constexpr (WPT == 4) *reinterpret_cast<u4*>(dst) = u4{word[0], word[1], word[2], word[3]};
+            if constexpr (WPT == 8) {
+                reinterpret_cast<u4*>(dst)[0] = u4{word[0], word[1], word[2], word[3]};
+                reinterpret_cast<u4*>(dst)[1] = u4{word[4], word[5], word[6], word[7]};
+            } else if constexpr (WPT == 4) *reinterpret_cast<u4*>(dst) = u4{word[0], word[1], word[2], word[3]};
             else if constexpr (WPT == 2) *reinterpret_cast<u2*>(dst) = u2{word[0], word[1]};
             else dst[0] = word[0];
             const int k = tcol * VPT;
@@ -430,9 +439,17 @@ int launch_quantize(const void* w, const void* delta, int64_t N, int64_t K, int6
 template <int BITS, int WDT, int MATH>
 int launch_quantize_bits(const void* w, const void* delta, int64_t N, int64_t K, int64_t ldw, int64_t ldd, int group,
                          int32_t* qweight, void* scale, int sdt, void* zp, int zdt, int recip, hipStream_t st) {
-    // 32 bytes of input per thread where the shape allows, else one word per thread, else the generic kernel
+    // 64 bytes of 16-bit input per thread (32 weights) where the shape allows - everything a thread does once per
+    // group share (extrema exchange, the two divisions of the group's parameters, addressing, the stores) then costs
+    // half as much per weight as with 32 bytes, and the kernel is bound by arithmetic, not memory: 28.6 -> see the
+    // benchmark - else 32 bytes, else one word per thread, else the generic kernel
     constexpr int VPI = 32 / BITS;
     constexpr int WIDE = (WDT == BW_F32 ? 8 : 16) / VPI;
+    if constexpr (WDT != BW_F32) {
+        constexpr int WIDER = 32 / VPI;
+        if (quantize_fits<BITS, WDT, WIDER>(w, delta, K, ldw, ldd, group, qweight))
+            return launch_quantize<BITS, WDT, MATH, WIDER>(w, delta, N, K, ldw, ldd, group, qweight, scale, sdt, zp, zdt, recip, st);
+    }
     if constexpr (WIDE > 1) {
         if (quantize_fits<BITS, WDT, WIDE>(w, delta, K, ldw, ldd, group, qweight))
             return launch_quantize<BITS, WDT, MATH, WIDE>(w, delta, N, K, ldw, ldd, group, qweight, scale, sdt, zp, zdt, recip, st);
