@@ -670,6 +670,12 @@ def extras_backward(torch, hip, QuantizedLinear, layers):
         out["4096x14336_M%d" % m] = {"fused_dgrad_us": round(t_fused, 1), "fused_TFLOPs": round(2.0 * m * n * k / t_fused / 1e6, 1),
                                      "dequantize_plus_gemm_us": round(t_ours, 1), "dequantize_us": round(t_deq, 1),
                                      "fp16_gemm_us": round(t_gemm, 1)}
+        # bfloat16 gradients: the same kernel with the weight rounded to bfloat16 in registers, against the
+        # dequantise-to-bfloat16 + library GEMM path of the module's unfused backward
+        gb = go.to(torch.bfloat16)
+        t_fused_b = time_calls(torch, lambda: hip.quantized_input_grad(gb, q.qweight, q.scale, q.zero_point, 4, 128), 30, 5)
+        t_ours_b = time_calls(torch, lambda: gb @ hip.dequantize(q.qweight, q.scale, q.zero_point, 128, 4, torch.bfloat16), 30, 5)
+        out["4096x14336_M%d" % m].update({"bf16_fused_dgrad_us": round(t_fused_b, 1), "bf16_dequantize_plus_gemm_us": round(t_ours_b, 1)})
     return out
 
 

@@ -1,9 +1,11 @@
 // bw_qdgrad.hip - input gradient of the quantised linear layer, fused with the dequantisation:
 //
-//     grad_x[M][K] = grad_y[M][N] @ W16[N][K],      W16 = fp16(scale * (q - zp))
+//     grad_x[M][K] = grad_y[M][N] @ W16[N][K],      W16 = fp16(scale * (q - zp))   (or bfloat16 for bfloat16 gradients)
 //
 // (QuantizedLinearFunction.backward, bitween/modules.py:108-141: it unpacks, forms W32 = scale * (q - zp),
-// casts to grad_output's dtype and calls matmul; for float16 gradients that cast gives exactly W16.)
+// casts to grad_output's dtype and calls matmul; for float16 gradients that cast gives exactly W16, for bfloat16
+// gradients the float32 product - exact: an 11-bit scale times an integer below 256 - rounded to nearest even, which
+// is what the kernel forms with the hardware's packed float32 -> bfloat16 conversion before a bfloat16 MFMA.)
 //
 // The reduction runs over N, the dimension the packed words do NOT run along, so a weight tile has to be
 // transposed on its way to the matrix core.  A workgroup owns a 128 or 256 (m) x 128 (k) tile of grad_x and walks
@@ -59,18 +61,36 @@ template <> struct WLoad<4> { typedef u2 type; };
 template <> struct WLoad<8> { typedef u4 type; };
 template <> struct WLoad<2> { typedef uint32_t type; };
 
-// 16 values of one row -> 8 float16 pairs; pair p, half h is element kmap(p, h) of the 16
-template <int BITS>
+// 16 values of one row -> 8 float16 pairs; pair p, half h is element kmap(p, h) of the 16.  SCALE = false: the
+// exact integers q - z (the caller multiplies by the scale in float32).
+template <int BITS, bool SCALE>
 BW_DEV void dequant16(const typename WLoad<BITS>::type& w, const GroupConst<BITS>& gc, h2* out) {
     if constexpr (BITS == 4) {
-        dequant_word4<true>(w[0], gc, out);
-        dequant_word4<true>(w[1], gc, out + 4);
+        dequant_word4<SCALE>(w[0], gc, out);
+        dequant_word4<SCALE>(w[1], gc, out + 4);
     } else if constexpr (BITS == 8) {
 #pragma unroll
-        for (int j = 0; j < 4; j++) dequant_word8<true>(w[j], gc, out + 2 * j);
+        for (int j = 0; j < 4; j++) dequant_word8<SCALE>(w[j], gc, out + 2 * j);
     } else {
-        dequant_word2<true>(w, gc, out);
+        dequant_word2<SCALE>(w, gc, out);
     }
+}
+
+typedef __bf16 bf2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf8 __attribute__((ext_vector_type(8)));
+typedef float f2 __attribute__((ext_vector_type(2)));
+
+// two float32 -> two 16-bit values of the gradient's type, round to nearest even, as one dword
+template <int DT>
+BW_DEV uint32_t pack2(float a, float b) {
+    if constexpr (DT == BW_F16) return as_u32(h2{(_Float16)a, (_Float16)b});
+    else return __builtin_bit_cast(uint32_t, __builtin_convertvector(f2{a, b}, bf2));
+}
+
+template <int DT>
+BW_DEV f4 mfma16(const h8& a, const h8& b, const f4& c) {
+    if constexpr (DT == BW_F16) return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+    else return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf8, a), __builtin_bit_cast(bf8, b), c, 0, 0, 0);
 }
 template <int BITS>
 BW_DEV constexpr int kmap(int p, int h) {
@@ -79,7 +99,7 @@ BW_DEV constexpr int kmap(int p, int h) {
     else return p + 8 * h;
 }
 
-template <int BITS, int GROUP, int MT>
+template <int BITS, int GROUP, int MT, int DT>
 __global__ __launch_bounds__(DTHREADS, MT == 4 ? 3 : 2) void qdgrad_kernel(const DgradArgs a) {   // workgroups per CU: 3 (<= 168 registers) or 2
     constexpr int DM = DgradTile<MT>::DM, A_BYTES = DgradTile<MT>::A_BYTES, STAGE = DgradTile<MT>::STAGE;
     constexpr int GR = DM / 128;                                      // grad_y rows a thread stages
@@ -145,10 +165,20 @@ __global__ __launch_bounds__(DTHREADS, MT == 4 ? 3 : 2) void qdgrad_kernel(const
         GroupConst<BITS> gc;
         gc.set(live ? sreg[slot] : (_Float16)0.f, zreg[slot]);        // past the slice's end: weights of zero
         h2 w16[8];
-        dequant16<BITS>(wreg[slot], gc, w16);
+        uint32_t wd[8];                                               // the 8 pairs in the gradient's type
+        if constexpr (DT == BW_F16) {
+            dequant16<BITS, true>(wreg[slot], gc, w16);
+#pragma unroll
+            for (int i = 0; i < 8; i++) wd[i] = as_u32(w16[i]);
+        } else {
+            dequant16<BITS, false>(wreg[slot], gc, w16);              // exact q - z; the product with the scale is exact in float32
+            const float sf = (float)gc.s[0];
+#pragma unroll
+            for (int i = 0; i < 8; i++) wd[i] = pack2<DT>(__fmul_rn((float)w16[i][0], sf), __fmul_rn((float)w16[i][1], sf));
+        }
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-            const uint32_t lo4 = as_u32(w16[i]), hi4 = as_u32(w16[4 + i]);
+            const uint32_t lo4 = wd[i], hi4 = wd[4 + i];
             const uint32_t keep = odd ? hi4 : lo4, recv = dpp_xor8(odd ? lo4 : hi4);
             *reinterpret_cast<uint32_t*>(Bs + b_dst + kmap<BITS>(i, 0) * DPITCH) = __builtin_amdgcn_perm(recv, keep, sel_lo);
             *reinterpret_cast<uint32_t*>(Bs + b_dst + kmap<BITS>(i, 1) * DPITCH) = __builtin_amdgcn_perm(recv, keep, sel_hi);
@@ -190,7 +220,7 @@ __global__ __launch_bounds__(DTHREADS, MT == 4 ? 3 : 2) void qdgrad_kernel(const
             for (int j = 0; j < MT; j++)
 #pragma unroll
                 for (int i = 0; i < 4; i++)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[i], bf[j], acc[i][j], 0, 0, 0);
+                    acc[i][j] = mfma16<DT>(af[i], bf[j], acc[i][j]);
             __syncthreads();
         }
     }
@@ -212,14 +242,14 @@ __global__ __launch_bounds__(DTHREADS, MT == 4 ? 3 : 2) void qdgrad_kernel(const
             for (int i = 0; i < 4; i++) {
                 const f4 v = acc[i][j];
                 _Float16* dst = a.gx + (int64_t)m * a.ldx + k0 + wk + 16 * i + 4 * q;
-                *reinterpret_cast<u2*>(dst) = u2{as_u32(h2{(_Float16)v[0], (_Float16)v[1]}), as_u32(h2{(_Float16)v[2], (_Float16)v[3]})};
+                *reinterpret_cast<u2*>(dst) = u2{pack2<DT>(v[0], v[1]), pack2<DT>(v[2], v[3])};
             }
         }
     }
 }
 
 // grad_x tile = sum of its slices' partial tiles, rounded once
-template <int DM>
+template <int DM, int DT>
 __global__ __launch_bounds__(256) void qdgrad_reduce_kernel(const DgradArgs a) {
     const int tile = blockIdx.y;
     const int quad = (int)(blockIdx.x * blockDim.x + threadIdx.x);    // < DM * DK / 4
@@ -233,8 +263,7 @@ __global__ __launch_bounds__(256) void qdgrad_reduce_kernel(const DgradArgs a) {
 #pragma unroll
         for (int i = 0; i < 4; i++) v[i] += t[i];
     }
-    *reinterpret_cast<u2*>(a.gx + (int64_t)m * a.ldx + k) =
-        u2{as_u32(h2{(_Float16)v[0], (_Float16)v[1]}), as_u32(h2{(_Float16)v[2], (_Float16)v[3]})};
+    *reinterpret_cast<u2*>(a.gx + (int64_t)m * a.ldx + k) = u2{pack2<DT>(v[0], v[1]), pack2<DT>(v[2], v[3])};
 }
 
 struct DgradPlan {
@@ -288,22 +317,22 @@ inline bool dgrad_fast_shape(int64_t M, int64_t N, int64_t K, int64_t ldg, int64
            M >= 1 && M < ((int64_t)1 << 24) && N * (K * bits / 8) < ((int64_t)1 << 40);
 }
 
-template <int BITS, int GROUP, int MT>
+template <int BITS, int GROUP, int MT, int DT>
 int launch_dgrad_mt(const DgradArgs& a, const DgradPlan& p, hipStream_t stream) {
     constexpr int DM = DgradTile<MT>::DM;
-    auto kern = qdgrad_kernel<BITS, GROUP, MT>;
+    auto kern = qdgrad_kernel<BITS, GROUP, MT, DT>;
     static uint64_t big_lds_devices = 0;                   // per instantiation
     if (2 * DgradTile<MT>::STAGE > 64 * 1024 && !bw_allow_big_lds(reinterpret_cast<const void*>(kern), big_lds_devices)) return BW_ELAUNCH;
     hipLaunchKernelGGL(kern, dim3((unsigned)(p.tiles * p.splits)), dim3(DTHREADS), 2 * DgradTile<MT>::STAGE, stream, a);
     if (hipGetLastError() != hipSuccess) return BW_ELAUNCH;
     if (p.splits > 1) {
-        hipLaunchKernelGGL(qdgrad_reduce_kernel<DM>, dim3(DM * DK / 4 / 256, (unsigned)p.tiles), dim3(256), 0, stream, a);
+        hipLaunchKernelGGL((qdgrad_reduce_kernel<DM, DT>), dim3(DM * DK / 4 / 256, (unsigned)p.tiles), dim3(256), 0, stream, a);
         if (hipGetLastError() != hipSuccess) return BW_ELAUNCH;
     }
     return BW_OK;
 }
 
-template <int BITS, int GROUP>
+template <int BITS, int GROUP, int DT>
 int launch_dgrad(DgradArgs a, void* workspace, size_t workspace_bytes, hipStream_t stream) {
     const DgradPlan p = dgrad_plan(a.M, a.N, a.K, workspace != nullptr);
     if (p.ws_bytes > workspace_bytes) return BW_EWORKSPACE;
@@ -311,7 +340,7 @@ int launch_dgrad(DgradArgs a, void* workspace, size_t workspace_bytes, hipStream
     a.tiles_k = p.tiles_k;
     a.splits = p.splits;
     a.steps_per_split = p.steps_per_split;
-    return p.mt == 8 ? launch_dgrad_mt<BITS, GROUP, 8>(a, p, stream) : launch_dgrad_mt<BITS, GROUP, 4>(a, p, stream);
+    return p.mt == 8 ? launch_dgrad_mt<BITS, GROUP, 8, DT>(a, p, stream) : launch_dgrad_mt<BITS, GROUP, 4, DT>(a, p, stream);
 }
 
 }  // namespace
@@ -326,7 +355,7 @@ extern "C" int bw_qdgrad(const void* grad_y, int act_dtype, int64_t M, int64_t N
                          int64_t ldx, void* workspace, size_t workspace_bytes, void* stream) {
     if (!grad_y || !qweight || !scale16 || !zp16 || !grad_x) return BW_EINVAL;
     if (!bw_shape_ok(N, K, bits, group) || M < 1 || ldg < N || ldx < K) return BW_EINVAL;
-    if (act_dtype != BW_F16) return BW_EUNSUPPORTED;
+    if (act_dtype != BW_F16 && act_dtype != BW_BF16) return BW_EUNSUPPORTED;
     if (!dgrad_fast_shape(M, N, K, ldg, ldx, bits, group)) return BW_EUNSUPPORTED;
     if (!bw_aligned(grad_y, 16) || !bw_aligned(grad_x, 8) || !bw_aligned(qweight, 16)) return BW_EALIGN;
     if (workspace && !bw_aligned(workspace, 16)) return BW_EALIGN;
@@ -336,8 +365,10 @@ extern "C" int bw_qdgrad(const void* grad_y, int act_dtype, int64_t M, int64_t N
     a.M = (int)M; a.N = (int)N; a.K = (int)K; a.ldg = (int)ldg; a.ldx = (int)ldx;
     a.groups = (int)(K / group); a.row_bytes = (int)(K * bits / 8);
     hipStream_t st = (hipStream_t)stream;
-#define BW_CASE(B, G) \
-    if (bits == B && group == G) return launch_dgrad<B, G>(a, workspace, workspace_bytes, st);
+#define BW_CASE(B, G)                                                                                                    \
+    if (bits == B && group == G)                                                                                         \
+        return act_dtype == BW_F16 ? launch_dgrad<B, G, BW_F16>(a, workspace, workspace_bytes, st)                       \
+                                   : launch_dgrad<B, G, BW_BF16>(a, workspace, workspace_bytes, st);
     BW_CASE(4, 128) BW_CASE(4, 64) BW_CASE(4, 32)
     BW_CASE(8, 128) BW_CASE(8, 64) BW_CASE(8, 32)
     BW_CASE(2, 128) BW_CASE(2, 64) BW_CASE(2, 32)

@@ -309,9 +309,10 @@ def decode_with_plan(plan, x, m):
 
 
 def quantized_input_grad(grad_y, qweight, scale, zero_point, bits, group_size):
-    """grad_x[M,K] = grad_y[M,N] @ W16[N,K] with the dequantisation fused in (bw_qdgrad); None when the library
-    has no fused kernel for this shape / dtype - the caller then dequantises and calls the library GEMM."""
-    if grad_y.dtype is not torch.float16 or not grad_y.is_cuda or grad_y.dim() != 2:
+    """grad_x[M,K] = grad_y[M,N] @ W[N,K] with the dequantisation fused in (bw_qdgrad), W being the dequantised weight
+    in grad_y's dtype (float16 or bfloat16); None when the library has no fused kernel for this shape / dtype - the
+    caller then dequantises and calls the library GEMM."""
+    if grad_y.dtype not in (torch.float16, torch.bfloat16) or not grad_y.is_cuda or grad_y.dim() != 2:
         return None
     if qweight.dtype is not torch.int32 or scale.dtype is not torch.float16 or zero_point.dtype is not torch.float16:
         return None
@@ -327,11 +328,11 @@ def quantized_input_grad(grad_y, qweight, scale, zero_point, bits, group_size):
             return None
     qweight, scale, zero_point = qweight.contiguous(), scale.contiguous(), zero_point.contiguous()
     lib = load()
-    grad_x = torch.empty((m, k), dtype=torch.float16, device=grad_y.device)
+    grad_x = torch.empty((m, k), dtype=grad_y.dtype, device=grad_y.device)
     with _on_device(grad_y.device) as index:
         nbytes = lib.bw_qdgrad_workspace_bytes(m, n, k, bits, group_size)
         ws = torch.empty(nbytes, dtype=torch.uint8, device=grad_y.device) if nbytes else None
-        st = lib.bw_qdgrad(grad_y.data_ptr(), BW_F16, m, n, grad_y.stride(0), qweight.data_ptr(), scale.data_ptr(),
+        st = lib.bw_qdgrad(grad_y.data_ptr(), _DTYPE_CODE[grad_y.dtype], m, n, grad_y.stride(0), qweight.data_ptr(), scale.data_ptr(),
                            zero_point.data_ptr(), k, bits, group_size, grad_x.data_ptr(), k,
                            None if ws is None else ws.data_ptr(), nbytes, _raw_stream(index))
     if st in (-2, -3):                                     # BW_EUNSUPPORTED / BW_EALIGN: the caller's unfused path

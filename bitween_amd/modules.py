@@ -37,11 +37,11 @@ class QuantizedLinearFunction(torch.autograd.Function):
         x, qweight, scale, zero_point, bias = ctx.saved_tensors
         grad_input = None
         if ctx.needs_input_grad[0]:
-            # float16 gradients, up to FUSED_DGRAD_MAX_ROWS rows: one fused kernel, the weights are never
+            # float16 / bfloat16 gradients, up to FUSED_DGRAD_MAX_ROWS rows: one fused kernel, the weights are never
             # materialised.  Beyond that the library GEMM on dequantised weights is faster (the fused kernel
             # re-dequantises the weights for every 128 rows of grad_output).
             go2 = grad_output.reshape(-1, grad_output.shape[-1])
-            if grad_output.dtype is torch.float16 and grad_output.is_cuda and go2.shape[0] <= FUSED_DGRAD_MAX_ROWS:
+            if grad_output.dtype in (torch.float16, torch.bfloat16) and grad_output.is_cuda and go2.shape[0] <= FUSED_DGRAD_MAX_ROWS:
                 gx = _hip.quantized_input_grad(go2, qweight, scale, zero_point, ctx.bits, ctx.group_size)
                 if gx is not None:
                     return gx.view(*grad_output.shape[:-1], gx.shape[-1]), None, None, None, None, None, None

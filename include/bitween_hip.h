@@ -168,8 +168,9 @@ int bw_cast_bf16_f16(const void* x, int64_t rows, int64_t cols, int64_t ldx, voi
 /* Input gradient, fused with the dequantisation:  grad_x[M][K] = grad_y[M][N] @ W16[N][K]
  * replaces QuantizedLinearFunction.backward (bitween/modules.py:108-141), which unpacks the weights, forms
  * scale * (q - zp), casts it to grad_output's dtype and calls matmul; for float16 gradients that cast gives the
- * same W16 as the forward.  Products accumulate in float32, grad_x is rounded once.
- *   grad_y [M][ldg], grad_x [M][ldx] of act_dtype (BW_F16 only)
+ * same W16 as the forward, for bfloat16 gradients it is the float32 product rounded once to bfloat16 (computed in the
+ * kernel from the exact q - zp and the float16 scale).  Products accumulate in float32, grad_x is rounded once.
+ *   grad_y [M][ldg], grad_x [M][ldx] of act_dtype (BW_F16 or BW_BF16)
  * Built for K % 128 == 0, N % 32 == 0, group 32 | 64 | 128, ldg % 8 == 0, ldx % 4 == 0; other shapes and dtypes
  * return BW_EUNSUPPORTED (the Python backward then dequantises with bw_dequantize and calls the library GEMM).
  * When M * K is small the reduction over N is cut into slices whose float32 partial sums go through a

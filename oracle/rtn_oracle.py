@@ -214,10 +214,20 @@ def qlinear_forward(x16, qweight, scale16, zp16, bias16, bits, group_size):
     return y, y64
 
 
-def qlinear_backward(grad_out, qweight, scale16, zp16, bits, group_size):
+def qlinear_backward(grad_out, qweight, scale16, zp16, bits, group_size, dtype="f16"):
     """bitween/modules.py:108-141: grad_input = grad_output @ W, W being the
-    float32 dequantized weight cast to grad_output's dtype (float16 here).
+    float32 dequantized weight cast to grad_output's dtype: float16 (default)
+    or bfloat16 (`grad_out` is then a float32 array holding bfloat16 values).
     Float64 accumulate, tolerance as for the forward."""
     w32 = dequantize_rtn_f32(qweight, scale16, zp16, group_size, bits)
-    w = w32.astype(np.float16).astype(np.float64)
-    return np.asarray(grad_out, np.float16).astype(np.float64) @ w
+    if dtype == "f16":
+        w = w32.astype(np.float16).astype(np.float64)
+        go = np.asarray(grad_out, np.float16).astype(np.float64)
+    elif dtype == "bf16":
+        w = _round_to(w32, "bf16").astype(np.float64)
+        go = np.asarray(grad_out, np.float32)
+        assert np.array_equal(go, _round_to(go, "bf16")), "grad_out must hold bfloat16 values"
+        go = go.astype(np.float64)
+    else:
+        raise ValueError("dtype must be 'f16' or 'bf16'")
+    return go @ w

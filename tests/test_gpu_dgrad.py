@@ -107,8 +107,8 @@ def test_dgrad_refusals_and_padding():
     st = lib.bw_qdgrad(go.data_ptr(), 0, 5, n, n, d[0].data_ptr(), d[1].data_ptr(), d[2].data_ptr(), k, bits, g,
                        gx.data_ptr(), k, None, 0, None)
     assert st == 0
-    assert lib.bw_qdgrad(go.data_ptr(), 1, 5, n, n, d[0].data_ptr(), d[1].data_ptr(), d[2].data_ptr(), k, bits, g,
-                         gx.data_ptr(), k, None, 0, None) == -2          # bfloat16: BW_EUNSUPPORTED
+    assert lib.bw_qdgrad(go.data_ptr(), 2, 5, n, n, d[0].data_ptr(), d[1].data_ptr(), d[2].data_ptr(), k, bits, g,
+                         gx.data_ptr(), k, None, 0, None) == -2          # float32 gradients: BW_EUNSUPPORTED
     assert lib.bw_qdgrad(go.data_ptr(), 0, 5, n, n, d[0].data_ptr(), d[1].data_ptr(), d[2].data_ptr(), k, 3, g,
                          gx.data_ptr(), k, None, 0, None) == -1          # BW_EINVAL
     assert lib.bw_qdgrad(None, 0, 5, n, n, d[0].data_ptr(), d[1].data_ptr(), d[2].data_ptr(), k, bits, g,
@@ -167,3 +167,67 @@ def test_dgrad_seeded_sweep(case):
         st, gx, _ = _call(lib, buf, d, m, n, k, bits, g, use_ws, ldg=n + pad)
         assert st == 0
         _check(gx, go16, qw, s16, z16, bits, g)
+
+
+def _bf16_values(a):
+    """float32 array rounded to bfloat16 values (what a bfloat16 tensor holds)."""
+    return torch.from_numpy(np.ascontiguousarray(a, dtype=np.float32)).to(torch.bfloat16)
+
+
+@pytest.mark.parametrize("bits,g", COMBOS)
+def test_dgrad_bfloat16_vs_oracle(bits, g):
+    """bfloat16 gradients: the kernel multiplies with W32.to(bfloat16) (bitween/modules.py:134-139) on the bfloat16
+    matrix core and returns bfloat16.  Against qlinear_backward(dtype="bf16"): one bfloat16 rounding of the result
+    (2^-8 relative) plus float32 accumulation slack; one-hot rows return rows of the bfloat16 weight bit for bit."""
+    from bitween_amd.kernels import hip_loader
+    lib = hip_loader.load()
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    for (n, k) in ((256, 384), (96, 768), (1024, 128)):
+        _, qw, s16, z16, _ = quantized_layer(n, k, bits, g, seed=n + k + bits + g + 1, outliers=True, bias=False)
+        d = [to_gpu(a) for a in (qw, s16, z16)]
+        wbf = orc.dequantize_bf16(qw, s16, z16, g, bits)                 # float32 holding bfloat16 values
+        rng = np.random.default_rng(n + 3 * k)
+        for m in (1, 17, 130, 600):
+            go = _bf16_values(rng.standard_normal((m, n))).cuda()
+            for use_ws in (True, False):
+                need = lib.bw_qdgrad_workspace_bytes(m, n, k, bits, g) if use_ws else 0
+                ws = torch.empty(max(need, 16), dtype=torch.uint8, device="cuda")
+                gx = torch.full((m, k), float("nan"), dtype=torch.bfloat16, device="cuda")
+                st = lib.bw_qdgrad(go.data_ptr(), 1, m, n, n, d[0].data_ptr(), d[1].data_ptr(), d[2].data_ptr(), k, bits, g,
+                                   gx.data_ptr(), k, ws.data_ptr() if need else None, need, stream)
+                torch.cuda.synchronize()
+                assert st == 0
+                go32 = go.float().cpu().numpy()
+                ref = orc.qlinear_backward(go32, qw, s16, z16, bits, g, dtype="bf16")
+                got = gx.double().cpu().numpy()
+                mag = np.abs(go32.astype(np.float64)) @ np.abs(wbf.astype(np.float64))
+                bound = 2.0 ** -8 * np.abs(ref) + 2e-6 * mag + 1e-7
+                assert (np.abs(got - ref) <= bound).all(), float((np.abs(got - ref) / bound).max())
+                assert np.abs(got - ref).max() <= 1e-2 * np.abs(ref).max()
+        # one-hot rows: rows of the bfloat16 weight, bit for bit
+        rows = [0, 1, n // 2 + 1, n - 1]
+        go = torch.zeros((len(rows), n), dtype=torch.bfloat16, device="cuda")
+        for i, r in enumerate(rows):
+            go[i, r] = 1.0
+        gx = torch.empty((len(rows), k), dtype=torch.bfloat16, device="cuda")
+        st = lib.bw_qdgrad(go.data_ptr(), 1, len(rows), n, n, d[0].data_ptr(), d[1].data_ptr(), d[2].data_ptr(), k, bits, g,
+                           gx.data_ptr(), k, None, 0, stream)
+        torch.cuda.synchronize()
+        assert st == 0
+        assert np.array_equal(gx.float().cpu().numpy(), wbf[rows])
+
+
+def test_module_backward_takes_the_fused_kernel_for_bfloat16_gradients():
+    """QuantizedLinearFunction.backward with a bfloat16 grad_output: the fused kernel's result equals the reference's
+    own sequence - dequantise to float32, cast to bfloat16, matmul (bitween/modules.py:125-139) - to bfloat16 rounding."""
+    import bitween_amd
+    torch.manual_seed(4)
+    lin = torch.nn.Linear(512, 384, bias=False, device="cuda", dtype=torch.float16)
+    q = bitween_amd.QuantizedLinear.from_float(lin, 4, 128)
+    go = torch.randn(40, 384, device="cuda", dtype=torch.bfloat16)
+    from bitween_amd.kernels import hip_loader as hip
+    got = hip.quantized_input_grad(go, q.qweight, q.scale, q.zero_point, 4, 128)
+    assert got is not None and got.dtype is torch.bfloat16
+    w = bitween_amd.dequantize_rtn(q.qweight, q.scale, q.zero_point, 128, 4).to(torch.bfloat16)
+    want = go.float() @ w.float()
+    assert (got.float() - want).abs().max().item() <= 2.0 ** -7 * want.abs().max().item()

@@ -317,3 +317,41 @@ def test_f64_oracle_matches_exact_vectors(name):
         assert np.array_equal(qw_t.numpy(), qw) and np.array_equal(s_t.numpy(), scale) and np.array_equal(z_t.numpy(), zp)
         w_t = tcp.dequantize_rtn(qw_t, s_t, z_t, g, bits)
         assert w_t.dtype == torch.float64 and np.array_equal(w_t.numpy().view(np.uint64), w64.view(np.uint64))
+
+
+def test_bfloat16_weights_of_the_backward_match_exact_rational_rounding():
+    """For bfloat16 gradients the reference multiplies with W32.to(bfloat16) (bitween/modules.py:134-139): the float32
+    product scale16 * (q - zp) - exact - rounded once to bfloat16, ties to even.  dequantize_bf16 against that rounding
+    carried out on exact fractions (tests/ieee_exact.py), over every (q, zp) difference and scales that put the product
+    on, just below and just above bfloat16 ties; then qlinear_backward(dtype="bf16") against plain loops."""
+    from fractions import Fraction
+    import ieee_exact as ex
+    rng = np.random.default_rng(21)
+    bits, g = 8, 32
+    n, k = 24, 64
+    q = rng.integers(0, 256, size=(n, k)).astype(np.int32)
+    qw = orc.pack_words(q, bits)
+    # scales: random float16 values, plus values with few significant bits (products that are exact ties in bfloat16)
+    s16 = np.abs(rng.standard_normal((n, k // g)).astype(np.float16) * np.float16(0.01)) + np.float16(1e-4)
+    s16[::3] = np.float16(0.0078125) * (1 + rng.integers(0, 8, size=s16[::3].shape) / 8).astype(np.float16)
+    z16 = rng.integers(0, 256, size=(n, k // g)).astype(np.float16)
+    got = orc.dequantize_bf16(qw, s16, z16, g, bits)
+    for i in range(n):
+        for j in range(k):
+            exact = Fraction(float(s16[i, j // g])) * (int(q[i, j]) - int(z16[i, j // g]))
+            want = ex.rn(exact, "bf16")
+            assert Fraction(float(got[i, j])) == want, (i, j)
+    go = orc._round_to(rng.standard_normal((3, n)).astype(np.float32), "bf16")
+    out = orc.qlinear_backward(go, qw, s16, z16, bits, g, dtype="bf16")
+    want = np.zeros((3, k))
+    for m in range(3):
+        for kk in range(k):
+            acc = 0.0
+            for nn in range(n):
+                acc += float(go[m, nn]) * float(got[nn, kk])
+            want[m, kk] = acc
+    assert np.allclose(out, want, rtol=1e-12, atol=1e-15)
+    eye = np.eye(n, dtype=np.float32)
+    assert np.array_equal(orc.qlinear_backward(eye, qw, s16, z16, bits, g, dtype="bf16"), got.astype(np.float64))
+    with pytest.raises(AssertionError):
+        orc.qlinear_backward(np.full((1, n), 1.001, np.float32), qw, s16, z16, bits, g, dtype="bf16")   # not a bfloat16 value
