@@ -22,10 +22,11 @@ bool bw_fast_shape(int64_t M, int64_t N, int64_t K, int64_t ldx, int bits, int g
 
 namespace {
 
-constexpr int WAVES = 4, NT = 4, MT = 8, BM = MT * 16, BN = WAVES * NT * 16;
+constexpr int WAVES = 4, NT = 4, BN = WAVES * NT * 16;   // a wave owns MT x NT MFMA tiles; MT = 8 or 16 (128 or 256 rows)
 
-template <int BITS, int GROUP>
+template <int BITS, int GROUP, int MT = 8>
 struct GemmCfg {
+    static constexpr int BM = MT * 16;
     // A lane takes WL adjacent 16-byte loads of a weight row per K step: VPL consecutive values.  Two loads
     // at 8 bits, so that every format runs 4 or 8 MFMA steps per K step (the per-step costs - barrier,
     // first fragments, scale and zero-point requests - are spread equally thin) and a lane's values never
@@ -56,6 +57,18 @@ struct GemmCfg {
     static constexpr int UPR = CHUNK_K / UNIT;                   // staging units per x row
     static constexpr int XL = BM * UPR / (WAVES * 64);           // staging units per thread
     static_assert(BM * UPR % (WAVES * 64) == 0, "tile must split evenly over the workgroup");
+    // The staging units of a thread pass through XR register sets in PH phases per K step, each phase in an MFMA
+    // step of its own: phase p writes its units of chunk c+1 to LDS (slots SLOT0[p] .. SLOT0[p] + XR - 1 of MFMA step
+    // STAGE_T[p]) and requests the units of the phase after it into the same registers.  One phase for 128 rows;
+    // two for 256 rows, two MFMA steps apart, so that a request has two steps (2 x 64 MFMAs) to land.
+    static constexpr int XR = XL > 8 ? 8 : XL, PH = XL / XR;
+    static_assert(XL % XR == 0 && PH <= 2, "staging phases");
+    static constexpr int STAGE_T0 = PH == 1 ? T_STAGE : (BITS == 4 ? 1 : 0), STAGE_T1 = PH == 1 ? -1 : (BITS == 4 ? 3 : 2);
+    static constexpr int SLOT0_0 = (PH == 2 && BITS == 4) ? 8 : 0, SLOT0_1 = 0;
+    // Activation fragments in registers: 128 rows - two sets of MT, the set of MFMA step t+1 read during step t;
+    // 256 rows - a ring of XRING, the fragment of slot i + XRING read when slot i has issued its MFMAs (256 cycles of
+    // matrix work ahead of its use).
+    static constexpr int XB = MT == 8 ? 2 : 1, XRING = MT == 8 ? MT : 8;
 };
 
 template <int BITS>
@@ -117,6 +130,7 @@ struct GemmArgs {
     // partial tiles go to ws (one BM x BN block per id) for qgemm_reduce_kernel to add up.
     float* ws;
     int tiles_n, full_tiles, splits, chunks_per_split;
+    int bm;                                        // rows of a tile: 128 or 256
 };
 
 BW_DEV __amdgpu_buffer_rsrc_t make_rsrc(const void* p, uint32_t bytes) {
@@ -129,9 +143,10 @@ BW_DEV __amdgpu_buffer_rsrc_t make_rsrc(const void* p, uint32_t bytes) {
 //   the activations of chunk c+1 were requested one step earlier and are written to buffer (c+1)&1 during
 //   step c, then re-requested for chunk c+2; the weights of chunk c+2 are requested into step c's own set
 //   once its last fragment is unpacked.  Every global load has a full K step (~2000 MFMA cycles) to land.
-template <int BITS, int GROUP, bool WIDE_META>
+template <int BITS, int GROUP, bool WIDE_META, int MT>
 __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
-    using C = GemmCfg<BITS, GROUP>;
+    using C = GemmCfg<BITS, GROUP, MT>;
+    constexpr int BM = C::BM;
     // WIDE_META (rows of scales on 4-byte boundaries): META4 = 8-byte requests over runs of K steps; PAIR = a lane whose
     // values span two groups fetches both scales (zero points) with one 4-byte request instead of two 2-byte ones
     constexpr bool META4 = WIDE_META && C::CAN_META4, PAIR = WIDE_META && !C::CAN_META4 && C::NG == 2;
@@ -159,14 +174,21 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
         w_off[j] = row < a.N ? (uint32_t)row * a.row_bytes + kq * 16 * C::WL : kOob;
         m_off[j] = (uint32_t)min(row, a.N - 1) * groups * 2;
     }
-    uint32_t x_off[C::XL];
+    // Staging unit i of a thread: row tid / UPR + i * RPI of the tile, the thread's UNIT-wide column ku of the chunk.
+    // 128-row tiles keep the byte offsets of their units in registers; 256-row tiles, which have none to spare, form
+    // them from the first (rows past M then lie past the end of x and are range-checked to zero by the hardware; the
+    // launcher checks that (M + 256) * ldx * 2 fits 32 bits).
+    static_assert((WAVES * 64) % C::UPR == 0, "a thread's staging units share one column");
+    constexpr int RPI = WAVES * 64 / C::UPR;
+    const int x_ku = tid % C::UPR;
+    const uint32_t x_base = (uint32_t)((m0 + tid / C::UPR) * a.ldx + x_ku * C::UNIT) * 2, x_pitch = (uint32_t)(RPI * a.ldx) * 2;
+    uint32_t x_off[C::PH == 1 ? C::XL : 1];
+    if constexpr (C::PH == 1) {
 #pragma unroll
-    for (int i = 0; i < C::XL; i++) {
-        const int u = tid + i * WAVES * 64, m = u / C::UPR, ku = u - m * C::UPR;
-        x_off[i] = (m0 + m < a.M) ? (uint32_t)((m0 + m) * a.ldx + ku * C::UNIT) * 2 : kOob;
+        for (int i = 0; i < C::XL; i++) x_off[i] = (m0 + tid / C::UPR + i * RPI < a.M) ? x_base + i * x_pitch : kOob;
     }
 
-    u4 xr[C::XL * C::UW];
+    u4 xr[C::XR * C::UW];
     // Two weight register sets, used alternately by even and odd K steps and never copied: a register move
     // of an outstanding load would stall on it.
     struct WSet { u4 w[NT][C::WL]; uint32_t s[NT][C::NG], z[NT][C::NG]; };   // 16-bit values, one register each
@@ -180,22 +202,24 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
         for (int j = 0; j < NT; j++) acc[i][j] = f4{0.f, 0.f, 0.f, 0.f};
 
     // Pieces of the staging / issue work, one per m-tile index, so they can be slotted between MFMA groups.
-    static_assert(C::XL <= MT && NT * 2 == MT, "at most one staging unit and half a weight tile per m-tile slot");
+    static_assert(C::XR <= MT && MT % (NT * 2) == 0, "at most one staging unit and half a weight tile per m-tile slot");
+    // unit i travels in register set i % XR
     auto stage_unit = [&](int i, _Float16* xs) {
-        const int u = tid + i * WAVES * 64, m = u / C::UPR, ku = u - m * C::UPR;
+        const int m = tid / C::UPR + i * RPI, r = (i % C::XR) * C::UW;
         uint32_t in[4 * C::UW], o[4 * C::UW];
 #pragma unroll
-        for (int j = 0; j < C::UW; j++) { in[4 * j] = xr[i * C::UW + j][0]; in[4 * j + 1] = xr[i * C::UW + j][1]; in[4 * j + 2] = xr[i * C::UW + j][2]; in[4 * j + 3] = xr[i * C::UW + j][3]; }
+        for (int j = 0; j < C::UW; j++) { in[4 * j] = xr[r + j][0]; in[4 * j + 1] = xr[r + j][1]; in[4 * j + 2] = xr[r + j][2]; in[4 * j + 3] = xr[r + j][3]; }
         permute_unit<BITS>(in, o);
-        u4* dst = reinterpret_cast<u4*>(xs + m * C::PITCH + ku * C::UNIT);
+        u4* dst = reinterpret_cast<u4*>(xs + m * C::PITCH + x_ku * C::UNIT);
 #pragma unroll
         for (int j = 0; j < C::UW; j++) dst[j] = u4{o[4 * j], o[4 * j + 1], o[4 * j + 2], o[4 * j + 3]};
     };
     auto issue_x_unit = [&](int i, int c) {
-        const int ku = (tid + i * WAVES * 64) % C::UPR;
-        const uint32_t off = (c < c_end && c * C::CHUNK_K + ku * C::UNIT < a.K) ? x_off[i] + (uint32_t)c * C::CHUNK_K * 2 : kOob;
+        const uint32_t row_off = C::PH == 1 ? x_off[C::PH == 1 ? i : 0] : x_base + i * x_pitch;
+        const uint32_t off = (c < c_end && c * C::CHUNK_K + x_ku * C::UNIT < a.K) ? row_off + (uint32_t)c * C::CHUNK_K * 2 : kOob;
+        const int r = (i % C::XR) * C::UW;
 #pragma unroll
-        for (int j = 0; j < C::UW; j++) xr[i * C::UW + j] = __builtin_amdgcn_raw_buffer_load_b128(rx, off + j * 16, 0, 0);
+        for (int j = 0; j < C::UW; j++) xr[r + j] = __builtin_amdgcn_raw_buffer_load_b128(rx, off + j * 16, 0, 0);
     };
     auto issue_w_load = [&](int j, int l, int c, WSet& ws) {
         const int b = c * C::CHUNK_BYTES + l * 16;
@@ -237,7 +261,7 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
     // `ph` (META4 only): position of the step in its run of four, a constant after inlining.
     static_assert(C::MF % 2 == 0, "the fragment double buffer returns to slot 0 at the end of a step");
     using GC = GroupConst<BITS>;
-    h8 xf[2][MT];
+    h8 xf[C::XB][C::XRING];
     h2 wf[2][NT][4];                                      // weight fragments as 4 register pairs each
     // group constants of tile j for the step that reads `from` (META4: half `half` of m_cur / m_next)
     auto set_consts = [&](GC* gj, int j, const WSet& from, const u2 (*m)[2], int half) {
@@ -260,7 +284,17 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
         __builtin_amdgcn_sched_barrier(0);
         const _Float16* xp = cur + nl * C::PITCH + kq * C::VPL;
 #pragma unroll
-        for (int i = 0; i < MT; i++) xf[0][i] = *reinterpret_cast<const h8*>(xp + i * 16 * C::PITCH);
+        for (int i = 0; i < C::XRING; i++) xf[0][i] = *reinterpret_cast<const h8*>(xp + i * 16 * C::PITCH);
+        // fragment of m-tile i for MFMA step t sits in xf[xc][i % XRING]; next_frag(t, i): the read issued from slot i
+        auto next_frag = [&](int t, int i) {
+            if constexpr (C::XB == 2) {
+                if (t < C::MF - 1) xf[(t & 1) ^ 1][i] = *reinterpret_cast<const h8*>(xp + i * 16 * C::PITCH + 8 * (t + 1));
+            } else {
+                const int i2 = (i + C::XRING) % MT, t2 = t + (i + C::XRING) / MT;
+                if (t2 < C::MF) xf[0][i % C::XRING] = *reinterpret_cast<const h8*>(xp + i2 * 16 * C::PITCH + 8 * t2);
+            }
+        };
+        constexpr int SPP = MT / (2 * NT);                // slots per half weight tile: work sits in the first of them
         if constexpr (!C::EARLY_W) {
 #pragma unroll
             for (int j = 0; j < NT; j++) {
@@ -279,15 +313,26 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
         auto slot_requests = [&](int t, int i) {
             static_assert(C::MF >= 4, "second and last MFMA step are distinct");
             if constexpr (META4) {
-                if (t == 1 && ph == 0) issue_meta4(i / 2, i & 1, c + C::SPR, m_next);
+                if (t == 1 && ph == 0 && i < 2 * NT) issue_meta4(i / 2, i & 1, c + C::SPR, m_next);
             } else {
-                if (t == 1) issue_meta(i / 2, i & 1, c + 2, ws);
+                if (t == 1 && i < 2 * NT) issue_meta(i / 2, i & 1, c + 2, ws);
             }
-            if (t == C::T_STAGE && i < C::XL) {
-                stage_unit(i, nxt);
-                issue_x_unit(i, c + 2);
+            if (t == C::STAGE_T0 && i >= C::SLOT0_0 && i < C::SLOT0_0 + C::XR) {
+                const int u = i - C::SLOT0_0;
+                stage_unit(u, nxt);
+                if constexpr (C::PH == 1) issue_x_unit(u, c + 2);
+                else issue_x_unit(u + C::XR, c + 1);
             }
-            if (t == C::MF - 1 && (C::WL == 2 || !(i & 1))) issue_w_load(i / 2, C::WL == 2 ? (i & 1) : 0, c + 2, ws);
+            if (C::PH == 2 && t == C::STAGE_T1 && i >= C::SLOT0_1 && i < C::SLOT0_1 + C::XR) {
+                const int u = i - C::SLOT0_1;
+                stage_unit(u + C::XR, nxt);
+                issue_x_unit(u, c + 2);
+            }
+            // weights: 2 * NT slots of the last MFMA step - the ones the second staging phase leaves free, if any
+            constexpr int W0 = (C::PH == 2 && C::STAGE_T1 == C::MF - 1) ? C::SLOT0_1 + C::XR : 0;
+            static_assert(W0 + 2 * NT <= MT, "weight requests fit behind the staging slots");
+            const int iw = i - W0;
+            if (t == C::MF - 1 && iw >= 0 && iw < 2 * NT && (C::WL == 2 || !(iw & 1))) issue_w_load(iw / 2, C::WL == 2 ? (iw & 1) : 0, c + 2, ws);
             asm volatile("" ::: "memory");
         };
         auto next_consts = [&](int j) {
@@ -297,6 +342,7 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
 #pragma unroll
         for (int t = 0; t < C::MF; t++) {
             const int cu = t & 1, nx = cu ^ 1;
+            const int xc = C::XB == 2 ? cu : 0;
             const bool last = t == C::MF - 1, early = last && C::EARLY_W;
 #pragma unroll
             for (int i = 0; i < MT; i++) {
@@ -304,8 +350,9 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
                     // An MFMA occupies the matrix pipe for 16 cycles but the issue port for 4: two or three
                     // VALU operations fit behind each one.  Slot i prepares half a weight fragment of
                     // the next MFMA step (tile i/2, words' low or high byte pair) in four such pieces.
-                    const int jn = i / 2;
-                    if (early && !(i & 1)) {
+                    const int jn = i / (2 * SPP), hi = (i / SPP) & 1;
+                    const bool act = i % SPP == 0;
+                    if (early && act && !hi) {
                         __builtin_amdgcn_sched_barrier(0);
                         next_consts(jn);
                     }
@@ -317,12 +364,12 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
 #pragma unroll
                     for (int j = 0; j < NT; j++) {
                         __builtin_amdgcn_sched_barrier(0);
-                        mfma_acc(acc[i][j], pack_h8(wf[cu][j]), xf[cu][i]);
+                        mfma_acc(acc[i][j], pack_h8(wf[cu][j]), xf[xc][i % C::XRING]);
                         __builtin_amdgcn_sched_barrier(0);
-                        if (!last || early) {
+                        if (j == (C::XB == 2 ? 0 : NT - 1)) next_frag(t, i);
+                        if ((!last || early) && act) {
                             if (j == 0) {
-                                if (!last) xf[nx][i] = *reinterpret_cast<const h8*>(xp + i * 16 * C::PITCH + 8 * (t + 1));
-                                wsrc = (i & 1) ? word >> 8 : word;
+                                wsrc = hi ? word >> 8 : word;
                                 pa = as_h2(and_or(wsrc, 0x000F000Fu, kMagic));
                             } else if (j == 1) {
                                 pb = as_h2(and_or(wsrc, 0x00F000F0u, kMagic));
@@ -332,8 +379,8 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
                                 pa = pa * g4.s;
                             } else {
                                 pb = pb * g4.s;
-                                wf[nx][jn][2 * (i & 1)] = pa;
-                                wf[nx][jn][2 * (i & 1) + 1] = pb;
+                                wf[nx][jn][2 * hi] = pa;
+                                wf[nx][jn][2 * hi + 1] = pb;
                             }
                         }
                         if (j == NT - 1) slot_requests(t, i);
@@ -342,15 +389,17 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
                     __builtin_amdgcn_sched_barrier(0);
                     // weights as the A operand: the result fragment holds 4 consecutive n per lane
 #pragma unroll
-                    for (int j = 0; j < NT; j++) mfma_acc(acc[i][j], pack_h8(wf[cu][j]), xf[cu][i]);
+                    for (int j = 0; j < NT; j++) mfma_acc(acc[i][j], pack_h8(wf[cu][j]), xf[xc][i % C::XRING]);
                     __builtin_amdgcn_sched_barrier(0);
-                    if (!last) xf[nx][i] = *reinterpret_cast<const h8*>(xp + i * 16 * C::PITCH + 8 * (t + 1));
-                    if (!(i & 1)) {
-                        if (early) next_consts(i / 2);
+                    next_frag(t, i);
+                    const int jn = i / (2 * SPP);
+                    if (i % SPP) {
+                    } else if (!((i / SPP) & 1)) {
+                        if (early) next_consts(jn);
                     } else if (!last || early) {
-                        const h8 f = early ? unpack(wsn, i / 2, 0, gn[i / 2]) : unpack(ws, i / 2, t + 1, gc[i / 2]);
+                        const h8 f = early ? unpack(wsn, jn, 0, gn[jn]) : unpack(ws, jn, t + 1, gc[jn]);
 #pragma unroll
-                        for (int e = 0; e < 4; e++) wf[nx][i / 2][e] = h2{f[2 * e], f[2 * e + 1]};
+                        for (int e = 0; e < 4; e++) wf[nx][jn][e] = h2{f[2 * e], f[2 * e + 1]};
                     }
                     slot_requests(t, i);
                 }
@@ -367,7 +416,7 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
     // any difference in order makes the steady state wait for requests it has only just issued.
     auto issue_batch = [&](int c, WSet& ws) {
 #pragma unroll
-        for (int i = 0; i < C::XL; i++) {
+        for (int i = 0; i < C::XR; i++) {           // all units of the chunk, or those of the first staging phase
             issue_x_unit(i, c);
             asm volatile("" ::: "memory");
             __builtin_amdgcn_sched_barrier(0);
@@ -400,10 +449,16 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
     }
     issue_batch(c_begin, set0);
 #pragma unroll
-    for (int i = 0; i < C::XL; i++) stage_unit(i, buf0);
+    for (int i = 0; i < C::XR; i++) stage_unit(i, buf0);
+    if constexpr (C::PH == 2) {
+#pragma unroll
+        for (int i = 0; i < C::XR; i++) issue_x_unit(C::XR + i, c_begin);
+#pragma unroll
+        for (int i = 0; i < C::XR; i++) stage_unit(C::XR + i, buf0);
+    }
     __builtin_amdgcn_sched_barrier(0);
     // second batch in the order of a steady-state step
-    if constexpr (C::T_STAGE == 0) {
+    if constexpr (C::T_STAGE == 0 || C::PH == 2) {
         issue_batch(c_begin + 1, set1);
     } else {
     if constexpr (!META4) {
@@ -416,7 +471,7 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
         }
     }
 #pragma unroll
-    for (int i = 0; i < MT; i++) {
+    for (int i = 0; i < 2 * NT; i++) {
         if (i < C::XL) issue_x_unit(i, c_begin + 1);
         if (C::WL == 2 || !(i & 1)) issue_w_load(i / 2, C::WL == 2 ? (i & 1) : 0, c_begin + 1, set1);
         asm volatile("" ::: "memory");
@@ -504,14 +559,15 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
 // a thread four consecutive n.  y[m][n] = fp16( sum_z partial_z[m][n] + bias[n] ).
 __global__ __launch_bounds__(256) void qgemm_reduce_kernel(const GemmArgs a) {
     const int tile = a.full_tiles + (int)blockIdx.y;
-    const int quad = (int)(blockIdx.x * blockDim.x + threadIdx.x);          // < BM * BN / 4
+    const int quad = (int)(blockIdx.x * blockDim.x + threadIdx.x);          // < bm * BN / 4
     const int ml = quad / (BN / 4), nl4 = (quad % (BN / 4)) * 4;
-    const int m = (tile / a.tiles_n) * BM + ml, n = (tile % a.tiles_n) * BN + nl4;
+    const int m = (tile / a.tiles_n) * a.bm + ml, n = (tile % a.tiles_n) * BN + nl4;
     if (m >= a.M || n >= a.N) return;
-    const float* src = a.ws + (size_t)blockIdx.y * a.splits * (BM * BN) + ml * BN + nl4;
+    const size_t blk = (size_t)a.bm * BN;
+    const float* src = a.ws + (size_t)blockIdx.y * a.splits * blk + ml * BN + nl4;
     f4 v = {0.f, 0.f, 0.f, 0.f};
     for (int z = 0; z < a.splits; z++) {
-        const f4 t = *reinterpret_cast<const f4*>(src + (size_t)z * (BM * BN));
+        const f4 t = *reinterpret_cast<const f4*>(src + (size_t)z * blk);
 #pragma unroll
         for (int i = 0; i < 4; i++) v[i] += t[i];
     }
@@ -537,31 +593,21 @@ struct GemmPlan {
     size_t ws_bytes;
 };
 
-inline int device_cus() {
-    static const int cus = [] {
-        int dev = 0, n = 0;
-        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess)
-            n = 0;
-        return n > 0 ? n : 256;
-    }();
-    return cus;
-}
-
 inline int gemm_chunks(int64_t K, int bits) {   // K steps of a whole row: GemmCfg::CHUNK_BYTES each
     const int64_t chunk = bits == 8 ? 128 : 64;
     return (int)((K * bits / 8 + chunk - 1) / chunk);
 }
 
-inline GemmPlan gemm_plan(int64_t M, int64_t N, int nchunks, bool have_workspace) {
+inline GemmPlan gemm_plan(int64_t M, int64_t N, int nchunks, bool have_workspace, int bm = 128) {
     GemmPlan p;
     p.tiles_n = (int)((N + BN - 1) / BN);
-    p.tiles = p.tiles_n * (int)((M + BM - 1) / BM);
+    p.tiles = p.tiles_n * (int)((M + bm - 1) / bm);
     p.full_tiles = p.tiles;
     p.splits = 1;
     p.chunks_per_split = nchunks;
     p.ws_bytes = 0;
     if (!have_workspace) return p;
-    const int cus = device_cus();
+    const int cus = bw_device_cus();
     const int rest = p.tiles <= cus / 2 ? p.tiles : p.tiles % cus;          // tiles of the (only or last) short round
     if (rest == 0 || rest > cus / 2) return p;
     int s = cus / rest;
@@ -575,30 +621,32 @@ inline GemmPlan gemm_plan(int64_t M, int64_t N, int nchunks, bool have_workspace
     p.full_tiles = p.tiles - rest;
     p.splits = s;
     p.chunks_per_split = cps;
-    p.ws_bytes = (size_t)rest * s * BM * BN * sizeof(float);
+    p.ws_bytes = (size_t)rest * s * bm * BN * sizeof(float);
     return p;
 }
 
-template <int BITS, int GROUP>
+template <int BITS, int GROUP, int MT = 8>
 int launch_gemm(GemmArgs a, void* workspace, size_t workspace_bytes, hipStream_t stream) {
-    using C = GemmCfg<BITS, GROUP>;
+    using C = GemmCfg<BITS, GROUP, MT>;
+    constexpr int BM = C::BM;
     static_assert(C::CHUNK_BYTES == (BITS == 8 ? 128 : 64), "gemm_chunks() counts K steps of this size");
     const size_t lds = 2 * (size_t)C::STAGE_BYTES;
-    void (*kern)(const GemmArgs) = qgemm_kernel<BITS, GROUP, false>;
+    void (*kern)(const GemmArgs) = qgemm_kernel<BITS, GROUP, false, MT>;
     static uint64_t big_lds_devices[2] = {0, 0};           // per kernel
     int which = 0;
     if constexpr (C::CAN_META4 || C::NG == 2) {
         // an even number of K steps (so that the loop never pads with a step that would read past the row's scales)
         // and rows of scales on 4-byte boundaries
         if (a.groups % (C::CAN_META4 ? 2 * C::GPS : 2) == 0 && bw_aligned(a.scale, 4) && bw_aligned(a.zp, 4)) {
-            kern = qgemm_kernel<BITS, GROUP, true>;
+            kern = qgemm_kernel<BITS, GROUP, true, MT>;
             which = 1;
         }
     }
     if (lds > 64 * 1024 && !bw_allow_big_lds(reinterpret_cast<const void*>(kern), big_lds_devices[which])) return BW_ELAUNCH;
-    const GemmPlan p = gemm_plan(a.M, a.N, a.nchunks, workspace != nullptr);
+    const GemmPlan p = gemm_plan(a.M, a.N, a.nchunks, workspace != nullptr, BM);
     if (p.ws_bytes > workspace_bytes) return BW_EWORKSPACE;
     a.ws = (float*)workspace;
+    a.bm = BM;
     a.tiles_n = p.tiles_n;
     a.full_tiles = p.full_tiles;
     a.splits = p.splits;
@@ -611,6 +659,22 @@ int launch_gemm(GemmArgs a, void* workspace, size_t workspace_bytes, hipStream_t
         if (hipGetLastError() != hipSuccess) return BW_ELAUNCH;
     }
     return BW_OK;
+}
+
+// Rows of a tile for this call.  A 256-row tile unpacks every weight once for twice the rows (0.8 instead of 1.5
+// unpack instructions per MFMA in a loop that is bound by the instructions a wave can issue) and runs 14 % faster per
+// row - when its grid fills the device: measured at 4 and 8 bits, K and N from 4096 to 14336, the 256-row grid wins
+// (3-15 %) from about 0.6 rounds of tiles on and loses (up to 28 %) below.  Not at 2 bits (a K step of 256 values for
+// 256 rows does not fit LDS twice), and only while the split-K blocks of its plan fit the workspace on offer.
+inline int gemm_tile_rows(int64_t M, int64_t N, int64_t ldx, int bits, int nchunks, bool have_workspace, size_t workspace_bytes) {
+    if (bits == 2 || (M + 256) * ldx * 2 >= ((int64_t)1 << 32)) return 128;
+#ifdef BW_TUNE
+    if (const char* e = getenv("BW_GEMM_BM")) return atoi(e) == 256 ? 256 : 128;
+#endif
+    const int64_t tiles = ((N + BN - 1) / BN) * ((M + 255) / 256);
+    if (tiles * 5 < (int64_t)bw_device_cus() * 3) return 128;
+    if (have_workspace && gemm_plan(M, N, nchunks, true, 256).ws_bytes > workspace_bytes) return 128;
+    return 256;
 }
 
 // Shape-generic fallback: one thread per output element, any group size and
@@ -696,7 +760,16 @@ int bw_qgemm_generic(const void* x, int act_dtype, int64_t M, int64_t K, int64_t
 
 extern "C" size_t bw_qgemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int bits, int group) {
     if (!bw_shape_ok(N, K, bits, group) || M < 1 || M >= ((int64_t)1 << 31) || !bw_fast_shape(M, N, K, K, bits, group)) return 0;
-    return gemm_plan(M, N, gemm_chunks(K, bits), true).ws_bytes;
+    const int nchunks = gemm_chunks(K, bits);
+    const size_t small = gemm_plan(M, N, nchunks, true, 128).ws_bytes;     // either plan may run: enough for both
+    if (gemm_tile_rows(M, N, K, bits, nchunks, false, 0) == 128) return small;
+    const size_t big = gemm_plan(M, N, nchunks, true, 256).ws_bytes;
+    return big > small ? big : small;
+}
+
+extern "C" int bw_qgemm_tile_rows(int64_t M, int64_t N, int64_t K, int bits, int group) {
+    if (!bw_shape_ok(N, K, bits, group) || M < 1 || M >= ((int64_t)1 << 31) || !bw_fast_shape(M, N, K, K, bits, group)) return 0;
+    return gemm_tile_rows(M, N, K, bits, gemm_chunks(K, bits), false, 0);
 }
 
 extern "C" int bw_qgemm_ws(const void* x, int act_dtype, int64_t M, int64_t K, int64_t ldx, const int32_t* qweight,
@@ -723,12 +796,16 @@ extern "C" int bw_qgemm_ws(const void* x, int act_dtype, int64_t M, int64_t K, i
     a.splits = 1;
     a.chunks_per_split = a.nchunks;
     hipStream_t st = (hipStream_t)stream;
+    const bool big = gemm_tile_rows(M, N, ldx, bits, a.nchunks, workspace != nullptr, workspace_bytes) == 256;
 #define BW_CASE(B, G) \
     if (bits == B && group == G) return launch_gemm<B, G>(a, workspace, workspace_bytes, st);
-    BW_CASE(4, 128) BW_CASE(4, 64) BW_CASE(4, 32)
-    BW_CASE(8, 128) BW_CASE(8, 64) BW_CASE(8, 32)
+#define BW_CASE2(B, G) \
+    if (bits == B && group == G) return big ? launch_gemm<B, G, 16>(a, workspace, workspace_bytes, st) : launch_gemm<B, G>(a, workspace, workspace_bytes, st);
+    BW_CASE2(4, 128) BW_CASE2(4, 64) BW_CASE2(4, 32)
+    BW_CASE2(8, 128) BW_CASE2(8, 64) BW_CASE2(8, 32)
     BW_CASE(2, 128) BW_CASE(2, 64) BW_CASE(2, 32)
 #undef BW_CASE
+#undef BW_CASE2
     return BW_EUNSUPPORTED;
 }
 

@@ -20,9 +20,9 @@ BW_F16, BW_BF16, BW_F32, BW_I32, BW_F64 = 0, 1, 2, 3, 4
 BW_SCALE_RECIPROCAL = 0x100   # flag for math_dtype: scale = (max - min) * fl32(1 / Qmax), as eager torch computes it on a GPU
 _DTYPE_CODE = {torch.float16: BW_F16, torch.bfloat16: BW_BF16, torch.float32: BW_F32, torch.int32: BW_I32, torch.float64: BW_F64}
 
-ABI_VERSION = 8            # what bw_abi_version() of a matching library returns
+ABI_VERSION = 9            # what bw_abi_version() of a matching library returns
 ENTRY_POINTS = ("bw_abi_version", "bw_strerror", "bw_quantize_pack", "bw_quantize_pack_add", "bw_dequantize", "bw_qgemv", "bw_qgemm",
-                "bw_qgemm_ws", "bw_qgemm_static", "bw_qgemm_workspace_bytes", "bw_qlinear", "bw_qdgrad", "bw_qdgrad_workspace_bytes", "bw_cast_bf16_f16", "bw_qlinear_decode_rows", "bw_qgemv_last_kernel")
+                "bw_qgemm_ws", "bw_qgemm_static", "bw_qgemm_workspace_bytes", "bw_qgemm_tile_rows", "bw_qlinear", "bw_qdgrad", "bw_qdgrad_workspace_bytes", "bw_cast_bf16_f16", "bw_qlinear_decode_rows", "bw_qgemv_last_kernel")
 
 
 class BitweenHipError(RuntimeError):
@@ -59,6 +59,8 @@ def load():
     lib.bw_qgemm_ws.argtypes = mm[:-1] + [vp, ctypes.c_size_t, vp]
     lib.bw_qgemm_workspace_bytes.argtypes = [i64, i64, i64, i32, i32]
     lib.bw_qgemm_workspace_bytes.restype = ctypes.c_size_t
+    lib.bw_qgemm_tile_rows.argtypes = [i64, i64, i64, i32, i32]
+    lib.bw_qgemm_tile_rows.restype = i32
     lib.bw_qdgrad_workspace_bytes.argtypes = [i64, i64, i64, i32, i32]
     lib.bw_qdgrad_workspace_bytes.restype = ctypes.c_size_t
     lib.bw_qdgrad.argtypes = [vp, i32, i64, i64, i64, vp, vp, vp, i64, i32, i32, vp, i64, vp, ctypes.c_size_t, vp]

@@ -903,3 +903,75 @@ def test_sibling_group_does_not_serve_a_member_twice_from_its_cache():
     assert torch.allclose(y2.float(), 2 * y1.float(), rtol=2e-3, atol=1e-3)
     ref_k = bitween_amd.kernels.hip_loader.quantized_matmul_hip(x, blk.k_proj.qweight, blk.k_proj.scale, blk.k_proj.zero_point, None, 4, 128)
     assert torch.equal(k2, ref_k)
+
+
+@pytest.mark.parametrize("bits,g", [(4, 128), (4, 64), (4, 32), (8, 128), (8, 64), (8, 32)])
+@pytest.mark.parametrize("k", [896, 1024])
+def test_prefill_256_row_tiles_vs_oracle(bits, g, k):
+    """Shapes whose grid of 256-row tiles fills the device take the 256-row variant of the prefill kernel (same
+    arithmetic as bitween/modules.py:85-97, twice the rows per unpacked weight): ragged in M and N, an even and an odd
+    number of K steps (with and without the wide scale requests), with and without bias - sampled rows from every part
+    of the row range against the oracle, one-hot rows bit for bit, and the workspace plan against the plain one."""
+    import ctypes
+    hip = _hip()
+    lib = hip.load()
+    m, n = 256 * 52 + 37, 700
+    if lib.bw_qgemm_tile_rows(m, n, k, bits, g) != 256:
+        pytest.skip("this device's CU count does not put the shape on 256-row tiles")
+    _, qw, s16, z16, b16 = quantized_layer(n, k, bits, g, seed=bits * 100 + g + k, outliers=True)
+    w16 = orc.dequantize_f16(qw, s16, z16, g, bits)
+    gen = torch.Generator(device="cuda").manual_seed(k + bits)
+    x = torch.randn(m, k, device="cuda", generator=gen).half()
+    hot = {0: 0, 255: k - 1, 256: 129, 4001: k // 2, m - 38: 31, m - 1: k - 2}       # row -> column of its single 1
+    for r, c in hot.items():
+        x[r] = 0
+        x[r, c] = 1.0
+    d = [to_gpu(a) for a in (qw, s16, z16, b16)]
+    y_ws = hip.quantized_gemm_hip(x, d[0], d[1], d[2], d[3], bits, g)
+    y_plain = torch.full((m, n), float("nan"), dtype=torch.float16, device="cuda")
+    assert lib.bw_qgemm(x.data_ptr(), 0, m, k, k, d[0].data_ptr(), d[1].data_ptr(), d[2].data_ptr(), None, n, bits, g,
+                        y_plain.data_ptr(), n, ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)) == 0
+    torch.cuda.synchronize()
+    rows = np.unique(np.concatenate([np.arange(0, m, 997), np.arange(250, 262), np.arange(m - 40, m)]))
+    x_np = x[torch.from_numpy(rows).cuda()].cpu().numpy()
+    check_matmul(y_ws[torch.from_numpy(rows).cuda()], x_np, qw, s16, z16, b16, bits, g)
+    check_matmul(y_plain[torch.from_numpy(rows).cuda()], x_np, qw, s16, z16, None, bits, g)
+    for r, c in hot.items():
+        assert np.array_equal(y_plain[r].cpu().numpy().view(np.uint16), w16[:, c].view(np.uint16))
+    # every row of the full result: finite, and equal to the library GEMM on the dequantised weights to float16 rounding
+    ref = x @ to_gpu(w16).T
+    assert torch.isfinite(y_plain).all()
+    assert ((y_plain.float() - ref.float()).abs().max() <= 2.0 ** -8 * ref.float().abs().max()).item()
+
+
+def test_prefill_256_row_tiles_split_the_short_last_round():
+    """260 tiles of 256 rows on 256 CUs: the four tiles of the second round are cut along K into partial tiles of
+    256 x 256 floats that the reduce kernel adds up; against the un-split run everywhere and the oracle on rows of both
+    kinds of tile."""
+    import ctypes
+    from bitween_amd.kernels import hip_loader
+    lib = hip_loader.load()
+    bits, g, m, k, n = 4, 128, 256 * 52, 2048, 1280
+    need = lib.bw_qgemm_workspace_bytes(m, n, k, bits, g)
+    if lib.bw_qgemm_tile_rows(m, n, k, bits, g) != 256 or need == 0:
+        pytest.skip("this device's CU count leaves no short last round of 256-row tiles for this shape")
+    assert need % (256 * 256 * 4) == 0
+    _, qw, s16, z16, b16 = quantized_layer(n, k, bits, g, seed=79, outliers=True)
+    gen = torch.Generator(device="cuda").manual_seed(80)
+    x = torch.randn(m, k, device="cuda", generator=gen).half()
+    d = [to_gpu(a) for a in (qw, s16, z16, b16)]
+    ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+    st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    ys = []
+    for ws_ptr, ws_bytes in ((ws.data_ptr(), need), (None, 0)):
+        y = torch.full((m, n), float("nan"), dtype=torch.float16, device="cuda")
+        assert lib.bw_qgemm_ws(x.data_ptr(), 0, m, k, k, d[0].data_ptr(), d[1].data_ptr(), d[2].data_ptr(), d[3].data_ptr(),
+                               n, bits, g, y.data_ptr(), n, ws_ptr, ws_bytes, st) == 0
+        ys.append(y)
+    torch.cuda.synchronize()
+    assert torch.isfinite(ys[0]).all()
+    diff = (ys[0].float() - ys[1].float()).abs().max().item()
+    assert diff <= 2.0 ** -9 * ys[1].float().abs().max().item()
+    rows = np.r_[0:20, m - 300:m - 280, m - 20:m]
+    idx = torch.from_numpy(rows).cuda()
+    check_matmul(ys[0][idx], x[idx].cpu().numpy(), qw, s16, z16, b16, bits, g)
