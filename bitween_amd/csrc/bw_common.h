@@ -1,6 +1,7 @@
 // Shared device helpers for the gfx950 kernels of libbitween_hip.so.
 #pragma once
 #include <hip/hip_runtime.h>
+#include <type_traits>
 #include <stdint.h>
 
 #include "../../include/bitween_hip.h"
@@ -165,6 +166,16 @@ BW_DEV h8 pack_h8(const h2* p) {
     r[0] = p[0][0]; r[1] = p[0][1]; r[2] = p[1][0]; r[3] = p[1][1];
     r[4] = p[2][0]; r[5] = p[2][1]; r[6] = p[3][0]; r[7] = p[3][1];
     return r;
+}
+
+// f(integral_constant<int, 0>{}), ..., f(integral_constant<int, N - 1>{}): a loop whose index is a constant expression
+// in the body (immediate operands, if constexpr) and that is unrolled whatever its size.
+template <int I, int N, class F>
+BW_DEV void static_for(F&& f) {
+    if constexpr (I < N) {
+        f(std::integral_constant<int, I>{});
+        static_for<I + 1, N>(f);
+    }
 }
 
 // Host-side argument checks shared by the entry points.

@@ -171,7 +171,9 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
 #pragma unroll
     for (int j = 0; j < NT; j++) {
         const int row = n0 + 16 * j + nl;
-        w_off[j] = row < a.N ? (uint32_t)row * a.row_bytes + kq * 16 * C::WL : kOob;
+        // (256-row tiles add a scalar chunk offset that is itself "out of range" past the last chunk: rows past N then
+        // read the last row's bytes instead of relying on a sum that could wrap; their outputs are never stored)
+        w_off[j] = row < a.N ? (uint32_t)row * a.row_bytes + kq * 16 * C::WL : MT == 16 ? (uint32_t)(a.N - 1) * a.row_bytes + kq * 16 * C::WL : kOob;
         m_off[j] = (uint32_t)min(row, a.N - 1) * groups * 2;
     }
     // Staging unit i of a thread: row tid / UPR + i * RPI of the tile, the thread's UNIT-wide column ku of the chunk.
@@ -279,7 +281,7 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
                 gj[g].set(__builtin_bit_cast(_Float16, (uint16_t)from.s[j][g]), __builtin_bit_cast(_Float16, (uint16_t)from.z[j][g]));
         }
     };
-    auto step = [&](int c, const _Float16* cur, _Float16* nxt, WSet& ws, const WSet& wsn, GC (&gc)[NT][C::NG],
+    auto step8 = [&](int c, const _Float16* cur, _Float16* nxt, WSet& ws, const WSet& wsn, GC (&gc)[NT][C::NG],
                     GC (&gn)[NT][C::NG], const int ph) {
         __builtin_amdgcn_sched_barrier(0);
         const _Float16* xp = cur + nl * C::PITCH + kq * C::VPL;
@@ -409,6 +411,138 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
         __syncthreads();
     };
 
+    // ---- One K step of the 256-row tile --------------------------------------------------------------------------
+    // A wave issues in order, and what it can put between two MFMAs without holding up the matrix pipe is about one
+    // VALU instruction plus one other (measured: 16 cycles per MFMA with one, 19 with two, 20 with three; LDS, scalar
+    // and wait instructions cost 1-2 each).  So the side work of an MFMA step is cut into single instructions and dealt
+    // out one per gap, by position: gap g = 4 i + j follows the MFMA of m-tile i and n-tile j; region r = g / 16 and
+    // k = g % 16 name the 16 gaps of four slots.
+    //   unpack    : n-tile r's fragment for the next MFMA step, 12-13 instructions, one in each of k = 0..12
+    //               (the last MFMA step prepares the first fragment of the next K step from the other register set);
+    //   staging   : unit u = 4 t + r of the next chunk, requested two MFMA steps earlier: permutes at k = 0, 2, 4, 6,
+    //               LDS write at k = 8, address at k = 10 and the request of unit u + 8 (of this chunk, or of the one
+    //               after it) into the same registers at k = 12;
+    //   fragments : slot i's last gap reads the activation fragment of slot i + 8 into the ring;
+    //   requests  : scales / zero points at k = 14, 15 of the second MFMA step, weights at k = 14, 15 of the last,
+    //               group constants of the next step at k = 13 of the last but one.
+    // Request addresses are one VGPR per thread plus a scalar: the chunk part of an offset is uniform, and past the
+    // slice it is replaced by an offset beyond every buffer, so that the hardware's range check returns zeros.
+    // Requires K % CHUNK_K == 0 (the launcher's condition for this variant): no request straddles the end of a row.
+    h2 up[NT][4];
+    uint32_t uw[NT];
+    uint32_t xo[4];
+    auto x_req16 = [&](int u, int cc) {
+        const uint32_t so = cc < c_end ? (uint32_t)u * x_pitch + (uint32_t)cc * C::CHUNK_K * 2 : kOob;
+        return x_base + so;
+    };
+    auto w_req16 = [&](int j, int l, int cc, WSet& ws) {
+        const uint32_t so = cc < c_end ? (uint32_t)cc * C::CHUNK_BYTES + l * 16 : kOob;
+        ws.w[j][l] = __builtin_amdgcn_raw_buffer_load_b128(rw, w_off[j] + so, 0, 0);
+    };
+    auto x_load16 = [&](int u, uint32_t off) {
+        const int r = (u % C::XR) * C::UW;
+#pragma unroll
+        for (int j = 0; j < C::UW; j++) xr[r + j] = __builtin_amdgcn_raw_buffer_load_b128(rx, off + j * 16, 0, 0);
+    };
+    auto step16 = [&](int c, const _Float16* cur, _Float16* nxt, WSet& ws, const WSet& wsn, GC (&gc)[NT][C::NG],
+                      GC (&gn)[NT][C::NG], const int ph) {
+        static_assert(MT != 16 || (C::NG == 1 && C::UW == 1 && C::XR == 8 && C::MF == 4), "layout of the 256-row schedule");
+        __builtin_amdgcn_sched_barrier(0);
+        const _Float16* xp = cur + nl * C::PITCH + kq * C::VPL;
+#pragma unroll
+        for (int i = 0; i < C::XRING; i++) xf[0][i] = *reinterpret_cast<const h8*>(xp + i * 16 * C::PITCH);
+        const h2 k16 = splat((_Float16)0.0625f);
+        static_for<0, C::MF>([&](auto tc) {
+            constexpr int t = decltype(tc)::value, cu = t & 1, nx = cu ^ 1;
+            constexpr bool early = t == C::MF - 1;
+            const WSet& src = early ? wsn : ws;
+            constexpr int tt = early ? 0 : t + 1;
+            static_for<0, 4 * MT>([&](auto gcnt) {
+                constexpr int g = decltype(gcnt)::value, i = g / NT, j = g % NT, r = g / 16, k = g % 16;
+                __builtin_amdgcn_sched_barrier(0);
+                mfma_acc(acc[i][j], pack_h8(wf[cu][j]), xf[0][i % C::XRING]);
+                __builtin_amdgcn_sched_barrier(0);
+                // ---- unpack of n-tile r ----
+                const GC& gr = early ? gn[r][0] : gc[r][0];
+                if constexpr (BITS == 4) {
+                    const uint32_t word = src.w[r][0][tt];
+                    if (k == 0) up[r][0] = as_h2(and_or(word, 0x000F000Fu, kMagic));
+                    if (k == 1) up[r][1] = as_h2(and_or(word, 0x00F000F0u, kMagic));
+                    if (k == 2) up[r][0] = up[r][0] + gr.z0;
+                    if (k == 3) up[r][1] = __builtin_elementwise_fma(up[r][1], k16, gr.z1);
+                    if (k == 4) wf[nx][r][0] = up[r][0] * gr.s;
+                    if (k == 5) wf[nx][r][1] = up[r][1] * gr.s;
+                    if (k == 6) uw[r] = word >> 8;
+                    if (k == 7) up[r][2] = as_h2(and_or(uw[r], 0x000F000Fu, kMagic));
+                    if (k == 8) up[r][3] = as_h2(and_or(uw[r], 0x00F000F0u, kMagic));
+                    if (k == 9) up[r][2] = up[r][2] + gr.z0;
+                    if (k == 10) up[r][3] = __builtin_elementwise_fma(up[r][3], k16, gr.z1);
+                    if (k == 11) wf[nx][r][2] = up[r][2] * gr.s;
+                    if (k == 12) wf[nx][r][3] = up[r][3] * gr.s;
+                } else {
+                    // 8 bits: the two words of MFMA step tt are words 2 (tt % 2), + 1 of lane load tt / 2
+                    const uint32_t w0 = src.w[r][tt / C::SPL][2 * (tt % C::SPL)], w1 = src.w[r][tt / C::SPL][2 * (tt % C::SPL) + 1];
+                    if (k == 0) up[r][0] = as_h2(__builtin_amdgcn_perm(0x64646464u, w0, 0x04010400u));
+                    if (k == 1) up[r][1] = as_h2(__builtin_amdgcn_perm(0x64646464u, w0, 0x04030402u));
+                    if (k == 2) up[r][0] = up[r][0] + gr.z0;
+                    if (k == 3) up[r][1] = up[r][1] + gr.z0;
+                    if (k == 4) wf[nx][r][0] = up[r][0] * gr.s;
+                    if (k == 5) wf[nx][r][1] = up[r][1] * gr.s;
+                    if (k == 6) up[r][2] = as_h2(__builtin_amdgcn_perm(0x64646464u, w1, 0x04010400u));
+                    if (k == 7) up[r][3] = as_h2(__builtin_amdgcn_perm(0x64646464u, w1, 0x04030402u));
+                    if (k == 8) up[r][2] = up[r][2] + gr.z0;
+                    if (k == 9) up[r][3] = up[r][3] + gr.z0;
+                    if (k == 10) wf[nx][r][2] = up[r][2] * gr.s;
+                    if (k == 11) wf[nx][r][3] = up[r][3] * gr.s;
+                }
+                // ---- staging of unit u, then the request of unit u + 8 ----
+                {
+                    const int u = 4 * t + r, rs = u % C::XR;
+                    if constexpr (BITS == 4) {
+                        if (k == 0) xo[0] = __builtin_amdgcn_perm(xr[rs][2], xr[rs][0], 0x05040100u);
+                        if (k == 2) xo[1] = __builtin_amdgcn_perm(xr[rs][2], xr[rs][0], 0x07060302u);
+                        if (k == 4) xo[2] = __builtin_amdgcn_perm(xr[rs][3], xr[rs][1], 0x05040100u);
+                        if (k == 6) xo[3] = __builtin_amdgcn_perm(xr[rs][3], xr[rs][1], 0x07060302u);
+                    }
+                    if (k == 8) {
+                        u4* dst = reinterpret_cast<u4*>(nxt + (tid / C::UPR + u * RPI) * C::PITCH + x_ku * C::UNIT);
+                        if constexpr (BITS == 4) *dst = u4{xo[0], xo[1], xo[2], xo[3]};
+                        else *dst = xr[rs];
+                    }
+                    const int u2 = (u + 8) % C::XL, c2 = c + 1 + (u + 8) / C::XL;
+                    if (k == 10) xo[0] = x_req16(u2, c2);
+                    if (k == 12) x_load16(u2, xo[0]);
+                }
+                // ---- fragment ring ----
+                if (j == NT - 1) {
+                    const int i2 = (i + C::XRING) % MT, t2 = t + (i + C::XRING) / MT;
+                    if (t2 < C::MF) xf[0][i % C::XRING] = *reinterpret_cast<const h8*>(xp + i2 * 16 * C::PITCH + 8 * t2);
+                }
+                // ---- requests and constants ----
+                if (t == 1 && k >= 14) {
+                    if constexpr (META4) {
+                        if (ph == 0) issue_meta4(r, k - 14, c + C::SPR, m_next);
+                    } else {
+                        issue_meta(r, k - 14, c + 2, ws);
+                    }
+                }
+                if (t == C::MF - 2 && k == 13) {
+                    if constexpr (META4) set_consts(gn[r], r, wsn, ph < C::SPR - 1 ? m_cur : m_next, ph < C::SPR - 1 ? ph + 1 : 0);
+                    else set_consts(gn[r], r, wsn, m_cur, 0);
+                }
+                if (t == C::MF - 1 && k >= 16 - C::WL) w_req16(r, k - (16 - C::WL), c + 2, ws);
+                asm volatile("" ::: "memory");
+            });
+        });
+        __builtin_amdgcn_sched_barrier(0);
+        __syncthreads();
+    };
+    auto step = [&](int c, const _Float16* cur, _Float16* nxt, WSet& ws, const WSet& wsn, GC (&gc)[NT][C::NG], GC (&gn)[NT][C::NG],
+                    const int ph) {
+        if constexpr (MT == 16) step16(c, cur, nxt, ws, wsn, gc, gn, ph);
+        else step8(c, cur, nxt, ws, wsn, gc, gn, ph);
+    };
+
     _Float16* buf0 = reinterpret_cast<_Float16*>(smem);
     _Float16* buf1 = reinterpret_cast<_Float16*>(smem + C::STAGE_BYTES);
     // Prologue: the same two request batches, in the same order, that a steady-state step finds
@@ -458,7 +592,33 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
     }
     __builtin_amdgcn_sched_barrier(0);
     // second batch in the order of a steady-state step
-    if constexpr (C::T_STAGE == 0 || C::PH == 2) {
+    if constexpr (MT == 16) {
+        if constexpr (!META4) {
+#pragma unroll
+            for (int j = 0; j < NT; j++) {
+                issue_meta(j, 0, c_begin + 1, set1);
+                issue_meta(j, 1, c_begin + 1, set1);
+                asm volatile("" ::: "memory");
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            x_load16(u, x_req16(u, c_begin + 1));
+            asm volatile("" ::: "memory");
+            __builtin_amdgcn_sched_barrier(0);
+        }
+#pragma unroll
+        for (int j = 0; j < NT; j++) {
+            x_load16(4 + j, x_req16(4 + j, c_begin + 1));
+            asm volatile("" ::: "memory");
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int l = 0; l < C::WL; l++) w_req16(j, l, c_begin + 1, set1);
+            asm volatile("" ::: "memory");
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    } else if constexpr (C::T_STAGE == 0 || C::PH == 2) {
         issue_batch(c_begin + 1, set1);
     } else {
     if constexpr (!META4) {
@@ -666,8 +826,8 @@ int launch_gemm(GemmArgs a, void* workspace, size_t workspace_bytes, hipStream_t
 // row - when its grid fills the device: measured at 4 and 8 bits, K and N from 4096 to 14336, the 256-row grid wins
 // (3-15 %) from about 0.6 rounds of tiles on and loses (up to 28 %) below.  Not at 2 bits (a K step of 256 values for
 // 256 rows does not fit LDS twice), and only while the split-K blocks of its plan fit the workspace on offer.
-inline int gemm_tile_rows(int64_t M, int64_t N, int64_t ldx, int bits, int nchunks, bool have_workspace, size_t workspace_bytes) {
-    if (bits == 2 || (M + 256) * ldx * 2 >= ((int64_t)1 << 32)) return 128;
+inline int gemm_tile_rows(int64_t M, int64_t N, int64_t K, int64_t ldx, int bits, int nchunks, bool have_workspace, size_t workspace_bytes) {
+    if (bits == 2 || K % 128 || (M + 256) * ldx * 2 >= ((int64_t)1 << 32)) return 128;   // whole K steps of 128 values only
 #ifdef BW_TUNE
     if (const char* e = getenv("BW_GEMM_BM")) return atoi(e) == 256 ? 256 : 128;
 #endif
@@ -762,14 +922,14 @@ extern "C" size_t bw_qgemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int 
     if (!bw_shape_ok(N, K, bits, group) || M < 1 || M >= ((int64_t)1 << 31) || !bw_fast_shape(M, N, K, K, bits, group)) return 0;
     const int nchunks = gemm_chunks(K, bits);
     const size_t small = gemm_plan(M, N, nchunks, true, 128).ws_bytes;     // either plan may run: enough for both
-    if (gemm_tile_rows(M, N, K, bits, nchunks, false, 0) == 128) return small;
+    if (gemm_tile_rows(M, N, K, K, bits, nchunks, false, 0) == 128) return small;
     const size_t big = gemm_plan(M, N, nchunks, true, 256).ws_bytes;
     return big > small ? big : small;
 }
 
 extern "C" int bw_qgemm_tile_rows(int64_t M, int64_t N, int64_t K, int bits, int group) {
     if (!bw_shape_ok(N, K, bits, group) || M < 1 || M >= ((int64_t)1 << 31) || !bw_fast_shape(M, N, K, K, bits, group)) return 0;
-    return gemm_tile_rows(M, N, K, bits, gemm_chunks(K, bits), false, 0);
+    return gemm_tile_rows(M, N, K, K, bits, gemm_chunks(K, bits), false, 0);
 }
 
 extern "C" int bw_qgemm_ws(const void* x, int act_dtype, int64_t M, int64_t K, int64_t ldx, const int32_t* qweight,
@@ -796,7 +956,7 @@ extern "C" int bw_qgemm_ws(const void* x, int act_dtype, int64_t M, int64_t K, i
     a.splits = 1;
     a.chunks_per_split = a.nchunks;
     hipStream_t st = (hipStream_t)stream;
-    const bool big = gemm_tile_rows(M, N, ldx, bits, a.nchunks, workspace != nullptr, workspace_bytes) == 256;
+    const bool big = gemm_tile_rows(M, N, K, ldx, bits, a.nchunks, workspace != nullptr, workspace_bytes) == 256;
 #define BW_CASE(B, G) \
     if (bits == B && group == G) return launch_gemm<B, G>(a, workspace, workspace_bytes, st);
 #define BW_CASE2(B, G) \

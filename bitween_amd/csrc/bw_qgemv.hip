@@ -698,15 +698,6 @@ BW_DEV void lds_barrier() {
     asm volatile("" ::: "memory");
 }
 
-// f(integral_constant<int, 0>{}), ..., f(integral_constant<int, N - 1>{}): a loop whose index is a constant expression
-template <int I, int N, class F>
-BW_DEV void static_for(F&& f) {
-    if constexpr (I < N) {
-        f(std::integral_constant<int, I>{});
-        static_for<I + 1, N>(f);
-    }
-}
-
 // wait until at most `n` of this wave's memory loads are outstanding (loads return in order)
 template <int N>
 BW_DEV void wait_loads() {
