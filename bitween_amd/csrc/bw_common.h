@@ -178,6 +178,23 @@ BW_DEV void static_for(F&& f) {
     }
 }
 
+// Workgroup barrier for LDS data that ordinary stores of this wave wrote: waits for the wave's own LDS operations and
+// then for the other waves, without the memory fence of __syncthreads() - a fence would also wait for every weight
+// request in flight, since those land in LDS too.
+BW_DEV void lds_barrier() {
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_waitcnt(0xC07F);                   // lgkmcnt(0)
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+}
+
+// wait until at most `n` of this wave's memory loads are outstanding (loads return in order)
+template <int N>
+BW_DEV void wait_loads() {
+    static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
+    __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | 0x0F70);   // expcnt and lgkmcnt left alone
+}
+
 // Host-side argument checks shared by the entry points.
 static inline bool bw_bits_ok(int bits) { return bits == 2 || bits == 4 || bits == 8; }
 static inline bool bw_shape_ok(int64_t N, int64_t K, int bits, int group) {

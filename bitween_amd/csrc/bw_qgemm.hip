@@ -51,7 +51,9 @@ struct GemmCfg {
     static constexpr bool EARLY_W = BITS == 4 || (BITS == 2 && GROUP == 32);
     static constexpr int T_STAGE = BITS == 4 ? MF - 1 : (BITS == 2 && GROUP == 32) ? MF - 2 : 0;
     static constexpr int PITCH = CHUNK_K + 8;                    // halves per LDS row
-    static constexpr int STAGE_BYTES = BM * PITCH * 2;
+    // 128 rows: padded rows written by the staging threads; 256 rows: 256-byte rows written by buffer loads with LDS
+    // destination, unpadded, the 16-byte slots of a row XOR-swizzled by the row number instead
+    static constexpr int STAGE_BYTES = MT == 16 ? BM * CHUNK_K * 2 : BM * PITCH * 2;
     static constexpr int UNIT = VPI > 8 ? VPI : 8;               // halves permuted together when staging x
     static constexpr int UW = UNIT / 8;
     static constexpr int UPR = CHUNK_K / UNIT;                   // staging units per x row
@@ -88,6 +90,30 @@ BW_DEV void permute_unit(const uint32_t* r, uint32_t* o) {
     }
 }
 
+// Group constants and unpack for fragments in natural k order (256-row tiles, whose activations go from memory to LDS
+// without passing through registers and so cannot be permuted on the way).  A 4-bit word w = bytes B0..B3, nibbles
+// n0..n7: p = [B0 B1 B0 B1] and q = [B2 B3 B2 B3] (one byte permute each) hold n0 in bits 0-3 of their low half and
+// n1 in bits 4-7 of their high half, p >> 8 likewise n2 and n3; masked into the mantissa of 1024.0 that is
+// (1024 + n0, 1024 + 16 n1), and one packed FMA with (1, 1/16) and (-(1024 + z), -(64 + z)) leaves (n0 - z, n1 - z),
+// both exact.  Times the scale: the float16 the reference's dequantize stores (bitween/modules.py:55-58).
+template <int BITS> struct GroupConstNat {
+    h2 s, zz;
+    BW_DEV void set(_Float16 sv, _Float16 zv) {
+        s = splat(sv);
+        if constexpr (BITS == 4) zz = h2{(_Float16)(-1024.0f) - zv, (_Float16)(-64.0f) - zv};
+        else zz = splat((_Float16)(-1024.0f) - zv);
+    }
+};
+
+BW_DEV void dequant_word4_nat(uint32_t w, const GroupConstNat<4>& c, h2 out[4]) {
+    const h2 kk = h2{(_Float16)1.0f, (_Float16)0.0625f};
+    const uint32_t p = __builtin_amdgcn_perm(w, w, 0x01000100u), q = __builtin_amdgcn_perm(w, w, 0x03020302u);
+    const uint32_t src[4] = {p, p >> 8, q, q >> 8};
+#pragma unroll
+    for (int e = 0; e < 4; e++)
+        out[e] = __builtin_elementwise_fma(as_h2(and_or(src[e], 0x00F0000Fu, kMagic)), kk, c.zz) * c.s;
+}
+
 // Unpack word t of a lane load (8 values for MFMA step t at 4 bits; two steps' worth at 2 bits, half a
 // step at 8 bits is handled by the caller) - thin wrappers so the K loop can unpack just in time.
 template <int BITS>
@@ -113,6 +139,14 @@ BW_DEV h8 unpack_step(const u4& w, int t, const GroupConst<BITS>* gc, int ng_wor
 // the epilogue, hundreds of cycles (an LDS staging pass and a barrier) after the last MFMA.
 BW_DEV void mfma_acc(f4& acc, const h8& a, const h8& b) {
     asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
+}
+
+// 16 bytes per lane from LDS byte address `addr` + OFF, as an instruction the compiler does not know to be an LDS read
+// (its result is ready only after an s_waitcnt lgkmcnt the caller places).
+template <int OFF>
+BW_DEV void lds_read_b128(h8& dst, uint32_t addr) {
+    static_assert(OFF >= 0 && OFF < 65536, "16-bit offset field");
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(OFF));
 }
 
 struct GemmArgs {
@@ -248,9 +282,24 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
         m[j][which] = __builtin_amdgcn_raw_buffer_load_b64(which == 0 ? rs : rz, m_off[j] + c * (2 * C::GPS), 0, 0);
     };
     // Weight fragment of MFMA step t: values [8 t, 8 t + 8) of the lane's VPL, from lane load t / SPL.
-    auto unpack = [&](const WSet& ws, int j, int t, const GroupConst<BITS>* gcj) {
+    auto unpack = [&](const WSet& ws, int j, int t, const auto* gcj) {
         static_assert(C::WL == 1 || C::NG == 1, "two lane loads share one group");
-        return unpack_step<BITS>(ws.w[j][t / C::SPL], t % C::SPL, gcj, C::WPG);
+        if constexpr (MT == 16) {                             // natural k order
+            h2 o[4];
+            if constexpr (BITS == 4) {
+                dequant_word4_nat(ws.w[j][0][t], gcj[0], o);
+            } else {
+#pragma unroll
+                for (int e = 0; e < 2; e++) {
+                    const uint32_t w = ws.w[j][t / C::SPL][2 * (t % C::SPL) + e];
+                    o[2 * e] = (as_h2(__builtin_amdgcn_perm(0x64646464u, w, 0x04010400u)) + gcj[0].zz) * gcj[0].s;
+                    o[2 * e + 1] = (as_h2(__builtin_amdgcn_perm(0x64646464u, w, 0x04030402u)) + gcj[0].zz) * gcj[0].s;
+                }
+            }
+            return pack_h8(o);
+        } else {
+            return unpack_step<BITS>(ws.w[j][t / C::SPL], t % C::SPL, gcj, C::WPG);
+        }
     };
 
     // One K step.  The 32 MFMAs of MFMA step t are issued in groups of 4 (one m-tile); between two groups
@@ -262,7 +311,7 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
     // count is exact.
     // `ph` (META4 only): position of the step in its run of four, a constant after inlining.
     static_assert(C::MF % 2 == 0, "the fragment double buffer returns to slot 0 at the end of a step");
-    using GC = GroupConst<BITS>;
+    using GC = std::conditional_t<MT == 16, GroupConstNat<BITS>, GroupConst<BITS>>;
     h8 xf[C::XB][C::XRING];
     h2 wf[2][NT][4];                                      // weight fragments as 4 register pairs each
     // group constants of tile j for the step that reads `from` (META4: half `half` of m_cur / m_next)
@@ -281,8 +330,7 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
                 gj[g].set(__builtin_bit_cast(_Float16, (uint16_t)from.s[j][g]), __builtin_bit_cast(_Float16, (uint16_t)from.z[j][g]));
         }
     };
-    auto step8 = [&](int c, const _Float16* cur, _Float16* nxt, WSet& ws, const WSet& wsn, GC (&gc)[NT][C::NG],
-                    GC (&gn)[NT][C::NG], const int ph) {
+    auto step8 = [&](int c, const _Float16* cur, _Float16* nxt, WSet& ws, const WSet& wsn, auto& gc, auto& gn, const int ph) {
         __builtin_amdgcn_sched_barrier(0);
         const _Float16* xp = cur + nl * C::PITCH + kq * C::VPL;
 #pragma unroll
@@ -417,41 +465,57 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
     // and wait instructions cost 1-2 each).  So the side work of an MFMA step is cut into single instructions and dealt
     // out one per gap, by position: gap g = 4 i + j follows the MFMA of m-tile i and n-tile j; region r = g / 16 and
     // k = g % 16 name the 16 gaps of four slots.
-    //   unpack    : n-tile r's fragment for the next MFMA step, 12-13 instructions, one in each of k = 0..12
-    //               (the last MFMA step prepares the first fragment of the next K step from the other register set);
-    //   staging   : unit u = 4 t + r of the next chunk, requested two MFMA steps earlier: permutes at k = 0, 2, 4, 6,
-    //               LDS write at k = 8, address at k = 10 and the request of unit u + 8 (of this chunk, or of the one
-    //               after it) into the same registers at k = 12;
-    //   fragments : slot i's last gap reads the activation fragment of slot i + 8 into the ring;
-    //   requests  : scales / zero points at k = 14, 15 of the second MFMA step, weights at k = 14, 15 of the last,
-    //               group constants of the next step at k = 13 of the last but one.
+    //   unpack      : n-tile r's fragment for the next MFMA step, one instruction in each of k = 0..15 (4 bits; 0..11 at
+    //                 8 bits); the last MFMA step prepares the first fragment of the next K step from the other set;
+    //   activations : the next chunk's 256 x 128 tile goes memory -> LDS by buffer loads with LDS destination, 16 per
+    //                 wave (4 rows of 256 bytes each), all issued in the first MFMA step so that they have three more
+    //                 to land; no registers, no permute, and nothing the matrix pipe waits for;
+    //   fragments   : slot i's last gap reads the activation fragment of slot i + 8 into the ring;
+    //   requests    : scales / zero points at k = 14, 15 of the second MFMA step, weights at k = 14, 15 of the last,
+    //                 group constants of the next step at k = 13 of the last but one.
+    // LDS row r of a buffer holds the chunk's 16-byte slot q of x row r at slot q ^ (r & 7): a lane group of 16 rows
+    // reading one slot then spreads over all banks (rows are 256 bytes apart: unswizzled they would share 4 banks).
+    // The fragment reads are written as assembly: the compiler orders every LDS read it knows of behind all pending
+    // loads with LDS destination, and would so wait for the next chunk before reading this one.  It does not track
+    // assembly results either, so the waits are here too: fragment reads complete in order and nothing else uses LDS
+    // in the loop, so before slot S of a K step (S = 16 t + i) at most 7 - max(0, S - 56) younger reads are in flight.
     // Request addresses are one VGPR per thread plus a scalar: the chunk part of an offset is uniform, and past the
     // slice it is replaced by an offset beyond every buffer, so that the hardware's range check returns zeros.
     // Requires K % CHUNK_K == 0 (the launcher's condition for this variant): no request straddles the end of a row.
     h2 up[NT][4];
-    uint32_t uw[NT];
-    uint32_t xo[4];
-    auto x_req16 = [&](int u, int cc) {
-        const uint32_t so = cc < c_end ? (uint32_t)u * x_pitch + (uint32_t)cc * C::CHUNK_K * 2 : kOob;
-        return x_base + so;
+    uint32_t uw[NT], pq[NT][2];
+    const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+    // activation loads: unit u of a wave = rows 64 wave + 4 u + (lane >> 4), lane & 15 = LDS slot
+    uint32_t xd_base[2];
+#pragma unroll
+    for (int par = 0; par < 2; par++) {
+        const int rr = 4 * par + (lane >> 4);
+        xd_base[par] = (uint32_t)((m0 + 64 * wave + rr) * a.ldx) * 2 + (((lane & 15) ^ (rr & 7)) * 16);
+    }
+    auto x_dma16 = [&](int u, int cc, char* buf) {
+        uint32_t so = cc < c_end ? (uint32_t)((u >> 1) * 8 * a.ldx) * 2 + (uint32_t)cc * C::CHUNK_K * 2 : kOob;
+        asm("" : "+s"(so));                                   // one scalar sum, one VALU add
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, (__attribute__((address_space(3))) void*)(buf + (64 * wave_u + 4 * u) * 256), 16,
+                                                 xd_base[u & 1] + so, 0, 0, 0);
     };
     auto w_req16 = [&](int j, int l, int cc, WSet& ws) {
         const uint32_t so = cc < c_end ? (uint32_t)cc * C::CHUNK_BYTES + l * 16 : kOob;
         ws.w[j][l] = __builtin_amdgcn_raw_buffer_load_b128(rw, w_off[j] + so, 0, 0);
     };
-    auto x_load16 = [&](int u, uint32_t off) {
-        const int r = (u % C::XR) * C::UW;
+    // fragment (m-tile i, MFMA step t) of the lane: slot 4 kq + t of row 16 i + nl, swizzled
+    uint32_t fa[4];
 #pragma unroll
-        for (int j = 0; j < C::UW; j++) xr[r + j] = __builtin_amdgcn_raw_buffer_load_b128(rx, off + j * 16, 0, 0);
-    };
-    auto step16 = [&](int c, const _Float16* cur, _Float16* nxt, WSet& ws, const WSet& wsn, GC (&gc)[NT][C::NG],
-                      GC (&gn)[NT][C::NG], const int ph) {
-        static_assert(MT != 16 || (C::NG == 1 && C::UW == 1 && C::XR == 8 && C::MF == 4), "layout of the 256-row schedule");
+    for (int t = 0; t < 4; t++) fa[t] = (uint32_t)(nl * 256 + (((4 * kq + t) ^ (nl & 7)) * 16));
+    auto step16 = [&](int c, const char* cur, char* nxt, WSet& ws, const WSet& wsn, auto& gc, auto& gn, const int ph) {
+        static_assert(MT != 16 || (C::NG == 1 && C::MF == 4 && C::CHUNK_K == 128 && C::XRING == 8), "layout of the 256-row schedule");
         __builtin_amdgcn_sched_barrier(0);
-        const _Float16* xp = cur + nl * C::PITCH + kq * C::VPL;
-#pragma unroll
-        for (int i = 0; i < C::XRING; i++) xf[0][i] = *reinterpret_cast<const h8*>(xp + i * 16 * C::PITCH);
-        const h2 k16 = splat((_Float16)0.0625f);
+        const uint32_t cur_a = (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) char*)cur;
+        auto frag_read = [&](auto tc, auto ic) {
+            constexpr int t = decltype(tc)::value, i = decltype(ic)::value;
+            lds_read_b128<i * 16 * 256>(xf[0][i % C::XRING], cur_a + fa[t]);
+        };
+        static_for<0, C::XRING>([&](auto ic) { frag_read(std::integral_constant<int, 0>{}, ic); });
+        const h2 k16 = h2{(_Float16)1.0f, (_Float16)0.0625f};
         static_for<0, C::MF>([&](auto tc) {
             constexpr int t = decltype(tc)::value, cu = t & 1, nx = cu ^ 1;
             constexpr bool early = t == C::MF - 1;
@@ -459,92 +523,103 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
             constexpr int tt = early ? 0 : t + 1;
             static_for<0, 4 * MT>([&](auto gcnt) {
                 constexpr int g = decltype(gcnt)::value, i = g / NT, j = g % NT, r = g / 16, k = g % 16;
+                constexpr int S = 16 * t + i;
                 __builtin_amdgcn_sched_barrier(0);
+                if constexpr (j == 0) __builtin_amdgcn_s_waitcnt(0xC07F | ((7 - (S > 56 ? S - 56 : 0)) << 8));
                 mfma_acc(acc[i][j], pack_h8(wf[cu][j]), xf[0][i % C::XRING]);
                 __builtin_amdgcn_sched_barrier(0);
                 // ---- unpack of n-tile r ----
-                const GC& gr = early ? gn[r][0] : gc[r][0];
+                const auto& gr = early ? gn[r][0] : gc[r][0];
                 if constexpr (BITS == 4) {
                     const uint32_t word = src.w[r][0][tt];
-                    if (k == 0) up[r][0] = as_h2(and_or(word, 0x000F000Fu, kMagic));
-                    if (k == 1) up[r][1] = as_h2(and_or(word, 0x00F000F0u, kMagic));
-                    if (k == 2) up[r][0] = up[r][0] + gr.z0;
-                    if (k == 3) up[r][1] = __builtin_elementwise_fma(up[r][1], k16, gr.z1);
-                    if (k == 4) wf[nx][r][0] = up[r][0] * gr.s;
-                    if (k == 5) wf[nx][r][1] = up[r][1] * gr.s;
-                    if (k == 6) uw[r] = word >> 8;
-                    if (k == 7) up[r][2] = as_h2(and_or(uw[r], 0x000F000Fu, kMagic));
-                    if (k == 8) up[r][3] = as_h2(and_or(uw[r], 0x00F000F0u, kMagic));
-                    if (k == 9) up[r][2] = up[r][2] + gr.z0;
-                    if (k == 10) up[r][3] = __builtin_elementwise_fma(up[r][3], k16, gr.z1);
-                    if (k == 11) wf[nx][r][2] = up[r][2] * gr.s;
-                    if (k == 12) wf[nx][r][3] = up[r][3] * gr.s;
+                    if constexpr (k == 0) pq[r][0] = __builtin_amdgcn_perm(word, word, 0x01000100u);
+                    if constexpr (k == 1) pq[r][1] = __builtin_amdgcn_perm(word, word, 0x03020302u);
+                    if constexpr (k == 2) up[r][0] = as_h2(and_or(pq[r][0], 0x00F0000Fu, kMagic));
+                    if constexpr (k == 3) uw[r] = pq[r][0] >> 8;
+                    if constexpr (k == 4) up[r][1] = as_h2(and_or(uw[r], 0x00F0000Fu, kMagic));
+                    if constexpr (k == 5) up[r][2] = as_h2(and_or(pq[r][1], 0x00F0000Fu, kMagic));
+                    if constexpr (k == 6) uw[r] = pq[r][1] >> 8;
+                    if constexpr (k == 7) up[r][3] = as_h2(and_or(uw[r], 0x00F0000Fu, kMagic));
+                    if constexpr (k >= 8 && k < 12) up[r][k - 8] = __builtin_elementwise_fma(up[r][k - 8], k16, gr.zz);
+                    if constexpr (k >= 12) wf[nx][r][k - 12] = up[r][k - 12] * gr.s;
                 } else {
                     // 8 bits: the two words of MFMA step tt are words 2 (tt % 2), + 1 of lane load tt / 2
                     const uint32_t w0 = src.w[r][tt / C::SPL][2 * (tt % C::SPL)], w1 = src.w[r][tt / C::SPL][2 * (tt % C::SPL) + 1];
-                    if (k == 0) up[r][0] = as_h2(__builtin_amdgcn_perm(0x64646464u, w0, 0x04010400u));
-                    if (k == 1) up[r][1] = as_h2(__builtin_amdgcn_perm(0x64646464u, w0, 0x04030402u));
-                    if (k == 2) up[r][0] = up[r][0] + gr.z0;
-                    if (k == 3) up[r][1] = up[r][1] + gr.z0;
-                    if (k == 4) wf[nx][r][0] = up[r][0] * gr.s;
-                    if (k == 5) wf[nx][r][1] = up[r][1] * gr.s;
-                    if (k == 6) up[r][2] = as_h2(__builtin_amdgcn_perm(0x64646464u, w1, 0x04010400u));
-                    if (k == 7) up[r][3] = as_h2(__builtin_amdgcn_perm(0x64646464u, w1, 0x04030402u));
-                    if (k == 8) up[r][2] = up[r][2] + gr.z0;
-                    if (k == 9) up[r][3] = up[r][3] + gr.z0;
-                    if (k == 10) wf[nx][r][2] = up[r][2] * gr.s;
-                    if (k == 11) wf[nx][r][3] = up[r][3] * gr.s;
+                    if constexpr (k == 0) up[r][0] = as_h2(__builtin_amdgcn_perm(0x64646464u, w0, 0x04010400u));
+                    if constexpr (k == 1) up[r][1] = as_h2(__builtin_amdgcn_perm(0x64646464u, w0, 0x04030402u));
+                    if constexpr (k == 2) up[r][2] = as_h2(__builtin_amdgcn_perm(0x64646464u, w1, 0x04010400u));
+                    if constexpr (k == 3) up[r][3] = as_h2(__builtin_amdgcn_perm(0x64646464u, w1, 0x04030402u));
+                    if constexpr (k >= 4 && k < 8) up[r][k - 4] = up[r][k - 4] + gr.zz;
+                    if constexpr (k >= 8 && k < 12) wf[nx][r][k - 8] = up[r][k - 8] * gr.s;
                 }
-                // ---- staging of unit u, then the request of unit u + 8 ----
-                {
-                    const int u = 4 * t + r, rs = u % C::XR;
-                    if constexpr (BITS == 4) {
-                        if (k == 0) xo[0] = __builtin_amdgcn_perm(xr[rs][2], xr[rs][0], 0x05040100u);
-                        if (k == 2) xo[1] = __builtin_amdgcn_perm(xr[rs][2], xr[rs][0], 0x07060302u);
-                        if (k == 4) xo[2] = __builtin_amdgcn_perm(xr[rs][3], xr[rs][1], 0x05040100u);
-                        if (k == 6) xo[3] = __builtin_amdgcn_perm(xr[rs][3], xr[rs][1], 0x07060302u);
-                    }
-                    if (k == 8) {
-                        u4* dst = reinterpret_cast<u4*>(nxt + (tid / C::UPR + u * RPI) * C::PITCH + x_ku * C::UNIT);
-                        if constexpr (BITS == 4) *dst = u4{xo[0], xo[1], xo[2], xo[3]};
-                        else *dst = xr[rs];
-                    }
-                    const int u2 = (u + 8) % C::XL, c2 = c + 1 + (u + 8) / C::XL;
-                    if (k == 10) xo[0] = x_req16(u2, c2);
-                    if (k == 12) x_load16(u2, xo[0]);
-                }
+                // ---- the next chunk's activations: unit u at gap 3 u + 1 of the first MFMA step ----
+                if constexpr (t == 0 && g % 3 == 1 && g / 3 < 16) x_dma16(g / 3, c + 1, nxt);
                 // ---- fragment ring ----
-                if (j == NT - 1) {
-                    const int i2 = (i + C::XRING) % MT, t2 = t + (i + C::XRING) / MT;
-                    if (t2 < C::MF) xf[0][i % C::XRING] = *reinterpret_cast<const h8*>(xp + i2 * 16 * C::PITCH + 8 * t2);
+                if constexpr (j == NT - 1) {
+                    constexpr int i2 = (i + C::XRING) % MT, t2 = t + (i + C::XRING) / MT;
+                    if constexpr (t2 < C::MF) frag_read(std::integral_constant<int, t2>{}, std::integral_constant<int, i2>{});
                 }
                 // ---- requests and constants ----
-                if (t == 1 && k >= 14) {
+                if constexpr (t == 1 && k >= 14) {
                     if constexpr (META4) {
                         if (ph == 0) issue_meta4(r, k - 14, c + C::SPR, m_next);
                     } else {
                         issue_meta(r, k - 14, c + 2, ws);
                     }
                 }
-                if (t == C::MF - 2 && k == 13) {
+                if constexpr (t == C::MF - 2 && k == 13) {
                     if constexpr (META4) set_consts(gn[r], r, wsn, ph < C::SPR - 1 ? m_cur : m_next, ph < C::SPR - 1 ? ph + 1 : 0);
                     else set_consts(gn[r], r, wsn, m_cur, 0);
                 }
-                if (t == C::MF - 1 && k >= 16 - C::WL) w_req16(r, k - (16 - C::WL), c + 2, ws);
+                if constexpr (t == C::MF - 1 && k >= 16 - C::WL) w_req16(r, k - (16 - C::WL), c + 2, ws);
                 asm volatile("" ::: "memory");
             });
         });
         __builtin_amdgcn_sched_barrier(0);
-        __syncthreads();
+        // this wave's rows of the next chunk are in LDS once only the requests made after them are still in flight:
+        // the weights of the last MFMA step and, in a step that made them, the scales and zero points
+        if ((META4 && ph != 0)) wait_loads<NT * C::WL>();
+        else wait_loads<NT * C::WL + 2 * NT>();
+        lds_barrier();
     };
-    auto step = [&](int c, const _Float16* cur, _Float16* nxt, WSet& ws, const WSet& wsn, GC (&gc)[NT][C::NG], GC (&gn)[NT][C::NG],
+    auto step = [&](int c, _Float16* cur, _Float16* nxt, WSet& ws, const WSet& wsn, GC (&gc)[NT][C::NG], GC (&gn)[NT][C::NG],
                     const int ph) {
-        if constexpr (MT == 16) step16(c, cur, nxt, ws, wsn, gc, gn, ph);
+        if constexpr (MT == 16) step16(c, reinterpret_cast<const char*>(cur), reinterpret_cast<char*>(nxt), ws, wsn, gc, gn, ph);
         else step8(c, cur, nxt, ws, wsn, gc, gn, ph);
     };
 
     _Float16* buf0 = reinterpret_cast<_Float16*>(smem);
     _Float16* buf1 = reinterpret_cast<_Float16*>(smem + C::STAGE_BYTES);
+    if constexpr (MT == 16) {
+        // Prologue of the 256-row tile: chunk c_begin's activations to the first buffer; scales and zero points and
+        // the weights of the first two chunks in the order a steady-state step finds them outstanding.
+        if constexpr (META4) {
+#pragma unroll
+            for (int j = 0; j < NT; j++) {
+                issue_meta4(j, 0, c_begin, m_cur);
+                issue_meta4(j, 1, c_begin, m_cur);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < 16; u++) x_dma16(u, c_begin, smem);
+#pragma unroll
+        for (int b = 0; b < 2; b++) {
+            WSet& ws = b ? set1 : set0;
+            if constexpr (!META4) {
+#pragma unroll
+                for (int j = 0; j < NT; j++) {
+                    issue_meta(j, 0, c_begin + b, ws);
+                    issue_meta(j, 1, c_begin + b, ws);
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < NT; j++)
+#pragma unroll
+                for (int l = 0; l < C::WL; l++) w_req16(j, l, c_begin + b, ws);
+            asm volatile("" ::: "memory");
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    } else {
     // Prologue: the same two request batches, in the same order, that a steady-state step finds
     // outstanding - the compiler merges the wait counts of the loop entry with those of the back edge, and
     // any difference in order makes the steady state wait for requests it has only just issued.
@@ -592,33 +667,7 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
     }
     __builtin_amdgcn_sched_barrier(0);
     // second batch in the order of a steady-state step
-    if constexpr (MT == 16) {
-        if constexpr (!META4) {
-#pragma unroll
-            for (int j = 0; j < NT; j++) {
-                issue_meta(j, 0, c_begin + 1, set1);
-                issue_meta(j, 1, c_begin + 1, set1);
-                asm volatile("" ::: "memory");
-                __builtin_amdgcn_sched_barrier(0);
-            }
-        }
-#pragma unroll
-        for (int u = 0; u < 4; u++) {
-            x_load16(u, x_req16(u, c_begin + 1));
-            asm volatile("" ::: "memory");
-            __builtin_amdgcn_sched_barrier(0);
-        }
-#pragma unroll
-        for (int j = 0; j < NT; j++) {
-            x_load16(4 + j, x_req16(4 + j, c_begin + 1));
-            asm volatile("" ::: "memory");
-            __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-            for (int l = 0; l < C::WL; l++) w_req16(j, l, c_begin + 1, set1);
-            asm volatile("" ::: "memory");
-            __builtin_amdgcn_sched_barrier(0);
-        }
-    } else if constexpr (C::T_STAGE == 0 || C::PH == 2) {
+    if constexpr (C::T_STAGE == 0 || C::PH == 2) {
         issue_batch(c_begin + 1, set1);
     } else {
     if constexpr (!META4) {
@@ -638,6 +687,7 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
         __builtin_amdgcn_sched_barrier(0);
     }
     }
+    }
     GC gc0[NT][C::NG], gc1[NT][C::NG];
 #pragma unroll
     for (int j = 0; j < NT; j++) {
@@ -646,7 +696,12 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
 #pragma unroll
         for (int e = 0; e < 4; e++) wf[0][j][e] = h2{f[2 * e], f[2 * e + 1]};
     }
-    __syncthreads();
+    if constexpr (MT == 16) {
+        wait_loads<NT * C::WL + (META4 ? 0 : 2 * NT)>();       // all but the second chunk's requests: the first buffer is written
+        lds_barrier();
+    } else {
+        __syncthreads();
+    }
     if constexpr (META4 && C::SPR == 2) {
         for (int c = c_begin; c < c_end; c += 2) {   // runs of two steps = one request; an odd count runs one step on zeros
             step(c, buf0, buf1, set0, set1, gc0, gc1, 0);

@@ -688,23 +688,6 @@ struct WeightTile {
     }
 };
 
-// Workgroup barrier for LDS data that ordinary stores of this wave wrote: waits for the wave's own LDS operations and
-// then for the other waves, without the memory fence of __syncthreads() - a fence would also wait for every weight
-// request in flight, since those land in LDS too.
-BW_DEV void lds_barrier() {
-    asm volatile("" ::: "memory");
-    __builtin_amdgcn_s_waitcnt(0xC07F);                   // lgkmcnt(0)
-    __builtin_amdgcn_s_barrier();
-    asm volatile("" ::: "memory");
-}
-
-// wait until at most `n` of this wave's memory loads are outstanding (loads return in order)
-template <int N>
-BW_DEV void wait_loads() {
-    static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
-    __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | 0x0F70);   // expcnt and lgkmcnt left alone
-}
-
 // ---- 4-bit, M <= 2: integer operands, scale and zero point taken out of the inner loop -------------------
 //
 // A masked packed word is already a float16: bits 0-3 of a half are the subnormal q * 2^-24, bits 4-7 the
