@@ -60,6 +60,16 @@ def time_calls(torch, fn, iters, warmup):
     return e0.elapsed_time(e1) * 1e3 / iters      # us per call
 
 
+def time_alternating(torch, fns, iters, warmup, rounds=3):
+    """Median over `rounds` of time_calls for each of `fns`, the functions taking turns within a round: clocks and
+    power state drift over a run of large GEMMs, and a figure and the one it is compared with should see the same drift."""
+    for fn in fns:
+        for _ in range(warmup):
+            fn()
+    runs = [[time_calls(torch, fn, iters, 2) for fn in fns] for _ in range(rounds)]
+    return [sorted(r[i] for r in runs)[rounds // 2] for i in range(len(fns))]
+
+
 def graph_of(torch, fn):
     g = torch.cuda.CUDAGraph()
     s = torch.cuda.Stream()
@@ -275,21 +285,25 @@ def extras_hipblaslt_decode(torch, hip, QuantizedLinear, layers):
 
 def extras_prefill(torch, hip, QuantizedLinear, layers):
     """Prefill on the Llama-3-8B MLP shapes, W4 g128, next to fp16 hipBLASLt on the dequantised weights.  `us` is
-    the kernel on float16 x; `bf16_x_us` the forward on bfloat16 x (cast + split-K workspace + kernel)."""
+    the kernel on float16 x; `bf16_x_us` the forward on bfloat16 x (cast + split-K workspace + kernel); `tile_rows` the
+    output tile the library picked (128 or 256 rows).  Every figure is the median of three rounds in which the kernels
+    take turns."""
     bits, g, out = 4, 128, {}
     for k, n in ((4096, 14336), (14336, 4096)):
         q = make_layer(torch, QuantizedLinear, k, n, bits, g, seed=7)
         w16 = hip.dequantize(q.qweight, q.scale, q.zero_point, g, bits, torch.float16)
         for mm in (128, 512, 2048):
             x = torch.randn(mm, k, device="cuda", dtype=torch.float16)
-            us_q = time_calls(torch, lambda: hip.quantized_gemm_hip(x, q.qweight, q.scale, q.zero_point, None, bits, g), 20, 5)
-            us_b = time_calls(torch, lambda: torch.matmul(x, w16.T), 20, 5)
             # the configuration names bfloat16 activations: the reference's forward casts them to float16
             # (bitween/modules.py:74) and so does this one, in a pass of its own ahead of the prefill kernel
             xb = x.to(torch.bfloat16)
-            us_qb = time_calls(torch, lambda: hip.quantized_matmul_hip(xb, q.qweight, q.scale, q.zero_point, None, bits, g), 20, 5)
+            us_q, us_b, us_qb = time_alternating(torch, [
+                lambda: hip.quantized_gemm_hip(x, q.qweight, q.scale, q.zero_point, None, bits, g),
+                lambda: torch.matmul(x, w16.T),
+                lambda: hip.quantized_matmul_hip(xb, q.qweight, q.scale, q.zero_point, None, bits, g)], 20, 10)
             fl = 2.0 * mm * n * k
             out[f"{k}x{n}_M{mm}"] = {"us": round(us_q, 1), "bf16_x_us": round(us_qb, 1), "TFLOPs": round(fl / us_q / 1e6, 1),
+                                     "tile_rows": hip.load().bw_qgemm_tile_rows(mm, n, k, bits, g),
                                      "pct_mfma_f16_peak": round(100 * fl / us_q / 1e6 / MFMA_F16_PEAK_TFLOPS, 1),
                                      "hipblaslt_fp16_us": round(us_b, 1), "hipblaslt_fp16_TFLOPs": round(fl / us_b / 1e6, 1),
                                      "frac_of_hipblaslt": round(us_b / us_q, 3)}
@@ -306,12 +320,13 @@ def extras_prefill_other_formats(torch, hip, QuantizedLinear, layers):
         w16 = hip.dequantize(q.qweight, q.scale, q.zero_point, g, bits, torch.float16)
         for mm in (512, 2048):
             x = torch.randn(mm, k, device="cuda", dtype=torch.float16)
-            # 60 untimed calls first: the first large GEMMs of a fresh process run ~18 % slow (clocks, first touch of
-            # the workspace), whichever kernel they are
-            us_q = time_calls(torch, lambda: hip.quantized_gemm_hip(x, q.qweight, q.scale, q.zero_point, None, bits, g), 20, 60)
-            us_b = time_calls(torch, lambda: torch.matmul(x, w16.T), 20, 20)
+            # 30 untimed calls of each first: the first large GEMMs of a fresh process run ~18 % slow (clocks, first touch
+            # of the workspace), whichever kernel they are
+            us_q, us_b = time_alternating(torch, [lambda: hip.quantized_gemm_hip(x, q.qweight, q.scale, q.zero_point, None, bits, g),
+                                                  lambda: torch.matmul(x, w16.T)], 20, 30)
             fl = 2.0 * mm * n * k
             out[f"w{bits}g{g}_{k}x{n}_M{mm}"] = {"us": round(us_q, 1), "TFLOPs": round(fl / us_q / 1e6, 1),
+                                                 "tile_rows": hip.load().bw_qgemm_tile_rows(mm, n, k, bits, g),
                                                  "hipblaslt_fp16_us": round(us_b, 1), "frac_of_hipblaslt": round(us_b / us_q, 3)}
         del q, w16
     return out

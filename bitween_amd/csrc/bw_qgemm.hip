@@ -12,6 +12,11 @@
 //   * activations go global -> LDS once per workgroup (double buffered,
 //     permuted into the k order the unpack emits) and every A fragment read
 //     from LDS feeds 4 MFMAs.
+// Grids that fill the device run the same kernel with 256 x 256 tiles at 4 and
+// 8 bits (a wave owns 256 x 64: all 256 accumulation registers): every weight
+// is unpacked once for twice the rows, the activations go memory -> LDS
+// without passing through registers, and the side work of an MFMA step is
+// dealt out one instruction per MFMA (step16 below).
 // Also holds the shape-generic fallback used when the fast layouts do not
 // apply (odd K or group size): correct for everything the reference accepts.
 #include "bw_common.h"
@@ -57,20 +62,11 @@ struct GemmCfg {
     static constexpr int UNIT = VPI > 8 ? VPI : 8;               // halves permuted together when staging x
     static constexpr int UW = UNIT / 8;
     static constexpr int UPR = CHUNK_K / UNIT;                   // staging units per x row
-    static constexpr int XL = BM * UPR / (WAVES * 64);           // staging units per thread
+    static constexpr int XL = BM * UPR / (WAVES * 64);           // staging units per thread (128-row tiles)
     static_assert(BM * UPR % (WAVES * 64) == 0, "tile must split evenly over the workgroup");
-    // The staging units of a thread pass through XR register sets in PH phases per K step, each phase in an MFMA
-    // step of its own: phase p writes its units of chunk c+1 to LDS (slots SLOT0[p] .. SLOT0[p] + XR - 1 of MFMA step
-    // STAGE_T[p]) and requests the units of the phase after it into the same registers.  One phase for 128 rows;
-    // two for 256 rows, two MFMA steps apart, so that a request has two steps (2 x 64 MFMAs) to land.
-    static constexpr int XR = XL > 8 ? 8 : XL, PH = XL / XR;
-    static_assert(XL % XR == 0 && PH <= 2, "staging phases");
-    static constexpr int STAGE_T0 = PH == 1 ? T_STAGE : (BITS == 4 ? 1 : 0), STAGE_T1 = PH == 1 ? -1 : (BITS == 4 ? 3 : 2);
-    static constexpr int SLOT0_0 = (PH == 2 && BITS == 4) ? 8 : 0, SLOT0_1 = 0;
     // Activation fragments in registers: 128 rows - two sets of MT, the set of MFMA step t+1 read during step t;
-    // 256 rows - a ring of XRING, the fragment of slot i + XRING read when slot i has issued its MFMAs (256 cycles of
-    // matrix work ahead of its use).
-    static constexpr int XB = MT == 8 ? 2 : 1, XRING = MT == 8 ? MT : 8;
+    // 256 rows - a ring of 8, the fragment of slot i + 8 read when slot i has issued its MFMAs.
+    static constexpr int XSETS = MT == 8 ? 2 : 1, XRING = MT == 8 ? MT : 8;
 };
 
 template <int BITS>
@@ -210,21 +206,15 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
         w_off[j] = row < a.N ? (uint32_t)row * a.row_bytes + kq * 16 * C::WL : MT == 16 ? (uint32_t)(a.N - 1) * a.row_bytes + kq * 16 * C::WL : kOob;
         m_off[j] = (uint32_t)min(row, a.N - 1) * groups * 2;
     }
-    // Staging unit i of a thread: row tid / UPR + i * RPI of the tile, the thread's UNIT-wide column ku of the chunk.
-    // 128-row tiles keep the byte offsets of their units in registers; 256-row tiles, which have none to spare, form
-    // them from the first (rows past M then lie past the end of x and are range-checked to zero by the hardware; the
-    // launcher checks that (M + 256) * ldx * 2 fits 32 bits).
-    static_assert((WAVES * 64) % C::UPR == 0, "a thread's staging units share one column");
-    constexpr int RPI = WAVES * 64 / C::UPR;
-    const int x_ku = tid % C::UPR;
-    const uint32_t x_base = (uint32_t)((m0 + tid / C::UPR) * a.ldx + x_ku * C::UNIT) * 2, x_pitch = (uint32_t)(RPI * a.ldx) * 2;
-    uint32_t x_off[C::PH == 1 ? C::XL : 1];
-    if constexpr (C::PH == 1) {
+    // 128-row tiles: byte offsets of the staging units of a thread
+    uint32_t x_off[C::XL];
 #pragma unroll
-        for (int i = 0; i < C::XL; i++) x_off[i] = (m0 + tid / C::UPR + i * RPI < a.M) ? x_base + i * x_pitch : kOob;
+    for (int i = 0; i < C::XL; i++) {
+        const int u = tid + i * WAVES * 64, m = u / C::UPR, ku = u - m * C::UPR;
+        x_off[i] = (m0 + m < a.M) ? (uint32_t)((m0 + m) * a.ldx + ku * C::UNIT) * 2 : kOob;
     }
 
-    u4 xr[C::XR * C::UW];
+    u4 xr[C::XL * C::UW];
     // Two weight register sets, used alternately by even and odd K steps and never copied: a register move
     // of an outstanding load would stall on it.
     struct WSet { u4 w[NT][C::WL]; uint32_t s[NT][C::NG], z[NT][C::NG]; };   // 16-bit values, one register each
@@ -238,24 +228,21 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
         for (int j = 0; j < NT; j++) acc[i][j] = f4{0.f, 0.f, 0.f, 0.f};
 
     // Pieces of the staging / issue work, one per m-tile index, so they can be slotted between MFMA groups.
-    static_assert(C::XR <= MT && MT % (NT * 2) == 0, "at most one staging unit and half a weight tile per m-tile slot");
-    // unit i travels in register set i % XR
     auto stage_unit = [&](int i, _Float16* xs) {
-        const int m = tid / C::UPR + i * RPI, r = (i % C::XR) * C::UW;
+        const int u = tid + i * WAVES * 64, m = u / C::UPR, ku = u - m * C::UPR;
         uint32_t in[4 * C::UW], o[4 * C::UW];
 #pragma unroll
-        for (int j = 0; j < C::UW; j++) { in[4 * j] = xr[r + j][0]; in[4 * j + 1] = xr[r + j][1]; in[4 * j + 2] = xr[r + j][2]; in[4 * j + 3] = xr[r + j][3]; }
+        for (int j = 0; j < C::UW; j++) { in[4 * j] = xr[i * C::UW + j][0]; in[4 * j + 1] = xr[i * C::UW + j][1]; in[4 * j + 2] = xr[i * C::UW + j][2]; in[4 * j + 3] = xr[i * C::UW + j][3]; }
         permute_unit<BITS>(in, o);
-        u4* dst = reinterpret_cast<u4*>(xs + m * C::PITCH + x_ku * C::UNIT);
+        u4* dst = reinterpret_cast<u4*>(xs + m * C::PITCH + ku * C::UNIT);
 #pragma unroll
         for (int j = 0; j < C::UW; j++) dst[j] = u4{o[4 * j], o[4 * j + 1], o[4 * j + 2], o[4 * j + 3]};
     };
     auto issue_x_unit = [&](int i, int c) {
-        const uint32_t row_off = C::PH == 1 ? x_off[C::PH == 1 ? i : 0] : x_base + i * x_pitch;
-        const uint32_t off = (c < c_end && c * C::CHUNK_K + x_ku * C::UNIT < a.K) ? row_off + (uint32_t)c * C::CHUNK_K * 2 : kOob;
-        const int r = (i % C::XR) * C::UW;
+        const int ku = (tid + i * WAVES * 64) % C::UPR;
+        const uint32_t off = (c < c_end && c * C::CHUNK_K + ku * C::UNIT < a.K) ? x_off[i] + (uint32_t)c * C::CHUNK_K * 2 : kOob;
 #pragma unroll
-        for (int j = 0; j < C::UW; j++) xr[r + j] = __builtin_amdgcn_raw_buffer_load_b128(rx, off + j * 16, 0, 0);
+        for (int j = 0; j < C::UW; j++) xr[i * C::UW + j] = __builtin_amdgcn_raw_buffer_load_b128(rx, off + j * 16, 0, 0);
     };
     auto issue_w_load = [&](int j, int l, int c, WSet& ws) {
         const int b = c * C::CHUNK_BYTES + l * 16;
@@ -312,7 +299,7 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
     // `ph` (META4 only): position of the step in its run of four, a constant after inlining.
     static_assert(C::MF % 2 == 0, "the fragment double buffer returns to slot 0 at the end of a step");
     using GC = std::conditional_t<MT == 16, GroupConstNat<BITS>, GroupConst<BITS>>;
-    h8 xf[C::XB][C::XRING];
+    h8 xf[C::XSETS][C::XRING];
     h2 wf[2][NT][4];                                      // weight fragments as 4 register pairs each
     // group constants of tile j for the step that reads `from` (META4: half `half` of m_cur / m_next)
     auto set_consts = [&](GC* gj, int j, const WSet& from, const u2 (*m)[2], int half) {
@@ -331,20 +318,11 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
         }
     };
     auto step8 = [&](int c, const _Float16* cur, _Float16* nxt, WSet& ws, const WSet& wsn, auto& gc, auto& gn, const int ph) {
+        static_assert(C::XL <= MT && NT * 2 == MT, "at most one staging unit and half a weight tile per m-tile slot");
         __builtin_amdgcn_sched_barrier(0);
         const _Float16* xp = cur + nl * C::PITCH + kq * C::VPL;
 #pragma unroll
-        for (int i = 0; i < C::XRING; i++) xf[0][i] = *reinterpret_cast<const h8*>(xp + i * 16 * C::PITCH);
-        // fragment of m-tile i for MFMA step t sits in xf[xc][i % XRING]; next_frag(t, i): the read issued from slot i
-        auto next_frag = [&](int t, int i) {
-            if constexpr (C::XB == 2) {
-                if (t < C::MF - 1) xf[(t & 1) ^ 1][i] = *reinterpret_cast<const h8*>(xp + i * 16 * C::PITCH + 8 * (t + 1));
-            } else {
-                const int i2 = (i + C::XRING) % MT, t2 = t + (i + C::XRING) / MT;
-                if (t2 < C::MF) xf[0][i % C::XRING] = *reinterpret_cast<const h8*>(xp + i2 * 16 * C::PITCH + 8 * t2);
-            }
-        };
-        constexpr int SPP = MT / (2 * NT);                // slots per half weight tile: work sits in the first of them
+        for (int i = 0; i < MT; i++) xf[0][i] = *reinterpret_cast<const h8*>(xp + i * 16 * C::PITCH);
         if constexpr (!C::EARLY_W) {
 #pragma unroll
             for (int j = 0; j < NT; j++) {
@@ -363,26 +341,15 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
         auto slot_requests = [&](int t, int i) {
             static_assert(C::MF >= 4, "second and last MFMA step are distinct");
             if constexpr (META4) {
-                if (t == 1 && ph == 0 && i < 2 * NT) issue_meta4(i / 2, i & 1, c + C::SPR, m_next);
+                if (t == 1 && ph == 0) issue_meta4(i / 2, i & 1, c + C::SPR, m_next);
             } else {
-                if (t == 1 && i < 2 * NT) issue_meta(i / 2, i & 1, c + 2, ws);
+                if (t == 1) issue_meta(i / 2, i & 1, c + 2, ws);
             }
-            if (t == C::STAGE_T0 && i >= C::SLOT0_0 && i < C::SLOT0_0 + C::XR) {
-                const int u = i - C::SLOT0_0;
-                stage_unit(u, nxt);
-                if constexpr (C::PH == 1) issue_x_unit(u, c + 2);
-                else issue_x_unit(u + C::XR, c + 1);
+            if (t == C::T_STAGE && i < C::XL) {
+                stage_unit(i, nxt);
+                issue_x_unit(i, c + 2);
             }
-            if (C::PH == 2 && t == C::STAGE_T1 && i >= C::SLOT0_1 && i < C::SLOT0_1 + C::XR) {
-                const int u = i - C::SLOT0_1;
-                stage_unit(u + C::XR, nxt);
-                issue_x_unit(u, c + 2);
-            }
-            // weights: 2 * NT slots of the last MFMA step - the ones the second staging phase leaves free, if any
-            constexpr int W0 = (C::PH == 2 && C::STAGE_T1 == C::MF - 1) ? C::SLOT0_1 + C::XR : 0;
-            static_assert(W0 + 2 * NT <= MT, "weight requests fit behind the staging slots");
-            const int iw = i - W0;
-            if (t == C::MF - 1 && iw >= 0 && iw < 2 * NT && (C::WL == 2 || !(iw & 1))) issue_w_load(iw / 2, C::WL == 2 ? (iw & 1) : 0, c + 2, ws);
+            if (t == C::MF - 1 && (C::WL == 2 || !(i & 1))) issue_w_load(i / 2, C::WL == 2 ? (i & 1) : 0, c + 2, ws);
             asm volatile("" ::: "memory");
         };
         auto next_consts = [&](int j) {
@@ -392,7 +359,6 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
 #pragma unroll
         for (int t = 0; t < C::MF; t++) {
             const int cu = t & 1, nx = cu ^ 1;
-            const int xc = C::XB == 2 ? cu : 0;
             const bool last = t == C::MF - 1, early = last && C::EARLY_W;
 #pragma unroll
             for (int i = 0; i < MT; i++) {
@@ -400,9 +366,8 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
                     // An MFMA occupies the matrix pipe for 16 cycles but the issue port for 4: two or three
                     // VALU operations fit behind each one.  Slot i prepares half a weight fragment of
                     // the next MFMA step (tile i/2, words' low or high byte pair) in four such pieces.
-                    const int jn = i / (2 * SPP), hi = (i / SPP) & 1;
-                    const bool act = i % SPP == 0;
-                    if (early && act && !hi) {
+                    const int jn = i / 2;
+                    if (early && !(i & 1)) {
                         __builtin_amdgcn_sched_barrier(0);
                         next_consts(jn);
                     }
@@ -414,12 +379,12 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
 #pragma unroll
                     for (int j = 0; j < NT; j++) {
                         __builtin_amdgcn_sched_barrier(0);
-                        mfma_acc(acc[i][j], pack_h8(wf[cu][j]), xf[xc][i % C::XRING]);
+                        mfma_acc(acc[i][j], pack_h8(wf[cu][j]), xf[cu][i]);
                         __builtin_amdgcn_sched_barrier(0);
-                        if (j == (C::XB == 2 ? 0 : NT - 1)) next_frag(t, i);
-                        if ((!last || early) && act) {
+                        if (!last || early) {
                             if (j == 0) {
-                                wsrc = hi ? word >> 8 : word;
+                                if (!last) xf[nx][i] = *reinterpret_cast<const h8*>(xp + i * 16 * C::PITCH + 8 * (t + 1));
+                                wsrc = (i & 1) ? word >> 8 : word;
                                 pa = as_h2(and_or(wsrc, 0x000F000Fu, kMagic));
                             } else if (j == 1) {
                                 pb = as_h2(and_or(wsrc, 0x00F000F0u, kMagic));
@@ -429,8 +394,8 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
                                 pa = pa * g4.s;
                             } else {
                                 pb = pb * g4.s;
-                                wf[nx][jn][2 * hi] = pa;
-                                wf[nx][jn][2 * hi + 1] = pb;
+                                wf[nx][jn][2 * (i & 1)] = pa;
+                                wf[nx][jn][2 * (i & 1) + 1] = pb;
                             }
                         }
                         if (j == NT - 1) slot_requests(t, i);
@@ -439,17 +404,15 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
                     __builtin_amdgcn_sched_barrier(0);
                     // weights as the A operand: the result fragment holds 4 consecutive n per lane
 #pragma unroll
-                    for (int j = 0; j < NT; j++) mfma_acc(acc[i][j], pack_h8(wf[cu][j]), xf[xc][i % C::XRING]);
+                    for (int j = 0; j < NT; j++) mfma_acc(acc[i][j], pack_h8(wf[cu][j]), xf[cu][i]);
                     __builtin_amdgcn_sched_barrier(0);
-                    next_frag(t, i);
-                    const int jn = i / (2 * SPP);
-                    if (i % SPP) {
-                    } else if (!((i / SPP) & 1)) {
-                        if (early) next_consts(jn);
+                    if (!last) xf[nx][i] = *reinterpret_cast<const h8*>(xp + i * 16 * C::PITCH + 8 * (t + 1));
+                    if (!(i & 1)) {
+                        if (early) next_consts(i / 2);
                     } else if (!last || early) {
-                        const h8 f = early ? unpack(wsn, jn, 0, gn[jn]) : unpack(ws, jn, t + 1, gc[jn]);
+                        const h8 f = early ? unpack(wsn, i / 2, 0, gn[i / 2]) : unpack(ws, i / 2, t + 1, gc[i / 2]);
 #pragma unroll
-                        for (int e = 0; e < 4; e++) wf[nx][jn][e] = h2{f[2 * e], f[2 * e + 1]};
+                        for (int e = 0; e < 4; e++) wf[nx][i / 2][e] = h2{f[2 * e], f[2 * e + 1]};
                     }
                     slot_requests(t, i);
                 }
@@ -625,7 +588,7 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
     // any difference in order makes the steady state wait for requests it has only just issued.
     auto issue_batch = [&](int c, WSet& ws) {
 #pragma unroll
-        for (int i = 0; i < C::XR; i++) {           // all units of the chunk, or those of the first staging phase
+        for (int i = 0; i < C::XL; i++) {
             issue_x_unit(i, c);
             asm volatile("" ::: "memory");
             __builtin_amdgcn_sched_barrier(0);
@@ -658,16 +621,10 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
     }
     issue_batch(c_begin, set0);
 #pragma unroll
-    for (int i = 0; i < C::XR; i++) stage_unit(i, buf0);
-    if constexpr (C::PH == 2) {
-#pragma unroll
-        for (int i = 0; i < C::XR; i++) issue_x_unit(C::XR + i, c_begin);
-#pragma unroll
-        for (int i = 0; i < C::XR; i++) stage_unit(C::XR + i, buf0);
-    }
+    for (int i = 0; i < C::XL; i++) stage_unit(i, buf0);
     __builtin_amdgcn_sched_barrier(0);
     // second batch in the order of a steady-state step
-    if constexpr (C::T_STAGE == 0 || C::PH == 2) {
+    if constexpr (C::T_STAGE == 0) {
         issue_batch(c_begin + 1, set1);
     } else {
     if constexpr (!META4) {
@@ -680,7 +637,7 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
         }
     }
 #pragma unroll
-    for (int i = 0; i < 2 * NT; i++) {
+    for (int i = 0; i < MT; i++) {
         if (i < C::XL) issue_x_unit(i, c_begin + 1);
         if (C::WL == 2 || !(i & 1)) issue_w_load(i / 2, C::WL == 2 ? (i & 1) : 0, c_begin + 1, set1);
         asm volatile("" ::: "memory");
@@ -876,18 +833,19 @@ int launch_gemm(GemmArgs a, void* workspace, size_t workspace_bytes, hipStream_t
     return BW_OK;
 }
 
-// Rows of a tile for this call.  A 256-row tile unpacks every weight once for twice the rows (0.8 instead of 1.5
-// unpack instructions per MFMA in a loop that is bound by the instructions a wave can issue) and runs 14 % faster per
-// row - when its grid fills the device: measured at 4 and 8 bits, K and N from 4096 to 14336, the 256-row grid wins
-// (3-15 %) from about 0.6 rounds of tiles on and loses (up to 28 %) below.  Not at 2 bits (a K step of 256 values for
-// 256 rows does not fit LDS twice), and only while the split-K blocks of its plan fit the workspace on offer.
+// Rows of a tile for this call.  A 256-row tile unpacks every weight once for twice the rows and keeps the matrix pipe
+// busier (step16) - when its grid fills the device.  Measured at 4 and 8 bits, K and N from 4096 to 14336, M from 256
+// to 4096: the 256-row grid wins by 5-20 % from about 0.6 rounds of tiles on and loses up to 25 % below, except that
+// with a long K (80 K steps and more) and a workspace to split it, a quarter of a round is enough (14336 -> 4096 at
+// 1024 and 2048 rows: 6-13 %).  Not at 2 bits (a K step of 256 values for 256 rows does not fit LDS twice), only for
+// whole K steps, and only while the split-K blocks of its plan fit the workspace on offer.
 inline int gemm_tile_rows(int64_t M, int64_t N, int64_t K, int64_t ldx, int bits, int nchunks, bool have_workspace, size_t workspace_bytes) {
-    if (bits == 2 || K % 128 || (M + 256) * ldx * 2 >= ((int64_t)1 << 32)) return 128;   // whole K steps of 128 values only
+    if (bits == 2 || K % 128 || (M + 256) * ldx * 2 >= ((int64_t)1 << 32)) return 128;
 #ifdef BW_TUNE
     if (const char* e = getenv("BW_GEMM_BM")) return atoi(e) == 256 ? 256 : 128;
 #endif
-    const int64_t tiles = ((N + BN - 1) / BN) * ((M + 255) / 256);
-    if (tiles * 5 < (int64_t)bw_device_cus() * 3) return 128;
+    const int64_t tiles = ((N + BN - 1) / BN) * ((M + 255) / 256), cus = bw_device_cus();
+    if (tiles * 5 < cus * 3 && !(have_workspace && tiles * 4 >= cus && nchunks >= 80)) return 128;
     if (have_workspace && gemm_plan(M, N, nchunks, true, 256).ws_bytes > workspace_bytes) return 128;
     return 256;
 }
@@ -977,14 +935,14 @@ extern "C" size_t bw_qgemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int 
     if (!bw_shape_ok(N, K, bits, group) || M < 1 || M >= ((int64_t)1 << 31) || !bw_fast_shape(M, N, K, K, bits, group)) return 0;
     const int nchunks = gemm_chunks(K, bits);
     const size_t small = gemm_plan(M, N, nchunks, true, 128).ws_bytes;     // either plan may run: enough for both
-    if (gemm_tile_rows(M, N, K, K, bits, nchunks, false, 0) == 128) return small;
+    if (gemm_tile_rows(M, N, K, K, bits, nchunks, true, ~(size_t)0) == 128) return small;
     const size_t big = gemm_plan(M, N, nchunks, true, 256).ws_bytes;
     return big > small ? big : small;
 }
 
 extern "C" int bw_qgemm_tile_rows(int64_t M, int64_t N, int64_t K, int bits, int group) {
     if (!bw_shape_ok(N, K, bits, group) || M < 1 || M >= ((int64_t)1 << 31) || !bw_fast_shape(M, N, K, K, bits, group)) return 0;
-    return gemm_tile_rows(M, N, K, K, bits, gemm_chunks(K, bits), false, 0);
+    return gemm_tile_rows(M, N, K, K, bits, gemm_chunks(K, bits), true, ~(size_t)0);
 }
 
 extern "C" int bw_qgemm_ws(const void* x, int act_dtype, int64_t M, int64_t K, int64_t ldx, const int32_t* qweight,
