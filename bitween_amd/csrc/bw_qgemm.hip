@@ -428,14 +428,15 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
     // and wait instructions cost 1-2 each).  So the side work of an MFMA step is cut into single instructions and dealt
     // out one per gap, by position: gap g = 4 i + j follows the MFMA of m-tile i and n-tile j; region r = g / 16 and
     // k = g % 16 name the 16 gaps of four slots.
-    //   unpack      : n-tile r's fragment for the next MFMA step, one instruction in each of k = 0..15 (4 bits; 0..11 at
-    //                 8 bits); the last MFMA step prepares the first fragment of the next K step from the other set;
+    //   unpack      : n-tile r's fragment for the next MFMA step, 16 instructions at 4 bits and 12 at 8, in the first
+    //                 three gaps of the region's slots (placement below); the last MFMA step prepares the first
+    //                 fragment of the next K step from the other set;
     //   activations : the next chunk's 256 x 128 tile goes memory -> LDS by buffer loads with LDS destination, 16 per
-    //                 wave (4 rows of 256 bytes each), all issued in the first MFMA step so that they have three more
+    //                 wave (4 rows of 256 bytes each), one per slot of the first MFMA step so that they have three more
     //                 to land; no registers, no permute, and nothing the matrix pipe waits for;
     //   fragments   : slot i's last gap reads the activation fragment of slot i + 8 into the ring;
-    //   requests    : scales / zero points at k = 14, 15 of the second MFMA step, weights at k = 14, 15 of the last,
-    //                 group constants of the next step at k = 13 of the last but one.
+    //   requests    : scales / zero points in the second MFMA step, weights in the last, group constants of the next
+    //                 step in the last but one.
     // LDS row r of a buffer holds the chunk's 16-byte slot q of x row r at slot q ^ (r & 7): a lane group of 16 rows
     // reading one slot then spreads over all banks (rows are 256 bytes apart: unswizzled they would share 4 banks).
     // The fragment reads are written as assembly: the compiler orders every LDS read it knows of behind all pending
@@ -491,50 +492,69 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
                 if constexpr (j == 0) __builtin_amdgcn_s_waitcnt(0xC07F | ((7 - (S > 56 ? S - 56 : 0)) << 8));
                 mfma_acc(acc[i][j], pack_h8(wf[cu][j]), xf[0][i % C::XRING]);
                 __builtin_amdgcn_sched_barrier(0);
-                // ---- unpack of n-tile r ----
+                // ---- unpack of n-tile r: instruction v of its sequence ----
                 const auto& gr = early ? gn[r][0] : gc[r][0];
+                auto unpack_op = [&](auto vc) {
+                    constexpr int v = decltype(vc)::value;
+                    if constexpr (BITS == 4) {
+                        const uint32_t word = src.w[r][0][tt];
+                        if constexpr (v == 0) pq[r][0] = __builtin_amdgcn_perm(word, word, 0x01000100u);
+                        if constexpr (v == 1) pq[r][1] = __builtin_amdgcn_perm(word, word, 0x03020302u);
+                        if constexpr (v == 2) up[r][0] = as_h2(and_or(pq[r][0], 0x00F0000Fu, kMagic));
+                        if constexpr (v == 3) uw[r] = pq[r][0] >> 8;
+                        if constexpr (v == 4) up[r][1] = as_h2(and_or(uw[r], 0x00F0000Fu, kMagic));
+                        if constexpr (v == 5) up[r][2] = as_h2(and_or(pq[r][1], 0x00F0000Fu, kMagic));
+                        if constexpr (v == 6) uw[r] = pq[r][1] >> 8;
+                        if constexpr (v == 7) up[r][3] = as_h2(and_or(uw[r], 0x00F0000Fu, kMagic));
+                        if constexpr (v >= 8 && v < 12) up[r][v - 8] = __builtin_elementwise_fma(up[r][v - 8], k16, gr.zz);
+                        if constexpr (v >= 12) wf[nx][r][v - 12] = up[r][v - 12] * gr.s;
+                    } else {
+                        // 8 bits: the two words of MFMA step tt are words 2 (tt % 2), + 1 of lane load tt / 2
+                        const uint32_t w0 = src.w[r][tt / C::SPL][2 * (tt % C::SPL)], w1 = src.w[r][tt / C::SPL][2 * (tt % C::SPL) + 1];
+                        if constexpr (v == 0) up[r][0] = as_h2(__builtin_amdgcn_perm(0x64646464u, w0, 0x04010400u));
+                        if constexpr (v == 1) up[r][1] = as_h2(__builtin_amdgcn_perm(0x64646464u, w0, 0x04030402u));
+                        if constexpr (v == 2) up[r][2] = as_h2(__builtin_amdgcn_perm(0x64646464u, w1, 0x04010400u));
+                        if constexpr (v == 3) up[r][3] = as_h2(__builtin_amdgcn_perm(0x64646464u, w1, 0x04030402u));
+                        if constexpr (v >= 4 && v < 8) up[r][v - 4] = up[r][v - 4] + gr.zz;
+                        if constexpr (v >= 8 && v < 12) wf[nx][r][v - 8] = up[r][v - 8] * gr.s;
+                    }
+                };
+                // A gap holds VALU work or the slot's fragment read, not both (measured: one VALU instruction in each of
+                // a slot's four gaps plus the read costs 8.4 ns per MFMA, the read in a gap of its own 7.0 = the bare
+                // MFMA rate; a second VALU instruction in a gap costs 3 cycles).  So the last gap of a slot belongs to the
+                // read; 8 bits puts its 12 instructions one into each other gap, 4 bits its 16 two into the first gap
+                // of each slot and one into the next two.
+                constexpr int sl = k / 4;                                  // slot of the region
                 if constexpr (BITS == 4) {
-                    const uint32_t word = src.w[r][0][tt];
-                    if constexpr (k == 0) pq[r][0] = __builtin_amdgcn_perm(word, word, 0x01000100u);
-                    if constexpr (k == 1) pq[r][1] = __builtin_amdgcn_perm(word, word, 0x03020302u);
-                    if constexpr (k == 2) up[r][0] = as_h2(and_or(pq[r][0], 0x00F0000Fu, kMagic));
-                    if constexpr (k == 3) uw[r] = pq[r][0] >> 8;
-                    if constexpr (k == 4) up[r][1] = as_h2(and_or(uw[r], 0x00F0000Fu, kMagic));
-                    if constexpr (k == 5) up[r][2] = as_h2(and_or(pq[r][1], 0x00F0000Fu, kMagic));
-                    if constexpr (k == 6) uw[r] = pq[r][1] >> 8;
-                    if constexpr (k == 7) up[r][3] = as_h2(and_or(uw[r], 0x00F0000Fu, kMagic));
-                    if constexpr (k >= 8 && k < 12) up[r][k - 8] = __builtin_elementwise_fma(up[r][k - 8], k16, gr.zz);
-                    if constexpr (k >= 12) wf[nx][r][k - 12] = up[r][k - 12] * gr.s;
+                    if constexpr (j == 0) {
+                        unpack_op(std::integral_constant<int, 4 * sl>{});
+                        unpack_op(std::integral_constant<int, 4 * sl + 1>{});
+                    } else if constexpr (j < 3) {
+                        unpack_op(std::integral_constant<int, 4 * sl + 1 + j>{});
+                    }
                 } else {
-                    // 8 bits: the two words of MFMA step tt are words 2 (tt % 2), + 1 of lane load tt / 2
-                    const uint32_t w0 = src.w[r][tt / C::SPL][2 * (tt % C::SPL)], w1 = src.w[r][tt / C::SPL][2 * (tt % C::SPL) + 1];
-                    if constexpr (k == 0) up[r][0] = as_h2(__builtin_amdgcn_perm(0x64646464u, w0, 0x04010400u));
-                    if constexpr (k == 1) up[r][1] = as_h2(__builtin_amdgcn_perm(0x64646464u, w0, 0x04030402u));
-                    if constexpr (k == 2) up[r][2] = as_h2(__builtin_amdgcn_perm(0x64646464u, w1, 0x04010400u));
-                    if constexpr (k == 3) up[r][3] = as_h2(__builtin_amdgcn_perm(0x64646464u, w1, 0x04030402u));
-                    if constexpr (k >= 4 && k < 8) up[r][k - 4] = up[r][k - 4] + gr.zz;
-                    if constexpr (k >= 8 && k < 12) wf[nx][r][k - 8] = up[r][k - 8] * gr.s;
+                    if constexpr (j < 3) unpack_op(std::integral_constant<int, 3 * sl + j>{});
                 }
-                // ---- the next chunk's activations: unit u at gap 3 u + 1 of the first MFMA step ----
-                if constexpr (t == 0 && g % 3 == 1 && g / 3 < 16) x_dma16(g / 3, c + 1, nxt);
+                // ---- the next chunk's activations: unit i of the wave in slot i of the first MFMA step ----
+                if constexpr (t == 0 && j == 1) x_dma16(i, c + 1, nxt);
                 // ---- fragment ring ----
                 if constexpr (j == NT - 1) {
                     constexpr int i2 = (i + C::XRING) % MT, t2 = t + (i + C::XRING) / MT;
                     if constexpr (t2 < C::MF) frag_read(std::integral_constant<int, t2>{}, std::integral_constant<int, i2>{});
                 }
-                // ---- requests and constants ----
-                if constexpr (t == 1 && k >= 14) {
+                // ---- requests and constants (second gap of a slot) ----
+                if constexpr (t == 1 && j == 1 && sl >= 2) {
                     if constexpr (META4) {
-                        if (ph == 0) issue_meta4(r, k - 14, c + C::SPR, m_next);
+                        if (ph == 0) issue_meta4(r, sl - 2, c + C::SPR, m_next);
                     } else {
-                        issue_meta(r, k - 14, c + 2, ws);
+                        issue_meta(r, sl - 2, c + 2, ws);
                     }
                 }
-                if constexpr (t == C::MF - 2 && k == 13) {
+                if constexpr (t == C::MF - 2 && k == 14) {
                     if constexpr (META4) set_consts(gn[r], r, wsn, ph < C::SPR - 1 ? m_cur : m_next, ph < C::SPR - 1 ? ph + 1 : 0);
                     else set_consts(gn[r], r, wsn, m_cur, 0);
                 }
-                if constexpr (t == C::MF - 1 && k >= 16 - C::WL) w_req16(r, k - (16 - C::WL), c + 2, ws);
+                if constexpr (t == C::MF - 1 && j == 1 && sl >= 4 - C::WL) w_req16(r, sl - (4 - C::WL), c + 2, ws);
                 asm volatile("" ::: "memory");
             });
         });
