@@ -719,6 +719,41 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
         }
         return;
     }
+    // A lane's 8 bytes per MFMA tile make a wave's store 16 pieces of 32 bytes in 16 different rows: a quarter of every
+    // cache line it touches.  Where the wave's 64 columns are all inside N and y allows 16-byte stores, the wave's
+    // BM x 64 block goes through its own quarter of LDS instead (free after the last K step; 128-byte rows, the 16-byte
+    // slots of a row XOR-swizzled by the row number) and leaves as whole 128-byte rows, 8 per store instruction.
+    if (n0 + NT * 16 <= a.N && a.ldy % 8 == 0 && (((uintptr_t)a.y) & 15) == 0) {
+        __builtin_amdgcn_s_waitcnt(0xC07F);                     // the assembly fragment reads of the last step (256-row tiles)
+        char* ob = smem + wave * (BM * 128);
+#pragma unroll
+        for (int j = 0; j < NT; j++) {
+            const int n = n0 + 16 * j + 4 * kq;
+            float bv[4] = {0.f, 0.f, 0.f, 0.f};
+            if (a.bias) {
+#pragma unroll
+                for (int r = 0; r < 4; r++) bv[r] = (float)a.bias[n + r];
+            }
+            const int ch = 4 * j + kq;                           // 8-byte piece of the 128-byte row
+#pragma unroll
+            for (int i = 0; i < MT; i++) {
+                const int row = 16 * i + nl;
+                const _Float16 v0 = (_Float16)(acc[i][j][0] + bv[0]), v1 = (_Float16)(acc[i][j][1] + bv[1]),
+                               v2 = (_Float16)(acc[i][j][2] + bv[2]), v3 = (_Float16)(acc[i][j][3] + bv[3]);
+                *reinterpret_cast<u2*>(ob + row * 128 + (((ch >> 1) ^ (row & 7)) * 16) + (ch & 1) * 8) = u2{as_u32(h2{v0, v1}), as_u32(h2{v2, v3})};
+            }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+        for (int q = 0; q < BM / 8; q++) {
+            const int row = 8 * q + (lane >> 3), unit = lane & 7;
+            const u4 v = *reinterpret_cast<const u4*>(ob + row * 128 + ((unit ^ (row & 7)) * 16));
+            if (m0 + row < a.M) *reinterpret_cast<u4*>(a.y + (int64_t)(m0 + row) * a.ldy + n0 + unit * 8) = v;
+        }
+        return;
+    }
 #pragma unroll
     for (int j = 0; j < NT; j++) {
         const int n = n0 + 16 * j + 4 * kq;
