@@ -8,7 +8,7 @@ A step is one decode pass (M = 1) through the 224 quantised linears of a 32-laye
 HBM: --layers distinct layers' weights (8: 860 MB, more than the 256 MiB Infinity Cache holds) are run through
 32 / layers times.  `value` is algorithmic bytes per step (packed weights + scales + zero points + activations
 in + out) over the time per step, in GB/s.  A step is one HIP graph of 224 launches, so the Python
-interpreter is not what is being timed and a run of 20 steps lasts about 25 ms.
+interpreter is not what is being timed; the default 100 steps (after 20 warm-ups) last about 110 ms.
 
 Also reported on the same JSON line: the roofline of the decode kernel (overall and per layer shape, next to
 this board's measured stream-copy rate), the CPU path timed on the host cores, and (unless --no-extras)

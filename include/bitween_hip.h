@@ -145,9 +145,11 @@ int bw_qgemm_ws(const void* x, int act_dtype, int64_t M, int64_t K, int64_t ldx,
  * so results are those of bw_qgemm_ws, bit for bit.  No counterpart in the reference; it is for callers that
  * cannot allocate: code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.
  * The first call on a device looks up the array's address there (hipGetSymbolAddress); no call allocates,
- * frees or synchronises.  A shape whose partial tiles exceed the array returns BW_EWORKSPACE (none does on a
- * 256-CU device).  Every call on a GPU shares that GPU's array: calls that overlap in time on one GPU (two
- * streams, two threads) race on it - serialise them or use bw_qgemm_ws with a workspace per stream. */
+ * frees or synchronises.  A shape whose 256-row plan needs more than the array runs with 128-row tiles; one whose
+ * partial tiles still exceed it returns BW_EWORKSPACE (none does on a 256-CU device).  One call at a time per GPU:
+ * every call on a GPU shares that GPU's array, so calls on one stream (ordered) are safe, and calls that overlap in
+ * time on one GPU (two streams, two threads) race on it - serialise them or use bw_qgemm_ws with a workspace per
+ * stream.  The entry point does not detect an overlap (it would need an event query per call). */
 int bw_qgemm_static(const void* x, int act_dtype, int64_t M, int64_t K, int64_t ldx,
                     const int32_t* qweight, const void* scale16, const void* zp16, const void* bias,
                     int64_t N, int bits, int group, void* y, int64_t ldy, void* stream);
