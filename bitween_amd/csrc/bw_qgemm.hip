@@ -896,7 +896,7 @@ int launch_gemm(GemmArgs a, void* workspace, size_t workspace_bytes, hipStream_t
 // whole K steps, and only while the split-K blocks of its plan fit the workspace on offer.
 inline int gemm_tile_rows(int64_t M, int64_t N, int64_t K, int64_t ldx, int bits, int nchunks, bool have_workspace, size_t workspace_bytes) {
     if (bits == 2 || K % 128 || (M + 256) * ldx * 2 >= ((int64_t)1 << 32)) return 128;
-#ifdef BW_TUNE
+#ifdef BW_TUNE   // measurement builds only (-DBW_TUNE, never the library build.py makes): the tile height from the environment, for A/B runs
     if (const char* e = getenv("BW_GEMM_BM")) return atoi(e) == 256 ? 256 : 128;
 #endif
     const int64_t tiles = ((N + BN - 1) / BN) * ((M + 255) / 256), cus = bw_device_cus();

@@ -91,9 +91,6 @@ struct GemvArgs {
     int x_bf16;                              // x holds bfloat16: every value is rounded to float16 as it is staged
     int ntiles, nsteps;                      // qgemv_tiles_kernel / qgemv_rounds_kernel: 16-row tiles of N; tiles or rounds per workgroup
     int meta_lds_off;                        // qgemv_tiles_kernel: where the scale blocks start in LDS
-#ifdef BW_TUNE
-    int tune;
-#endif
 };
 
 // two bfloat16 -> two float16, round to nearest even (what torch's .to(float16) does)
@@ -667,20 +664,6 @@ struct WeightTile {
     static constexpr int kPair = 2 * kHalf;               // LDS bytes per pair of chunks (16 rows x 128 bytes + padding)
     static constexpr int kAuxNt = 2;                      // cache-policy bits of the buffer load: non-temporal
 
-    // request pair q of a wave's batch: chunks c, c + 1 of rows n0 .. n0 + 15 (rows past N and chunks past the row's end
-    // are range-checked to zero by the buffer resource)
-    static BW_DEV void request(const __amdgpu_buffer_rsrc_t& rw, char* tile, int q, uint32_t n0, int c, int row_bytes, int lane) {
-        const int a = lane >> 3, p = (lane & 7) ^ a;
-        const int cc = c + (p >> 2);
-#pragma unroll
-        for (int i = 0; i < 2; i++) {
-            uint32_t off = (n0 + 8 * i + a) * (uint32_t)row_bytes + cc * 64 + (p & 3) * 16;
-            asm volatile("" : "+v"(off));                     // a value of its own: the select below stays a select
-            off = cc * 64 < row_bytes ? off : 0x80000000u;
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, (__attribute__((address_space(3))) void*)(tile + q * kPair + i * kHalf),
-                                                     16, off, 0, 0, kAuxNt);
-        }
-    }
     // the 16 bytes lane (n = lane & 15, j = lane >> 4) feeds the matrix core with for chunk b of the batch
     static BW_DEV u4 fetch(const char* tile, int b, int lane) {
         const int n = lane & 15, j = lane >> 4, a = n & 7, p = (b & 1) * 4 + j;
@@ -961,7 +944,7 @@ int launch_w4(const GemvArgs& a, hipStream_t stream) {
     // Chunks a wave requests per round (pairs, each landing in LDS), from timing the Llama-7B shapes on MI355X at
     // M = 1 (us: 4096 x 4096 / 4096 -> 11008 / 11008 -> 4096): 2 chunks 4.00 / 7.02 / 6.20, 4 chunks 3.98 / 6.22 / 6.45,
     // 8 chunks 4.24 / 6.45 / 6.95 - rows that fit one round of up to 16 waves take 4, longer rows many short rounds
-#ifdef BW_TUNE
+#ifdef BW_TUNE   // measurement builds only (-DBW_TUNE, never the library build.py makes): kernel choices from the environment, for A/B runs
     if (const char* e = getenv("BW_W4_KB")) {
         switch (atoi(e)) {
             case 2: return launch_w4_kb<GROUP, MT, 2>(a, stream);
@@ -1700,9 +1683,6 @@ extern "C" int bw_qgemv(const void* x, int act_dtype, int64_t M, int64_t K, int6
     a.w_bytes = (uint32_t)(N * a.row_bytes);
     a.meta_bytes = (uint32_t)(N * a.groups * 2);
     hipStream_t st = (hipStream_t)stream;
-#ifdef BW_TUNE
-    a.tune = getenv("BW_TUNE_FLAGS") ? atoi(getenv("BW_TUNE_FLAGS")) : 0;
-#endif
 #define BW_CASE(B, G) \
     if (bits == B && group == G) return launch_gemv<B, G>(a, st);
     BW_CASE(4, 128) BW_CASE(4, 64) BW_CASE(4, 32)
