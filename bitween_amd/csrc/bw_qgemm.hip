@@ -37,9 +37,12 @@ struct GemmCfg {
     // first fragments, scale and zero-point requests - are spread equally thin) and a lane's values never
     // span more than one group of 32.
     static constexpr int WL = BITS == 8 ? 2 : 1;
-    static constexpr int VPI = 32 / BITS, VPL = WL * 128 / BITS, CHUNK_K = 4 * VPL, MF = VPL / 8;
+    // bytes of a lane load: 16, except 8 at 2 bits with 256-row tiles - there a K step is 128 values like at the other
+    // widths (a 256-value step of 256 rows of activations would not fit LDS twice)
+    static constexpr int LB = (BITS == 2 && MT == 16) ? 8 : 16;
+    static constexpr int VPI = 32 / BITS, VPL = WL * LB * 8 / BITS, CHUNK_K = 4 * VPL, MF = VPL / 8;
     static constexpr int SPL = MF / WL;                          // MFMA steps per lane load
-    static constexpr int CHUNK_BYTES = 64 * WL;                  // of a packed weight row
+    static constexpr int CHUNK_BYTES = 4 * LB * WL;              // of a packed weight row
     static constexpr int NG = (VPL > GROUP) ? VPL / GROUP : 1;   // groups inside a lane's values
     static constexpr int WPG = 4 * WL / NG;                      // words of a lane's values per group
     // One K step = one group, or two: the scales (zero points) of four (two) consecutive steps are 8 adjacent bytes
@@ -92,14 +95,31 @@ BW_DEV void permute_unit(const uint32_t* r, uint32_t* o) {
 // n1 in bits 4-7 of their high half, p >> 8 likewise n2 and n3; masked into the mantissa of 1024.0 that is
 // (1024 + n0, 1024 + 16 n1), and one packed FMA with (1, 1/16) and (-(1024 + z), -(64 + z)) leaves (n0 - z, n1 - z),
 // both exact.  Times the scale: the float16 the reference's dequantize stores (bitween/modules.py:55-58).
+// 2 bits: a 16-bit half-word h = bytes b0 b1 holds fields c0..c7; p = [b0 b1 b0 b1] and p >> 8 = [b1 b0 b1 0] carry c0 / c4
+// in bits 0-1 and c2 / c6 in bits 4-5 of their low half, c1 / c5 in bits 2-3 and c3 / c7 in bits 6-7 of their high half:
+// masks 0x000C0003 and 0x00C00030 give (1024 + c0, 1024 + 4 c1) and (1024 + 16 c2, 1024 + 64 c3); packed FMAs with
+// (1, 1/4), (-(1024+z), -(256+z)) and (1/16, 1/64), (-(64+z), -(16+z)) leave the exact differences.
 template <int BITS> struct GroupConstNat {
-    h2 s, zz;
+    h2 s, zz, zz2;
     BW_DEV void set(_Float16 sv, _Float16 zv) {
         s = splat(sv);
         if constexpr (BITS == 4) zz = h2{(_Float16)(-1024.0f) - zv, (_Float16)(-64.0f) - zv};
-        else zz = splat((_Float16)(-1024.0f) - zv);
+        else if constexpr (BITS == 2) {
+            zz = h2{(_Float16)(-1024.0f) - zv, (_Float16)(-256.0f) - zv};
+            zz2 = h2{(_Float16)(-64.0f) - zv, (_Float16)(-16.0f) - zv};
+        } else zz = splat((_Float16)(-1024.0f) - zv);
     }
 };
+
+// half-word `half` (0 or 1) of a 2-bit word -> 4 pairs in natural order
+BW_DEV void dequant_halfword2_nat(uint32_t w, int half, const GroupConstNat<2>& c, h2 out[4]) {
+    const h2 ka = h2{(_Float16)1.0f, (_Float16)0.25f}, kb = h2{(_Float16)0.0625f, (_Float16)0.015625f};
+    const uint32_t p = half ? __builtin_amdgcn_perm(w, w, 0x03020302u) : __builtin_amdgcn_perm(w, w, 0x01000100u), q = p >> 8;
+    out[0] = __builtin_elementwise_fma(as_h2(and_or(p, 0x000C0003u, kMagic)), ka, c.zz) * c.s;
+    out[1] = __builtin_elementwise_fma(as_h2(and_or(p, 0x00C00030u, kMagic)), kb, c.zz2) * c.s;
+    out[2] = __builtin_elementwise_fma(as_h2(and_or(q, 0x000C0003u, kMagic)), ka, c.zz) * c.s;
+    out[3] = __builtin_elementwise_fma(as_h2(and_or(q, 0x00C00030u, kMagic)), kb, c.zz2) * c.s;
+}
 
 BW_DEV void dequant_word4_nat(uint32_t w, const GroupConstNat<4>& c, h2 out[4]) {
     const h2 kk = h2{(_Float16)1.0f, (_Float16)0.0625f};
@@ -203,7 +223,7 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
         const int row = n0 + 16 * j + nl;
         // (256-row tiles add a scalar chunk offset that is itself "out of range" past the last chunk: rows past N then
         // read the last row's bytes instead of relying on a sum that could wrap; their outputs are never stored)
-        w_off[j] = row < a.N ? (uint32_t)row * a.row_bytes + kq * 16 * C::WL : MT == 16 ? (uint32_t)(a.N - 1) * a.row_bytes + kq * 16 * C::WL : kOob;
+        w_off[j] = row < a.N ? (uint32_t)row * a.row_bytes + kq * C::LB * C::WL : MT == 16 ? (uint32_t)(a.N - 1) * a.row_bytes + kq * C::LB * C::WL : kOob;
         m_off[j] = (uint32_t)min(row, a.N - 1) * groups * 2;
     }
     // 128-row tiles: byte offsets of the staging units of a thread
@@ -275,6 +295,8 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
             h2 o[4];
             if constexpr (BITS == 4) {
                 dequant_word4_nat(ws.w[j][0][t], gcj[0], o);
+            } else if constexpr (BITS == 2) {
+                dequant_halfword2_nat(ws.w[j][0][t / 2], t % 2, gcj[0], o);
             } else {
 #pragma unroll
                 for (int e = 0; e < 2; e++) {
@@ -464,7 +486,13 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
     };
     auto w_req16 = [&](int j, int l, int cc, WSet& ws) {
         const uint32_t so = cc < c_end ? (uint32_t)cc * C::CHUNK_BYTES + l * 16 : kOob;
-        ws.w[j][l] = __builtin_amdgcn_raw_buffer_load_b128(rw, w_off[j] + so, 0, 0);
+        if constexpr (C::LB == 8) {
+            const u2 v = __builtin_amdgcn_raw_buffer_load_b64(rw, w_off[j] + so, 0, 0);
+            ws.w[j][l][0] = v[0];
+            ws.w[j][l][1] = v[1];
+        } else {
+            ws.w[j][l] = __builtin_amdgcn_raw_buffer_load_b128(rw, w_off[j] + so, 0, 0);
+        }
     };
     // fragment (m-tile i, MFMA step t) of the lane: slot 4 kq + t of row 16 i + nl, swizzled
     uint32_t fa[4];
@@ -480,6 +508,7 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
         };
         static_for<0, C::XRING>([&](auto ic) { frag_read(std::integral_constant<int, 0>{}, ic); });
         const h2 k16 = h2{(_Float16)1.0f, (_Float16)0.0625f};
+        const h2 k2a = h2{(_Float16)1.0f, (_Float16)0.25f}, k2b = h2{(_Float16)0.0625f, (_Float16)0.015625f};
         static_for<0, C::MF>([&](auto tc) {
             constexpr int t = decltype(tc)::value, cu = t & 1, nx = cu ^ 1;
             constexpr bool early = t == C::MF - 1;
@@ -508,6 +537,17 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
                         if constexpr (v == 7) up[r][3] = as_h2(and_or(uw[r], 0x00F0000Fu, kMagic));
                         if constexpr (v >= 8 && v < 12) up[r][v - 8] = __builtin_elementwise_fma(up[r][v - 8], k16, gr.zz);
                         if constexpr (v >= 12) wf[nx][r][v - 12] = up[r][v - 12] * gr.s;
+                    } else if constexpr (BITS == 2) {
+                        // half-word tt of the lane's 8 bytes
+                        const uint32_t word = src.w[r][0][tt / 2];
+                        if constexpr (v == 0) pq[r][0] = tt % 2 ? __builtin_amdgcn_perm(word, word, 0x03020302u) : __builtin_amdgcn_perm(word, word, 0x01000100u);
+                        if constexpr (v == 1) uw[r] = pq[r][0] >> 8;
+                        if constexpr (v == 2) up[r][0] = as_h2(and_or(pq[r][0], 0x000C0003u, kMagic));
+                        if constexpr (v == 3) up[r][1] = as_h2(and_or(pq[r][0], 0x00C00030u, kMagic));
+                        if constexpr (v == 4) up[r][2] = as_h2(and_or(uw[r], 0x000C0003u, kMagic));
+                        if constexpr (v == 5) up[r][3] = as_h2(and_or(uw[r], 0x00C00030u, kMagic));
+                        if constexpr (v >= 6 && v < 10) up[r][v - 6] = __builtin_elementwise_fma(up[r][v - 6], (v & 1) ? k2b : k2a, (v & 1) ? gr.zz2 : gr.zz);
+                        if constexpr (v >= 10 && v < 14) wf[nx][r][v - 10] = up[r][v - 10] * gr.s;
                     } else {
                         // 8 bits: the two words of MFMA step tt are words 2 (tt % 2), + 1 of lane load tt / 2
                         const uint32_t w0 = src.w[r][tt / C::SPL][2 * (tt % C::SPL)], w1 = src.w[r][tt / C::SPL][2 * (tt % C::SPL) + 1];
@@ -525,7 +565,7 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
                 // read; 8 bits puts its 12 instructions one into each other gap, 4 bits its 16 two into the first gap
                 // of each slot and one into the next two.
                 constexpr int sl = k / 4;                                  // slot of the region
-                if constexpr (BITS == 4) {
+                if constexpr (BITS != 8) {
                     if constexpr (j == 0) {
                         unpack_op(std::integral_constant<int, 4 * sl>{});
                         unpack_op(std::integral_constant<int, 4 * sl + 1>{});
@@ -820,8 +860,8 @@ struct GemmPlan {
     size_t ws_bytes;
 };
 
-inline int gemm_chunks(int64_t K, int bits) {   // K steps of a whole row: GemmCfg::CHUNK_BYTES each
-    const int64_t chunk = bits == 8 ? 128 : 64;
+inline int gemm_chunks(int64_t K, int bits, int tile_rows = 128) {   // K steps of a whole row: GemmCfg::CHUNK_BYTES each
+    const int64_t chunk = bits == 8 ? 128 : (bits == 2 && tile_rows == 256) ? 32 : 64;
     return (int)((K * bits / 8 + chunk - 1) / chunk);
 }
 
@@ -856,7 +896,7 @@ template <int BITS, int GROUP, int MT = 8>
 int launch_gemm(GemmArgs a, void* workspace, size_t workspace_bytes, hipStream_t stream) {
     using C = GemmCfg<BITS, GROUP, MT>;
     constexpr int BM = C::BM;
-    static_assert(C::CHUNK_BYTES == (BITS == 8 ? 128 : 64), "gemm_chunks() counts K steps of this size");
+    static_assert(C::CHUNK_BYTES == (BITS == 8 ? 128 : (BITS == 2 && MT == 16) ? 32 : 64), "gemm_chunks() counts K steps of this size");
     const size_t lds = 2 * (size_t)C::STAGE_BYTES;
     void (*kern)(const GemmArgs) = qgemm_kernel<BITS, GROUP, false, MT>;
     static uint64_t big_lds_devices[2] = {0, 0};           // per kernel
@@ -892,10 +932,11 @@ int launch_gemm(GemmArgs a, void* workspace, size_t workspace_bytes, hipStream_t
 // busier (step16) - when its grid fills the device.  Measured at 4 and 8 bits, K and N from 4096 to 14336, M from 256
 // to 4096: the 256-row grid wins by 5-20 % from about 0.6 rounds of tiles on and loses up to 25 % below, except that
 // with a long K (80 K steps and more) and a workspace to split it, a quarter of a round is enough (14336 -> 4096 at
-// 1024 and 2048 rows: 6-13 %).  Not at 2 bits (a K step of 256 values for 256 rows does not fit LDS twice), only for
-// whole K steps, and only while the split-K blocks of its plan fit the workspace on offer.
-inline int gemm_tile_rows(int64_t M, int64_t N, int64_t K, int64_t ldx, int bits, int nchunks, bool have_workspace, size_t workspace_bytes) {
-    if (bits == 2 || K % 128 || (M + 256) * ldx * 2 >= ((int64_t)1 << 32)) return 128;
+// 1024 and 2048 rows: 6-13 %).  Only for whole K steps of 128 values, and only while the split-K blocks of its plan fit
+// the workspace on offer.  (The K steps counted here are those of the 256-row kernel: 128 values at every width.)
+inline int gemm_tile_rows(int64_t M, int64_t N, int64_t K, int64_t ldx, int bits, bool have_workspace, size_t workspace_bytes) {
+    if (K % 128 || (M + 256) * ldx * 2 >= ((int64_t)1 << 32)) return 128;
+    const int nchunks = gemm_chunks(K, bits, 256);
 #ifdef BW_TUNE   // measurement builds only (-DBW_TUNE, never the library build.py makes): the tile height from the environment, for A/B runs
     if (const char* e = getenv("BW_GEMM_BM")) return atoi(e) == 256 ? 256 : 128;
 #endif
@@ -988,16 +1029,15 @@ int bw_qgemm_generic(const void* x, int act_dtype, int64_t M, int64_t K, int64_t
 
 extern "C" size_t bw_qgemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int bits, int group) {
     if (!bw_shape_ok(N, K, bits, group) || M < 1 || M >= ((int64_t)1 << 31) || !bw_fast_shape(M, N, K, K, bits, group)) return 0;
-    const int nchunks = gemm_chunks(K, bits);
-    const size_t small = gemm_plan(M, N, nchunks, true, 128).ws_bytes;     // either plan may run: enough for both
-    if (gemm_tile_rows(M, N, K, K, bits, nchunks, true, ~(size_t)0) == 128) return small;
-    const size_t big = gemm_plan(M, N, nchunks, true, 256).ws_bytes;
+    const size_t small = gemm_plan(M, N, gemm_chunks(K, bits), true, 128).ws_bytes;     // either plan may run: enough for both
+    if (gemm_tile_rows(M, N, K, K, bits, true, ~(size_t)0) == 128) return small;
+    const size_t big = gemm_plan(M, N, gemm_chunks(K, bits, 256), true, 256).ws_bytes;
     return big > small ? big : small;
 }
 
 extern "C" int bw_qgemm_tile_rows(int64_t M, int64_t N, int64_t K, int bits, int group) {
     if (!bw_shape_ok(N, K, bits, group) || M < 1 || M >= ((int64_t)1 << 31) || !bw_fast_shape(M, N, K, K, bits, group)) return 0;
-    return gemm_tile_rows(M, N, K, K, bits, gemm_chunks(K, bits), true, ~(size_t)0);
+    return gemm_tile_rows(M, N, K, K, bits, true, ~(size_t)0);
 }
 
 extern "C" int bw_qgemm_ws(const void* x, int act_dtype, int64_t M, int64_t K, int64_t ldx, const int32_t* qweight,
@@ -1024,14 +1064,15 @@ extern "C" int bw_qgemm_ws(const void* x, int act_dtype, int64_t M, int64_t K, i
     a.splits = 1;
     a.chunks_per_split = a.nchunks;
     hipStream_t st = (hipStream_t)stream;
-    const bool big = gemm_tile_rows(M, N, K, ldx, bits, a.nchunks, workspace != nullptr, workspace_bytes) == 256;
+    const bool big = gemm_tile_rows(M, N, K, ldx, bits, workspace != nullptr, workspace_bytes) == 256;
+    if (big) a.chunks_per_split = a.nchunks = gemm_chunks(K, bits, 256);
 #define BW_CASE(B, G) \
     if (bits == B && group == G) return launch_gemm<B, G>(a, workspace, workspace_bytes, st);
 #define BW_CASE2(B, G) \
     if (bits == B && group == G) return big ? launch_gemm<B, G, 16>(a, workspace, workspace_bytes, st) : launch_gemm<B, G>(a, workspace, workspace_bytes, st);
     BW_CASE2(4, 128) BW_CASE2(4, 64) BW_CASE2(4, 32)
     BW_CASE2(8, 128) BW_CASE2(8, 64) BW_CASE2(8, 32)
-    BW_CASE(2, 128) BW_CASE(2, 64) BW_CASE(2, 32)
+    BW_CASE2(2, 128) BW_CASE2(2, 64) BW_CASE2(2, 32)
 #undef BW_CASE
 #undef BW_CASE2
     return BW_EUNSUPPORTED;

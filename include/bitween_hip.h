@@ -131,7 +131,7 @@ int bw_qgemm(const void* x, int act_dtype, int64_t M, int64_t K, int64_t ldx,
 size_t bw_qgemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int bits, int group);
 
 /* Rows of the output tile the prefill kernel runs this shape with (x rows K apart, any workspace it asks for granted):
- * 128, or 256 once a grid of 256-row tiles fills most of the device (4 and 8 bits); 0 = the shape-generic kernel.
+ * 128, or 256 once a grid of 256-row tiles fills most of the device; 0 = the shape-generic kernel.
  * A diagnostic for benchmarks and tests; no counterpart in the reference. */
 int bw_qgemm_tile_rows(int64_t M, int64_t N, int64_t K, int bits, int group);
 

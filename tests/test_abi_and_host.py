@@ -66,8 +66,8 @@ def test_split_k_workspace_size_is_a_pure_host_function():
     assert ws(4096, 4096, 4096, 4, 128) == 0 and rows(4096, 4096, 4096, 4, 128) == 256    # 512 tiles of 128 rows, or 256 of 256
     # a long K with a quarter round of 256-row tiles and more: those, every tile cut in two (128 tiles x 2 slices of 256 x 256)
     assert rows(2048, 4096, 14336, 4, 128) == 256 and ws(2048, 4096, 14336, 4, 128) == 128 * 2 * 2 * tile
-    # 256-row tiles need 4 or 8 bits, whole K steps of 128 values and a grid that fills the device
-    assert rows(4096, 4096, 4096, 2, 128) == 128 and rows(4096, 4096, 4096 + 64, 4, 64) == 128 and rows(512, 14336, 4096, 4, 128) == 128
+    # 256-row tiles need whole K steps of 128 values and a grid that fills the device
+    assert rows(4096, 4096, 4096, 2, 128) == 256 and rows(4096, 4096, 4096 + 64, 4, 64) == 128 and rows(512, 14336, 4096, 4, 128) == 128
     assert rows(128, 20, 96, 4, 48) == 0                        # the shape-generic kernel
     assert ws(512, 14336, 4096, 4, 128) == 0                    # 224 tiles: 0.875 of a round
     # few tiles and a long K: every tile split so that one round is filled

@@ -905,7 +905,7 @@ def test_sibling_group_does_not_serve_a_member_twice_from_its_cache():
     assert torch.equal(k2, ref_k)
 
 
-@pytest.mark.parametrize("bits,g", [(4, 128), (4, 64), (4, 32), (8, 128), (8, 64), (8, 32)])
+@pytest.mark.parametrize("bits,g", [(4, 128), (4, 64), (4, 32), (8, 128), (8, 64), (8, 32), (2, 128), (2, 64), (2, 32)])
 @pytest.mark.parametrize("k", [896, 1024])
 def test_prefill_256_row_tiles_vs_oracle(bits, g, k):
     """Shapes whose grid of 256-row tiles fills the device take the 256-row variant of the prefill kernel (same
