@@ -12,8 +12,8 @@
 //   * activations go global -> LDS once per workgroup (double buffered,
 //     permuted into the k order the unpack emits) and every A fragment read
 //     from LDS feeds 4 MFMAs.
-// Grids that fill the device run the same kernel with 256 x 256 tiles at 4 and
-// 8 bits (a wave owns 256 x 64: all 256 accumulation registers): every weight
+// Grids that fill the device run the same kernel with 256 x 256 tiles (a wave
+// owns 256 x 64: all 256 accumulation registers): every weight
 // is unpacked once for twice the rows, the activations go memory -> LDS
 // without passing through registers, and the side work of an MFMA step is
 // dealt out one instruction per MFMA (step16 below).
