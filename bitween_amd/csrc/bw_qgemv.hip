@@ -246,7 +246,7 @@ BW_DEV float half_of(uint32_t word, int hi) {
     return (float)__builtin_bit_cast(_Float16, (uint16_t)(hi ? word >> 16 : word));
 }
 
-// ---- 3 <= M <= 16, K <= 4096: every request of a workgroup in flight at once ----------------------------------
+// ---- M <= 16 (from the row count tiles_min_rows names per format), K <= 4096: every request of a workgroup in flight at once ----
 //
 // qgemv_kernel re-reads and re-stages its slice of x in every round of every 16-row workgroup, and a wave only
 // has one round of weights requested at a time: with 4 to 16 activation rows the x traffic (from L2) is several
@@ -454,7 +454,7 @@ __global__ __launch_bounds__(1024) void qgemv_tiles_kernel(const GemvArgs a) {
     }
 }
 
-// ---- 3 <= M <= 16, long K: one 16-row tile per workgroup, rounds of K -------------------------------------------
+// ---- M <= 16 (same table), long K: one 16-row tile per workgroup, rounds of K -----------------------------------
 //
 // Wave w of up to 16 owns chunks [(r waves + w) KBW, +KBW) of round r.  The weights of DEPTH rounds are requested
 // ahead in registers (all rounds, for the usual shapes; else a ring that is refilled as it drains); x is restaged
@@ -671,7 +671,7 @@ struct WeightTile {
     }
 };
 
-// ---- 4-bit, M <= 2: integer operands, scale and zero point taken out of the inner loop -------------------
+// ---- 4-bit, up to four MFMA rows (M x groups per chunk): integer operands, scale and zero point taken out of the inner loop ----
 //
 // A masked packed word is already a float16: bits 0-3 of a half are the subnormal q * 2^-24, bits 4-7 the
 // subnormal q * 2^-20, and the matrix core keeps subnormal inputs exactly.  So a word unpacks with one shift
@@ -957,7 +957,7 @@ int launch_w4(const GemvArgs& a, hipStream_t stream) {
     return launch_w4_kb<GROUP, MT, 2>(a, stream);
 }
 
-// ---- 8-bit, M <= 4: the same integer-operand scheme ---------------------------------------------------------
+// ---- 8-bit, up to four MFMA rows: the same integer-operand scheme ----------------------------------------------
 //
 // A byte in bits 0-7 of a half is the subnormal q * 2^-24, so a packed word becomes two operand dwords with two byte
 // permutes (bytes 0, 1 and bytes 2, 3, each byte zero-extended to a half): in natural k order, with a single
