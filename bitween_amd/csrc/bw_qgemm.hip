@@ -29,7 +29,7 @@ namespace {
 
 constexpr int WAVES = 4, NT = 4, BN = WAVES * NT * 16;   // a wave owns MT x NT MFMA tiles; MT = 8 or 16 (128 or 256 rows)
 
-template <int BITS, int GROUP, int MT = 8>
+template <int BITS, int GROUP, int MT = 8, bool NAT = false>
 struct GemmCfg {
     static constexpr int BM = MT * 16;
     // A lane takes WL adjacent 16-byte loads of a weight row per K step: VPL consecutive values.  Two loads
@@ -39,7 +39,7 @@ struct GemmCfg {
     static constexpr int WL = BITS == 8 ? 2 : 1;
     // bytes of a lane load: 16, except 8 at 2 bits with 256-row tiles - there a K step is 128 values like at the other
     // widths (a 256-value step of 256 rows of activations would not fit LDS twice)
-    static constexpr int LB = (BITS == 2 && MT == 16) ? 8 : 16;
+    static constexpr int LB = (BITS == 2 && NAT) ? 8 : 16;
     static constexpr int VPI = 32 / BITS, VPL = WL * LB * 8 / BITS, CHUNK_K = 4 * VPL, MF = VPL / 8;
     static constexpr int SPL = MF / WL;                          // MFMA steps per lane load
     static constexpr int CHUNK_BYTES = 4 * LB * WL;              // of a packed weight row
@@ -61,7 +61,7 @@ struct GemmCfg {
     static constexpr int PITCH = CHUNK_K + 8;                    // halves per LDS row
     // 128 rows: padded rows written by the staging threads; 256 rows: 256-byte rows written by buffer loads with LDS
     // destination, unpadded, the 16-byte slots of a row XOR-swizzled by the row number instead
-    static constexpr int STAGE_BYTES = MT == 16 ? BM * CHUNK_K * 2 : BM * PITCH * 2;
+    static constexpr int STAGE_BYTES = NAT ? BM * CHUNK_K * 2 : BM * PITCH * 2;
     static constexpr int UNIT = VPI > 8 ? VPI : 8;               // halves permuted together when staging x
     static constexpr int UW = UNIT / 8;
     static constexpr int UPR = CHUNK_K / UNIT;                   // staging units per x row
@@ -69,7 +69,7 @@ struct GemmCfg {
     static_assert(BM * UPR % (WAVES * 64) == 0, "tile must split evenly over the workgroup");
     // Activation fragments in registers: 128 rows - two sets of MT, the set of MFMA step t+1 read during step t;
     // 256 rows - a ring of 8, the fragment of slot i + 8 read when slot i has issued its MFMAs.
-    static constexpr int XSETS = MT == 8 ? 2 : 1, XRING = MT == 8 ? MT : 8;
+    static constexpr int XSETS = NAT ? 1 : 2, XRING = NAT ? 8 : MT;
 };
 
 template <int BITS>
@@ -193,9 +193,10 @@ BW_DEV __amdgpu_buffer_rsrc_t make_rsrc(const void* p, uint32_t bytes) {
 //   the activations of chunk c+1 were requested one step earlier and are written to buffer (c+1)&1 during
 //   step c, then re-requested for chunk c+2; the weights of chunk c+2 are requested into step c's own set
 //   once its last fragment is unpacked.  Every global load has a full K step (~2000 MFMA cycles) to land.
-template <int BITS, int GROUP, bool WIDE_META, int MT>
+template <int BITS, int GROUP, bool WIDE_META, int MT, bool NAT>
 __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
-    using C = GemmCfg<BITS, GROUP, MT>;
+    static_assert(NAT || MT == 8, "256-row tiles exist with the natural-order schedule only");
+    using C = GemmCfg<BITS, GROUP, MT, NAT>;
     constexpr int BM = C::BM;
     // WIDE_META (rows of scales on 4-byte boundaries): META4 = 8-byte requests over runs of K steps; PAIR = a lane whose
     // values span two groups fetches both scales (zero points) with one 4-byte request instead of two 2-byte ones
@@ -223,7 +224,7 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
         const int row = n0 + 16 * j + nl;
         // (256-row tiles add a scalar chunk offset that is itself "out of range" past the last chunk: rows past N then
         // read the last row's bytes instead of relying on a sum that could wrap; their outputs are never stored)
-        w_off[j] = row < a.N ? (uint32_t)row * a.row_bytes + kq * C::LB * C::WL : MT == 16 ? (uint32_t)(a.N - 1) * a.row_bytes + kq * C::LB * C::WL : kOob;
+        w_off[j] = row < a.N ? (uint32_t)row * a.row_bytes + kq * C::LB * C::WL : NAT ? (uint32_t)(a.N - 1) * a.row_bytes + kq * C::LB * C::WL : kOob;
         m_off[j] = (uint32_t)min(row, a.N - 1) * groups * 2;
     }
     // 128-row tiles: byte offsets of the staging units of a thread
@@ -291,7 +292,7 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
     // Weight fragment of MFMA step t: values [8 t, 8 t + 8) of the lane's VPL, from lane load t / SPL.
     auto unpack = [&](const WSet& ws, int j, int t, const auto* gcj) {
         static_assert(C::WL == 1 || C::NG == 1, "two lane loads share one group");
-        if constexpr (MT == 16) {                             // natural k order
+        if constexpr (NAT) {                                  // natural k order
             h2 o[4];
             if constexpr (BITS == 4) {
                 dequant_word4_nat(ws.w[j][0][t], gcj[0], o);
@@ -320,7 +321,7 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
     // count is exact.
     // `ph` (META4 only): position of the step in its run of four, a constant after inlining.
     static_assert(C::MF % 2 == 0, "the fragment double buffer returns to slot 0 at the end of a step");
-    using GC = std::conditional_t<MT == 16, GroupConstNat<BITS>, GroupConst<BITS>>;
+    using GC = std::conditional_t<NAT, GroupConstNat<BITS>, GroupConst<BITS>>;
     h8 xf[C::XSETS][C::XRING];
     h2 wf[2][NT][4];                                      // weight fragments as 4 register pairs each
     // group constants of tile j for the step that reads `from` (META4: half `half` of m_cur / m_next)
@@ -471,17 +472,18 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
     h2 up[NT][4];
     uint32_t uw[NT], pq[NT][2];
     const int wave_u = __builtin_amdgcn_readfirstlane(wave);
-    // activation loads: unit u of a wave = rows 64 wave + 4 u + (lane >> 4), lane & 15 = LDS slot
+    // activation loads: a wave brings in BM / 4 rows, 4 per instruction: unit u = rows RW wave + 4 u + (lane >> 4), lane & 15 = LDS slot
+    constexpr int RW = BM / WAVES;
     uint32_t xd_base[2];
 #pragma unroll
     for (int par = 0; par < 2; par++) {
         const int rr = 4 * par + (lane >> 4);
-        xd_base[par] = (uint32_t)((m0 + 64 * wave + rr) * a.ldx) * 2 + (((lane & 15) ^ (rr & 7)) * 16);
+        xd_base[par] = (uint32_t)((m0 + RW * wave + rr) * a.ldx) * 2 + (((lane & 15) ^ (rr & 7)) * 16);
     }
     auto x_dma16 = [&](int u, int cc, char* buf) {
         uint32_t so = cc < c_end ? (uint32_t)((u >> 1) * 8 * a.ldx) * 2 + (uint32_t)cc * C::CHUNK_K * 2 : kOob;
         asm("" : "+s"(so));                                   // one scalar sum, one VALU add
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, (__attribute__((address_space(3))) void*)(buf + (64 * wave_u + 4 * u) * 256), 16,
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, (__attribute__((address_space(3))) void*)(buf + (RW * wave_u + 4 * u) * 256), 16,
                                                  xd_base[u & 1] + so, 0, 0, 0);
     };
     auto w_req16 = [&](int j, int l, int cc, WSet& ws) {
@@ -498,8 +500,8 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
     uint32_t fa[4];
 #pragma unroll
     for (int t = 0; t < 4; t++) fa[t] = (uint32_t)(nl * 256 + (((4 * kq + t) ^ (nl & 7)) * 16));
-    auto step16 = [&](int c, const char* cur, char* nxt, WSet& ws, const WSet& wsn, auto& gc, auto& gn, const int ph) {
-        static_assert(MT != 16 || (C::NG == 1 && C::MF == 4 && C::CHUNK_K == 128 && C::XRING == 8), "layout of the 256-row schedule");
+    auto step16 = [&](int c, const char* cur, char* nxt, WSet& ws, const WSet& wsn, auto& gc, auto& gn, const int ph, const bool tail) {
+        static_assert(!NAT || (C::NG == 1 && C::MF == 4 && C::CHUNK_K == 128 && C::XRING == 8), "layout of the natural-order schedule");
         __builtin_amdgcn_sched_barrier(0);
         const uint32_t cur_a = (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) char*)cur;
         auto frag_read = [&](auto tc, auto ic) {
@@ -515,10 +517,12 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
             const WSet& src = early ? wsn : ws;
             constexpr int tt = early ? 0 : t + 1;
             static_for<0, 4 * MT>([&](auto gcnt) {
-                constexpr int g = decltype(gcnt)::value, i = g / NT, j = g % NT, r = g / 16, k = g % 16;
-                constexpr int S = 16 * t + i;
+                // RG gaps (SLOTS slots) per region: 16 (4) with 256-row tiles, 8 (2) with 128-row tiles
+                constexpr int RG = 4 * MT / NT, SLOTS = RG / 4;
+                constexpr int g = decltype(gcnt)::value, i = g / NT, j = g % NT, r = g / RG, k = g % RG;
+                constexpr int S = MT * t + i, SLAST = MT * C::MF - 1 - C::XRING;          // SLAST: the last slot that issues a fragment read
                 __builtin_amdgcn_sched_barrier(0);
-                if constexpr (j == 0) __builtin_amdgcn_s_waitcnt(0xC07F | ((7 - (S > 56 ? S - 56 : 0)) << 8));
+                if constexpr (j == 0) __builtin_amdgcn_s_waitcnt(0xC07F | ((C::XRING - 1 - (S > SLAST + 1 ? S - SLAST - 1 : 0)) << 8));
                 mfma_acc(acc[i][j], pack_h8(wf[cu][j]), xf[0][i % C::XRING]);
                 __builtin_amdgcn_sched_barrier(0);
                 // ---- unpack of n-tile r: instruction v of its sequence ----
@@ -564,17 +568,15 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
                 // MFMA rate; a second VALU instruction in a gap costs 3 cycles).  So the last gap of a slot belongs to the
                 // read; 8 bits puts its 12 instructions one into each other gap, 4 bits its 16 two into the first gap
                 // of each slot and one into the next two.
+                // With 128-row tiles a region has two slots for the same instructions: twice as many per gap (8 bits: two in
+                // each of the first three gaps; 4 and 2 bits: three, three and two, the read's gap still free).
                 constexpr int sl = k / 4;                                  // slot of the region
-                if constexpr (BITS != 8) {
-                    if constexpr (j == 0) {
-                        unpack_op(std::integral_constant<int, 4 * sl>{});
-                        unpack_op(std::integral_constant<int, 4 * sl + 1>{});
-                    } else if constexpr (j < 3) {
-                        unpack_op(std::integral_constant<int, 4 * sl + 1 + j>{});
-                    }
-                } else {
-                    if constexpr (j < 3) unpack_op(std::integral_constant<int, 3 * sl + j>{});
-                }
+                constexpr int OPS = BITS == 8 ? 12 : 16, PER_SLOT = OPS / SLOTS;          // (2 bits: 14 of the 16 do something)
+                // instructions of a slot in its gaps 0, 1, 2: PER_SLOT = 3 -> 1 1 1, 4 -> 2 1 1, 6 -> 2 2 2, 8 -> 3 3 2
+                constexpr int n0 = PER_SLOT == 3 ? 1 : PER_SLOT == 8 ? 3 : 2, n1 = PER_SLOT <= 4 ? 1 : PER_SLOT == 8 ? 3 : 2;
+                constexpr int first = sl * PER_SLOT + (j == 0 ? 0 : j == 1 ? n0 : n0 + n1);
+                constexpr int count = j == 0 ? n0 : j == 1 ? n1 : j == 2 ? PER_SLOT - n0 - n1 : 0;
+                static_for<0, count>([&](auto oc) { unpack_op(std::integral_constant<int, first + decltype(oc)::value>{}); });
                 // ---- the next chunk's activations: unit i of the wave in slot i of the first MFMA step ----
                 if constexpr (t == 0 && j == 1) x_dma16(i, c + 1, nxt);
                 // ---- fragment ring ----
@@ -583,37 +585,47 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
                     if constexpr (t2 < C::MF) frag_read(std::integral_constant<int, t2>{}, std::integral_constant<int, i2>{});
                 }
                 // ---- requests and constants (second gap of a slot) ----
-                if constexpr (t == 1 && j == 1 && sl >= 2) {
+                // two requests per region: slots 2 and 3 of four (second gap), or gaps 1 and 2 of the second slot of two
+                constexpr bool meta_here = SLOTS == 4 ? (j == 1 && sl >= 2) : (sl == 1 && (j == 1 || j == 2));
+                if constexpr (t == 1 && meta_here) {
+                    constexpr int which = SLOTS == 4 ? sl - 2 : j - 1;
                     if constexpr (META4) {
-                        if (ph == 0) issue_meta4(r, sl - 2, c + C::SPR, m_next);
+                        if (ph == 0) issue_meta4(r, which, c + C::SPR, m_next);
                     } else {
-                        issue_meta(r, sl - 2, c + 2, ws);
+                        issue_meta(r, which, c + 2, ws);
                     }
                 }
-                if constexpr (t == C::MF - 2 && k == 14) {
+                if constexpr (t == C::MF - 2 && k == RG - 2) {
                     if constexpr (META4) set_consts(gn[r], r, wsn, ph < C::SPR - 1 ? m_cur : m_next, ph < C::SPR - 1 ? ph + 1 : 0);
                     else set_consts(gn[r], r, wsn, m_cur, 0);
                 }
-                if constexpr (t == C::MF - 1 && j == 1 && sl >= 4 - C::WL) w_req16(r, sl - (4 - C::WL), c + 2, ws);
+                if constexpr (SLOTS == 4) {
+                    if constexpr (t == C::MF - 1 && j == 1 && sl >= 4 - C::WL) w_req16(r, sl - (4 - C::WL), c + 2, ws);
+                } else {                                                   // two slots: gaps 1 (and 2 at 8 bits) of the second
+                    if constexpr (t == C::MF - 1 && sl == 1 && j >= 1 && j <= C::WL) w_req16(r, j - 1, c + 2, ws);
+                }
                 asm volatile("" ::: "memory");
             });
         });
         __builtin_amdgcn_sched_barrier(0);
         // this wave's rows of the next chunk are in LDS once only the requests made after them are still in flight:
-        // the weights of the last MFMA step and, in a step that made them, the scales and zero points
-        if ((META4 && ph != 0)) wait_loads<NT * C::WL>();
+        // the weights of the last MFMA step and, in a step that made them, the scales and zero points.  That count
+        // holds inside the K loop, where every request feeds a later iteration; in the steps after the loop the
+        // compiler drops the requests nothing reads any more, so those steps wait for everything.
+        if (tail) wait_loads<0>();
+        else if ((META4 && ph != 0)) wait_loads<NT * C::WL>();
         else wait_loads<NT * C::WL + 2 * NT>();
         lds_barrier();
     };
     auto step = [&](int c, _Float16* cur, _Float16* nxt, WSet& ws, const WSet& wsn, GC (&gc)[NT][C::NG], GC (&gn)[NT][C::NG],
-                    const int ph) {
-        if constexpr (MT == 16) step16(c, reinterpret_cast<const char*>(cur), reinterpret_cast<char*>(nxt), ws, wsn, gc, gn, ph);
+                    const int ph, const bool tail = false) {
+        if constexpr (NAT) step16(c, reinterpret_cast<const char*>(cur), reinterpret_cast<char*>(nxt), ws, wsn, gc, gn, ph, tail);
         else step8(c, cur, nxt, ws, wsn, gc, gn, ph);
     };
 
     _Float16* buf0 = reinterpret_cast<_Float16*>(smem);
     _Float16* buf1 = reinterpret_cast<_Float16*>(smem + C::STAGE_BYTES);
-    if constexpr (MT == 16) {
+    if constexpr (NAT) {
         // Prologue of the 256-row tile: chunk c_begin's activations to the first buffer; scales and zero points and
         // the weights of the first two chunks in the order a steady-state step finds them outstanding.
         if constexpr (META4) {
@@ -624,7 +636,7 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
             }
         }
 #pragma unroll
-        for (int u = 0; u < 16; u++) x_dma16(u, c_begin, smem);
+        for (int u = 0; u < MT; u++) x_dma16(u, c_begin, smem);
 #pragma unroll
         for (int b = 0; b < 2; b++) {
             WSet& ws = b ? set1 : set0;
@@ -713,7 +725,7 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
 #pragma unroll
         for (int e = 0; e < 4; e++) wf[0][j][e] = h2{f[2 * e], f[2 * e + 1]};
     }
-    if constexpr (MT == 16) {
+    if constexpr (NAT) {
         wait_loads<NT * C::WL + (META4 ? 0 : 2 * NT)>();       // all but the second chunk's requests: the first buffer is written
         lds_barrier();
     } else {
@@ -737,8 +749,8 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
             for (int j = 0; j < NT; j++) { m_cur[j][0] = m_next[j][0]; m_cur[j][1] = m_next[j][1]; }
         }
         if (c < c_end) {                         // one or two steps left
-            step(c, buf0, buf1, set0, set1, gc0, gc1, 0);
-            step(c + 1, buf1, buf0, set1, set0, gc1, gc0, 1);
+            step(c, buf0, buf1, set0, set1, gc0, gc1, 0, true);
+            step(c + 1, buf1, buf0, set1, set0, gc1, gc0, 1, true);
         }
     } else {
         for (int c = c_begin; c < c_end; c += 2) {   // an odd chunk count runs one extra step on zeros
@@ -860,8 +872,8 @@ struct GemmPlan {
     size_t ws_bytes;
 };
 
-inline int gemm_chunks(int64_t K, int bits, int tile_rows = 128) {   // K steps of a whole row: GemmCfg::CHUNK_BYTES each
-    const int64_t chunk = bits == 8 ? 128 : (bits == 2 && tile_rows == 256) ? 32 : 64;
+inline int gemm_chunks(int64_t K, int bits, bool nat) {   // K steps of a whole row: GemmCfg::CHUNK_BYTES each
+    const int64_t chunk = bits == 8 ? 128 : (bits == 2 && nat) ? 32 : 64;
     return (int)((K * bits / 8 + chunk - 1) / chunk);
 }
 
@@ -892,20 +904,20 @@ inline GemmPlan gemm_plan(int64_t M, int64_t N, int nchunks, bool have_workspace
     return p;
 }
 
-template <int BITS, int GROUP, int MT = 8>
+template <int BITS, int GROUP, int MT, bool NAT>
 int launch_gemm(GemmArgs a, void* workspace, size_t workspace_bytes, hipStream_t stream) {
-    using C = GemmCfg<BITS, GROUP, MT>;
+    using C = GemmCfg<BITS, GROUP, MT, NAT>;
     constexpr int BM = C::BM;
-    static_assert(C::CHUNK_BYTES == (BITS == 8 ? 128 : (BITS == 2 && MT == 16) ? 32 : 64), "gemm_chunks() counts K steps of this size");
+    static_assert(C::CHUNK_BYTES == (BITS == 8 ? 128 : (BITS == 2 && NAT) ? 32 : 64), "gemm_chunks() counts K steps of this size");
     const size_t lds = 2 * (size_t)C::STAGE_BYTES;
-    void (*kern)(const GemmArgs) = qgemm_kernel<BITS, GROUP, false, MT>;
+    void (*kern)(const GemmArgs) = qgemm_kernel<BITS, GROUP, false, MT, NAT>;
     static uint64_t big_lds_devices[2] = {0, 0};           // per kernel
     int which = 0;
     if constexpr (C::CAN_META4 || C::NG == 2) {
         // an even number of K steps (so that the loop never pads with a step that would read past the row's scales)
         // and rows of scales on 4-byte boundaries
         if (a.groups % (C::CAN_META4 ? 2 * C::GPS : 2) == 0 && bw_aligned(a.scale, 4) && bw_aligned(a.zp, 4)) {
-            kern = qgemm_kernel<BITS, GROUP, true, MT>;
+            kern = qgemm_kernel<BITS, GROUP, true, MT, NAT>;
             which = 1;
         }
     }
@@ -928,16 +940,25 @@ int launch_gemm(GemmArgs a, void* workspace, size_t workspace_bytes, hipStream_t
     return BW_OK;
 }
 
+// The natural-order schedule (activations memory -> LDS by buffer loads with LDS destination, step16) takes whole K
+// steps of 128 values and offsets of rows past M that still fit 32 bits; other shapes run the register-staged kernel.
+inline bool gemm_nat(int64_t M, int64_t K, int64_t ldx) {
+#ifdef BW_TUNE   // measurement builds only (-DBW_TUNE, never the library build.py makes): kernel choices from the environment, for A/B runs
+    if (const char* e = getenv("BW_GEMM_NAT")) if (atoi(e) == 0) return false;
+#endif
+    return K % 128 == 0 && (M + 256) * ldx * 2 < ((int64_t)1 << 32);
+}
+
 // Rows of a tile for this call.  A 256-row tile unpacks every weight once for twice the rows and keeps the matrix pipe
-// busier (step16) - when its grid fills the device.  Measured at 4 and 8 bits, K and N from 4096 to 14336, M from 256
+// busier - when its grid fills the device.  Measured at 4 and 8 bits, K and N from 4096 to 14336, M from 256
 // to 4096: the 256-row grid wins by 5-20 % from about 0.6 rounds of tiles on and loses up to 25 % below, except that
 // with a long K (80 K steps and more) and a workspace to split it, a quarter of a round is enough (14336 -> 4096 at
-// 1024 and 2048 rows: 6-13 %).  Only for whole K steps of 128 values, and only while the split-K blocks of its plan fit
-// the workspace on offer.  (The K steps counted here are those of the 256-row kernel: 128 values at every width.)
+// 1024 and 2048 rows: 6-13 %).  Only with the natural-order schedule, and only while the split-K blocks of its plan
+// fit the workspace on offer.
 inline int gemm_tile_rows(int64_t M, int64_t N, int64_t K, int64_t ldx, int bits, bool have_workspace, size_t workspace_bytes) {
-    if (K % 128 || (M + 256) * ldx * 2 >= ((int64_t)1 << 32)) return 128;
-    const int nchunks = gemm_chunks(K, bits, 256);
-#ifdef BW_TUNE   // measurement builds only (-DBW_TUNE, never the library build.py makes): the tile height from the environment, for A/B runs
+    if (!gemm_nat(M, K, ldx)) return 128;
+    const int nchunks = gemm_chunks(K, bits, true);
+#ifdef BW_TUNE
     if (const char* e = getenv("BW_GEMM_BM")) return atoi(e) == 256 ? 256 : 128;
 #endif
     const int64_t tiles = ((N + BN - 1) / BN) * ((M + 255) / 256), cus = bw_device_cus();
@@ -1029,10 +1050,17 @@ int bw_qgemm_generic(const void* x, int act_dtype, int64_t M, int64_t K, int64_t
 
 extern "C" size_t bw_qgemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int bits, int group) {
     if (!bw_shape_ok(N, K, bits, group) || M < 1 || M >= ((int64_t)1 << 31) || !bw_fast_shape(M, N, K, K, bits, group)) return 0;
-    const size_t small = gemm_plan(M, N, gemm_chunks(K, bits), true, 128).ws_bytes;     // either plan may run: enough for both
-    if (gemm_tile_rows(M, N, K, K, bits, true, ~(size_t)0) == 128) return small;
-    const size_t big = gemm_plan(M, N, gemm_chunks(K, bits, 256), true, 256).ws_bytes;
-    return big > small ? big : small;
+    // any of the plans may run (the call's own ldx and workspace decide): enough for each of them
+    size_t need = gemm_plan(M, N, gemm_chunks(K, bits, false), true, 128).ws_bytes;
+    if (gemm_nat(M, K, K)) {
+        const size_t nat128 = gemm_plan(M, N, gemm_chunks(K, bits, true), true, 128).ws_bytes;
+        if (nat128 > need) need = nat128;
+        if (gemm_tile_rows(M, N, K, K, bits, true, ~(size_t)0) == 256) {
+            const size_t big = gemm_plan(M, N, gemm_chunks(K, bits, true), true, 256).ws_bytes;
+            if (big > need) need = big;
+        }
+    }
+    return need;
 }
 
 extern "C" int bw_qgemm_tile_rows(int64_t M, int64_t N, int64_t K, int bits, int group) {
@@ -1055,7 +1083,8 @@ extern "C" int bw_qgemm_ws(const void* x, int act_dtype, int64_t M, int64_t K, i
     a.M = (int)M; a.N = (int)N; a.K = (int)K; a.ldx = (int)ldx; a.ldy = (int)ldy;
     a.groups = (int)(K / group);
     a.row_bytes = (int)(K * bits / 8);
-    a.nchunks = gemm_chunks(K, bits);
+    const bool nat = gemm_nat(M, K, ldx);
+    a.nchunks = gemm_chunks(K, bits, nat);
     a.x_bytes = (uint32_t)(((M - 1) * ldx + K) * 2);
     a.w_bytes = (uint32_t)(N * a.row_bytes);
     a.meta_bytes = (uint32_t)(N * a.groups * 2);
@@ -1064,17 +1093,16 @@ extern "C" int bw_qgemm_ws(const void* x, int act_dtype, int64_t M, int64_t K, i
     a.splits = 1;
     a.chunks_per_split = a.nchunks;
     hipStream_t st = (hipStream_t)stream;
-    const bool big = gemm_tile_rows(M, N, K, ldx, bits, workspace != nullptr, workspace_bytes) == 256;
-    if (big) a.chunks_per_split = a.nchunks = gemm_chunks(K, bits, 256);
-#define BW_CASE(B, G) \
-    if (bits == B && group == G) return launch_gemm<B, G>(a, workspace, workspace_bytes, st);
-#define BW_CASE2(B, G) \
-    if (bits == B && group == G) return big ? launch_gemm<B, G, 16>(a, workspace, workspace_bytes, st) : launch_gemm<B, G>(a, workspace, workspace_bytes, st);
-    BW_CASE2(4, 128) BW_CASE2(4, 64) BW_CASE2(4, 32)
-    BW_CASE2(8, 128) BW_CASE2(8, 64) BW_CASE2(8, 32)
-    BW_CASE2(2, 128) BW_CASE2(2, 64) BW_CASE2(2, 32)
+    const bool big = nat && gemm_tile_rows(M, N, K, ldx, bits, workspace != nullptr, workspace_bytes) == 256;
+#define BW_CASE(B, G)                                                                               \
+    if (bits == B && group == G)                                                                     \
+        return big   ? launch_gemm<B, G, 16, true>(a, workspace, workspace_bytes, st)                \
+               : nat ? launch_gemm<B, G, 8, true>(a, workspace, workspace_bytes, st)                 \
+                     : launch_gemm<B, G, 8, false>(a, workspace, workspace_bytes, st);
+    BW_CASE(4, 128) BW_CASE(4, 64) BW_CASE(4, 32)
+    BW_CASE(8, 128) BW_CASE(8, 64) BW_CASE(8, 32)
+    BW_CASE(2, 128) BW_CASE(2, 64) BW_CASE(2, 32)
 #undef BW_CASE
-#undef BW_CASE2
     return BW_EUNSUPPORTED;
 }
 

@@ -906,11 +906,12 @@ def test_sibling_group_does_not_serve_a_member_twice_from_its_cache():
 
 
 @pytest.mark.parametrize("bits,g", [(4, 128), (4, 64), (4, 32), (8, 128), (8, 64), (8, 32), (2, 128), (2, 64), (2, 32)])
-@pytest.mark.parametrize("k", [896, 1024])
+@pytest.mark.parametrize("k", [768, 896, 1024])
 def test_prefill_256_row_tiles_vs_oracle(bits, g, k):
     """Shapes whose grid of 256-row tiles fills the device take the 256-row variant of the prefill kernel (same
     arithmetic as bitween/modules.py:85-97, twice the rows per unpacked weight): ragged in M and N, an even and an odd
-    number of K steps (with and without the wide scale requests), with and without bias - sampled rows from every part
+    number of K steps (with and without the wide scale requests; 768 = six steps: a run of four and two steps after
+    the loop), with and without bias - sampled rows from every part
     of the row range against the oracle, one-hot rows bit for bit, and the workspace plan against the plain one."""
     import ctypes
     hip = _hip()
