@@ -950,19 +950,29 @@ inline bool gemm_nat(int64_t M, int64_t K, int64_t ldx) {
 }
 
 // Rows of a tile for this call.  A 256-row tile unpacks every weight once for twice the rows and keeps the matrix pipe
-// busier - when its grid fills the device.  Measured at 4 and 8 bits, K and N from 4096 to 14336, M from 256
-// to 4096: the 256-row grid wins by 5-20 % from about 0.6 rounds of tiles on and loses up to 25 % below, except that
-// with a long K (80 K steps and more) and a workspace to split it, a quarter of a round is enough (14336 -> 4096 at
-// 1024 and 2048 rows: 6-13 %).  Only with the natural-order schedule, and only while the split-K blocks of its plan
-// fit the workspace on offer.
+// busier: a full round of 256-row tiles takes about 1.65 x the time of a full round of 128-row tiles for twice the
+// work.  Which grid finishes first then depends on how each fills its rounds (one workgroup per CU): whole rounds,
+// plus a last round that costs a full one when more than half full and about three quarters of one when its tiles are
+// split along K (a workspace is on offer).  That model reproduces a sweep of both heights over K, N in {4096, 11008,
+// 14336} and M = 512 ... 2048 (4 bits; e.g. 4096 -> 14336 at 2048 rows: 3.75 against 3.3 rounds, measured 207 against
+// 184 us; 4096 x 4096 at 2048 rows: 1.0 against 1.24, measured 60 against 75 us); the 256-row grid is taken when it is
+// ahead by 5 % or more.  Only with the natural-order schedule, and only while the split-K blocks of its plan fit the
+// workspace on offer.
 inline int gemm_tile_rows(int64_t M, int64_t N, int64_t K, int64_t ldx, int bits, bool have_workspace, size_t workspace_bytes) {
     if (!gemm_nat(M, K, ldx)) return 128;
     const int nchunks = gemm_chunks(K, bits, true);
 #ifdef BW_TUNE
     if (const char* e = getenv("BW_GEMM_BM")) return atoi(e) == 256 ? 256 : 128;
 #endif
-    const int64_t tiles = ((N + BN - 1) / BN) * ((M + 255) / 256), cus = bw_device_cus();
-    if (tiles * 5 < cus * 3 && !(have_workspace && tiles * 4 >= cus && nchunks >= 80)) return 128;
+    const int64_t cus = bw_device_cus();
+    auto rounds = [&](int64_t tiles) {
+        const int64_t full = tiles / cus, rest = tiles % cus;
+        const bool split = have_workspace && nchunks >= 8 && rest <= cus / 2;
+        return (double)full + (rest == 0 ? 0.0 : split ? 0.75 : 1.0);
+    };
+    const int64_t tiles_n = (N + BN - 1) / BN;
+    const double t128 = rounds(tiles_n * ((M + 127) / 128)), t256 = 1.65 * rounds(tiles_n * ((M + 255) / 256));
+    if (t256 > 0.95 * t128) return 128;
     if (have_workspace && gemm_plan(M, N, nchunks, true, 256).ws_bytes > workspace_bytes) return 128;
     return 256;
 }

@@ -64,8 +64,9 @@ def test_split_k_workspace_size_is_a_pure_host_function():
     # whole rounds of 256 tiles (one workgroup per CU), or a last round that is more than half full: no workspace
     assert ws(2048, 4096, 4096, 4, 128) == 0 and rows(2048, 4096, 4096, 4, 128) == 128    # 16 x 16 tiles = exactly one round
     assert ws(4096, 4096, 4096, 4, 128) == 0 and rows(4096, 4096, 4096, 4, 128) == 256    # 512 tiles of 128 rows, or 256 of 256
-    # a long K with a quarter round of 256-row tiles and more: those, every tile cut in two (128 tiles x 2 slices of 256 x 256)
-    assert rows(2048, 4096, 14336, 4, 128) == 256 and ws(2048, 4096, 14336, 4, 128) == 128 * 2 * 2 * tile
+    # the tile height is the one whose grid fills its rounds better: 1.75 rounds of 128-row tiles against one of 256-row tiles
+    assert rows(1024, 14336, 4096, 4, 128) == 256 and rows(2048, 14336, 4096, 4, 128) == 256 and rows(2048, 4096, 14336, 4, 128) == 128
+    assert ws(2048, 4096, 14336, 4, 128) == 0                    # 256 tiles of 128 rows: exactly one round
     # 256-row tiles need whole K steps of 128 values and a grid that fills the device
     assert rows(4096, 4096, 4096, 2, 128) == 256 and rows(4096, 4096, 4096 + 64, 4, 64) == 128 and rows(512, 14336, 4096, 4, 128) == 128
     assert rows(128, 20, 96, 4, 48) == 0                        # the shape-generic kernel
