@@ -1147,12 +1147,14 @@ extern "C" int bw_qgemm(const void* x, int act_dtype, int64_t M, int64_t K, int6
 }
 
 // Rows up to which bw_qlinear stays on the decode kernel (16 rows per launch; the later launches find the weights
-// in L2 / Infinity Cache).  Two launches always beat a mostly empty 128-row MFMA tile; a third does only while the
-// packed weights are small (4096 x 4096 at 4 or 8 bits: 13-17 us against 17-20 us), not for 20 MiB and more
-// (4096 x 11008 at 4 bits: 24-28 us against 22-23 us; at 8 bits 37-41 against 27).
+// in L2 / Infinity Cache).  Two launches always beat a mostly empty 128-row MFMA tile for small layers; a third does only
+// while the packed weights are small (4096 x 4096 at 4 or 8 bits: 15-18 us against 18-19 us), not for 20 MiB and more
+// (4096 x 11008 at 4 bits: 21-24 us against 21.5-22 us); from 40 MiB on (4096 x 11008 at 8 bits) even the second launch
+// loses to the prefill kernel (26.9 against 22.2 us at 32 rows, 22.1 against 21.6 at 17).
 extern "C" int bw_qlinear_decode_rows(int64_t N, int64_t K, int bits) {
     if (N < 1 || K < 1 || !bw_bits_ok(bits)) return 0;
-    return N * (K * bits / 8) < ((int64_t)20 << 20) ? 48 : 32;
+    const int64_t bytes = N * (K * bits / 8);
+    return bytes < ((int64_t)20 << 20) ? 48 : bytes < ((int64_t)40 << 20) ? 32 : 16;
 }
 
 extern "C" int bw_qlinear(const void* x, int act_dtype, int64_t M, int64_t K, int64_t ldx, const int32_t* qweight,

@@ -198,8 +198,8 @@ def _matmul(entry, x, qweight, scale, zero_point, bias, bits, group_size):
     if qweight.dtype is not torch.int32 or scale.dtype is not torch.float16 or zero_point.dtype is not torch.float16:
         raise TypeError("qweight must be int32 and scale / zero_point float16 (the QuantizedLinear buffers)")
     m = x.shape[0]
-    # rows that bw_qlinear keeps on the decode kernel: 32, and up to 48 for small layers
-    decode_rows = 32 if m <= 32 or entry != "bw_qlinear" else load().bw_qlinear_decode_rows(qweight.shape[0], x.shape[1], bits)
+    # rows that bw_qlinear keeps on the decode kernel: always 16, and 32 or 48 for layers that are not too large
+    decode_rows = 16 if m <= 16 or entry != "bw_qlinear" else load().bw_qlinear_decode_rows(qweight.shape[0], x.shape[1], bits)
     act = BW_F16
     if x.dtype is torch.bfloat16:
         # the decode kernels round bfloat16 to float16 as they stage x (the reference's x.to(float16),

@@ -85,12 +85,12 @@ def test_split_k_workspace_size_is_a_pure_host_function():
 
 
 def test_decode_rows_switch_is_a_pure_host_function():
-    """bw_qlinear keeps up to 48 rows on the decode kernel for small layers and 32 for 20 MiB of packed weights and
-    more (three 16-row launches over a large layer lose to one prefill launch)."""
+    """bw_qlinear keeps up to 48 rows on the decode kernel for small layers, 32 for 20 MiB of packed weights and more
+    (three 16-row launches over a large layer lose to one prefill launch) and 16 from 40 MiB on."""
     from bitween_amd.kernels import hip_loader
     rows = hip_loader.load().bw_qlinear_decode_rows
     assert rows(4096, 4096, 4) == 48 and rows(4096, 4096, 8) == 48 and rows(4096, 11008, 2) == 48
-    assert rows(11008, 4096, 4) == 32 and rows(4096, 11008, 8) == 32 and rows(14336, 4096, 4) == 32
+    assert rows(11008, 4096, 4) == 32 and rows(14336, 4096, 4) == 32 and rows(4096, 11008, 8) == 16 and rows(12288, 4096, 8) == 16
     assert rows(0, 4096, 4) == 0 and rows(4096, 4096, 3) == 0
 
 

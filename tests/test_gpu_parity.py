@@ -775,19 +775,21 @@ def test_forward_under_graph_capture_replays_like_eager(m, dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
-def test_rows_33_to_48_on_a_large_layer_take_the_prefill_kernel(dtype):
-    """For a layer of 20 MiB of packed weights and more bw_qlinear hands 33-48 rows to the prefill kernel; the module
-    forward (validated-buffer path, bfloat16 cast included) must follow it and agree with the C entry point."""
+@pytest.mark.parametrize("bits,switch,ms", [(4, 32, (32, 33, 40, 48)), (8, 16, (16, 17, 32, 33))])
+def test_rows_33_to_48_on_a_large_layer_take_the_prefill_kernel(dtype, bits, switch, ms):
+    """For a layer of 20 MiB of packed weights and more bw_qlinear hands 33-48 rows to the prefill kernel, from 40 MiB on
+    (4096 -> 11008 at 8 bits) 17-32 rows too; the module forward (validated-buffer path, bfloat16 cast included) must
+    follow it and agree with the C entry point."""
     import ctypes
     from bitween_amd import QuantizedLinear
     from bitween_amd.kernels import hip_loader as hip
     lib = hip.load()
-    k, n, bits, g = 4096, 11008, 4, 128
-    assert lib.bw_qlinear_decode_rows(n, k, bits) == 32
+    k, n, g = 4096, 11008, 128
+    assert lib.bw_qlinear_decode_rows(n, k, bits) == switch
     lin = torch.nn.Linear(k, n, bias=True, dtype=torch.float16, device="cuda")
     q = QuantizedLinear.from_float(lin, bits=bits, group_size=g)
     w16 = hip.dequantize(q.qweight, q.scale, q.zero_point, g, bits, torch.float16)
-    for m in (32, 33, 40, 48):
+    for m in ms:
         x = torch.randn(m, k, device="cuda").to(dtype)
         with torch.no_grad():
             y = q(x)
@@ -800,7 +802,7 @@ def test_rows_33_to_48_on_a_large_layer_take_the_prefill_kernel(dtype):
                             q.bias.data_ptr(), n, bits, g, yc.data_ptr(), n, ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
         assert st == 0
         torch.cuda.synchronize()
-        if m <= 32:
+        if m <= switch:
             assert torch.equal(y, yc)                            # same decode launches either way
         else:
             assert ((y.double() - yc.double()).abs() <= 2.0 ** -9 * ref.abs() + 2.0 ** -12 * mag).all()   # split-K or not
