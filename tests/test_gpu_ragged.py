@@ -161,3 +161,35 @@ def test_quantize_dequantize_ragged(bits, g, n, k):
     assert (out[:, k:] == 3.0).all()
     expect = (s_o.repeat(g, axis=1) * (orc.unpack_words(qw_o, bits).astype(np.float32) - z_o.repeat(g, axis=1).astype(np.float32)))
     assert np.array_equal(out[:, :k].cpu().numpy().view(np.uint32), expect.astype(np.float32).view(np.uint32))
+
+
+@pytest.mark.parametrize("bits,g", [(4, 128), (8, 64), (2, 32)])
+@pytest.mark.parametrize("m,n,k,ypad", [(300, 320, 512, 8), (300, 330, 640, 16), (129, 64, 256, 8), (256 * 52 + 5, 1000, 384, 8)])
+def test_prefill_padded_rows_of_x_and_y(bits, g, m, n, k, ypad):
+    """Prefill through the C ABI with padded rows on both sides: x rows K + 8 apart with NaN in the padding (never
+    read: the activations go to LDS by buffer loads of whole 16-byte pieces), y rows N + ypad apart (a multiple of 8,
+    so the whole-row stores of the LDS epilogue run where a wave's 64 columns lie inside N, the piecewise stores
+    elsewhere) - nothing may be written past a row's N outputs.  Both tile heights (the last case has 53 row tiles)."""
+    from bitween_amd.kernels import hip_loader
+    lib = hip_loader.load()
+    _, qw, s16, z16, b16 = quantized_layer(n, k, bits, g, seed=m + n + k + bits, outliers=True)
+    gen = torch.Generator(device="cuda").manual_seed(m + k)
+    x = torch.randn(m, k, device="cuda", generator=gen).half()
+    ldx, ldy = k + 8, n + ypad
+    xbuf = torch.full((m, ldx), float("nan"), dtype=torch.float16, device="cuda")
+    xbuf[:, :k] = x
+    d = [to_gpu(a) for a in (qw, s16, z16, b16)]
+    need = lib.bw_qgemm_workspace_bytes(m, n, k, bits, g)
+    ws = torch.empty(max(need, 16), dtype=torch.uint8, device="cuda")
+    y = torch.full((m, ldy), 7.0, dtype=torch.float16, device="cuda")
+    st = lib.bw_qgemm_ws(xbuf.data_ptr(), 0, m, k, ldx, d[0].data_ptr(), d[1].data_ptr(), d[2].data_ptr(), d[3].data_ptr(), n, bits, g,
+                         y.data_ptr(), ldy, ws.data_ptr() if need else None, need, ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    assert st == 0
+    torch.cuda.synchronize()
+    assert (y[:, n:] == 7.0).all()
+    rows = np.unique(np.concatenate([np.arange(0, m, max(1, m // 40)), np.arange(max(0, m - 6), m)]))
+    idx = torch.from_numpy(rows).cuda()
+    check_matmul(y[idx][:, :n], x[idx].cpu().numpy(), qw, s16, z16, b16, bits, g)
+    w16 = to_gpu(orc.dequantize_f16(qw, s16, z16, g, bits))
+    ref = (x @ w16.T).float() + to_gpu(b16).float()
+    assert ((y[:, :n].float() - ref).abs().max() <= 2.0 ** -8 * ref.abs().max()).item()
