@@ -181,7 +181,22 @@ struct GemmArgs {
     float* ws;
     int tiles_n, full_tiles, splits, chunks_per_split;
     int bm;                                        // rows of a tile: 128 or 256
+    // Order of the tiles.  Tile t sits in panel t / (panel * tiles_n) of `panel` m-tiles, n-major inside the panel, so
+    // consecutive tiles form blocks a few m-tiles high.  Workgroup ids go to the 8 XCDs round-robin; id i < xcd_tiles (a
+    // multiple of 8) takes tile (i % 8) * xcd_tiles / 8 + i / 8: an XCD works through one contiguous eighth of the tile
+    // order, and the 32 workgroups it runs together share `panel` activation tiles and 32 / panel weight tiles in its L2
+    // instead of every activation tile (plain row-major ids give an XCD every 8th tile: all m-tiles and few n-tiles
+    // whenever tiles_n is a multiple of 8).
+    int tiles_m, panel, xcd_tiles;
 };
+
+BW_DEV void tile_coords(int tile, const GemmArgs& a, int& tm, int& tn) {
+    const int per_panel = a.panel * a.tiles_n;
+    const int p = tile / per_panel, within = tile - p * per_panel;
+    const int rows = min(a.panel, a.tiles_m - p * a.panel);
+    tn = within / rows;
+    tm = p * a.panel + (within - tn * rows);
+}
 
 BW_DEV __amdgpu_buffer_rsrc_t make_rsrc(const void* p, uint32_t bytes) {
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), (short)0, (int)bytes, 0x00020000);
@@ -208,9 +223,11 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
     const int id = (int)blockIdx.x;
     const bool partial = id >= a.full_tiles;
     const int run = partial ? id - a.full_tiles : 0;
-    const int tile = partial ? a.full_tiles + run / a.splits : id;
-    const int m0 = (tile / a.tiles_n) * BM;
-    const int n0 = (tile % a.tiles_n) * BN + wave * (NT * 16);
+    const int tile = partial ? a.full_tiles + run / a.splits : id < a.xcd_tiles ? (id & 7) * (a.xcd_tiles >> 3) + (id >> 3) : id;
+    int tm, tn;
+    tile_coords(tile, a, tm, tn);
+    const int m0 = tm * BM;
+    const int n0 = tn * BN + wave * (NT * 16);
     const int groups = a.groups;
     // a partial workgroup takes chunks [c_begin, c_end); requests beyond c_end read as zero
     const int c_begin = partial ? (run % a.splits) * a.chunks_per_split : 0;
@@ -840,7 +857,9 @@ __global__ __launch_bounds__(256) void qgemm_reduce_kernel(const GemmArgs a) {
     const int tile = a.full_tiles + (int)blockIdx.y;
     const int quad = (int)(blockIdx.x * blockDim.x + threadIdx.x);          // < bm * BN / 4
     const int ml = quad / (BN / 4), nl4 = (quad % (BN / 4)) * 4;
-    const int m = (tile / a.tiles_n) * a.bm + ml, n = (tile % a.tiles_n) * BN + nl4;
+    int tm, tn;
+    tile_coords(tile, a, tm, tn);
+    const int m = tm * a.bm + ml, n = tn * BN + nl4;
     if (m >= a.M || n >= a.N) return;
     const size_t blk = (size_t)a.bm * BN;
     const float* src = a.ws + (size_t)blockIdx.y * a.splits * blk + ml * BN + nl4;
@@ -927,6 +946,16 @@ int launch_gemm(GemmArgs a, void* workspace, size_t workspace_bytes, hipStream_t
     a.ws = (float*)workspace;
     a.bm = BM;
     a.tiles_n = p.tiles_n;
+    a.tiles_m = p.tiles / p.tiles_n;
+    a.panel = a.tiles_m < 4 ? a.tiles_m : 4;
+    a.xcd_tiles = p.full_tiles & ~7;
+#ifdef BW_TUNE
+    if (const char* e = getenv("BW_GEMM_PANEL")) {
+        const int v = atoi(e);
+        if (v <= 0) { a.panel = 1; a.xcd_tiles = 0; }
+        else a.panel = a.tiles_m < v ? a.tiles_m : v;
+    }
+#endif
     a.full_tiles = p.full_tiles;
     a.splits = p.splits;
     a.chunks_per_split = p.chunks_per_split;
@@ -1100,6 +1129,8 @@ extern "C" int bw_qgemm_ws(const void* x, int act_dtype, int64_t M, int64_t K, i
     a.meta_bytes = (uint32_t)(N * a.groups * 2);
     a.ws = nullptr;
     a.tiles_n = a.full_tiles = 0;
+    a.tiles_m = a.panel = 1;
+    a.xcd_tiles = 0;
     a.splits = 1;
     a.chunks_per_split = a.nchunks;
     hipStream_t st = (hipStream_t)stream;
