@@ -283,6 +283,40 @@ def extras_hipblaslt_decode(torch, hip, QuantizedLinear, layers):
     return out
 
 
+def sclk_under_load(torch, fn, seconds=0.4, batch=200):
+    """Mean / min of the driver's current shader clock (sysfs pp_dpm_sclk, MHz) sampled while batches of `fn` are in
+    flight; None where the file is absent or unreadable.  A slow average that includes the gaps between launches:
+    it ranks loads, the in-kernel counters of board_probes measure one."""
+    import glob
+    import re
+    import time
+    files = glob.glob("/sys/class/drm/card*/device/pp_dpm_sclk")
+    if len(files) != 1:
+        return None            # no file, or several cards and no way to tell which one is this process's
+    def read():
+        try:
+            for line in open(files[0]).read().split("\n"):
+                if "*" in line:
+                    m = re.search(r"(\d+)\s*[Mm]hz", line)
+                    if m:
+                        return int(m.group(1))
+        except OSError:
+            pass
+        return None
+    torch.cuda.synchronize()
+    samples, t_end = [], time.time() + seconds
+    while time.time() < t_end:
+        for _ in range(batch):
+            fn()
+        v = read()                                     # taken with the batch still in flight
+        torch.cuda.synchronize()
+        if v is None:
+            return None
+        samples.append(v)
+    samples = samples[2:] or samples
+    return {"mean_MHz": round(sum(samples) / len(samples)), "min_MHz": min(samples), "samples": len(samples)}
+
+
 def extras_prefill(torch, hip, QuantizedLinear, layers):
     """Prefill on the Llama-3-8B MLP shapes, W4 g128, next to fp16 hipBLASLt on the dequantised weights.  `us` is
     the kernel on float16 x; `bf16_x_us` the forward on bfloat16 x (cast + split-K workspace + kernel); `tile_rows` the
@@ -307,7 +341,70 @@ def extras_prefill(torch, hip, QuantizedLinear, layers):
                                      "pct_mfma_f16_peak": round(100 * fl / us_q / 1e6 / MFMA_F16_PEAK_TFLOPS, 1),
                                      "hipblaslt_fp16_us": round(us_b, 1), "hipblaslt_fp16_TFLOPs": round(fl / us_b / 1e6, 1),
                                      "frac_of_hipblaslt": round(us_b / us_q, 3)}
+            if (k, n, mm) == (4096, 14336, 2048):
+                # both kernels run this shape at the part's power limit: the clock each is allowed
+                out["sclk_under_load_4096x14336_M2048"] = {
+                    "this_kernel": sclk_under_load(torch, lambda: hip.quantized_gemm_hip(x, q.qweight, q.scale, q.zero_point, None, bits, g)),
+                    "hipblaslt_fp16": sclk_under_load(torch, lambda: torch.matmul(x, w16.T))}
         del q, w16
+    return out
+
+
+def extras_prefill_clock(torch, hip, QuantizedLinear, layers):
+    """The shader clock inside the prefill kernel.  The measurement build of the library (python -m
+    bitween_amd.csrc.build --tune) lets workgroups 0..255 of a launch leave the core-clock ticks and the real-time
+    ticks of their K loop in a buffer; ticks / ticks x the real-time rate is the clock the part allowed under that
+    load, cycles / MFMAs how close the loop is to the bare MFMA stream (board_probes: 18.4 cycles per MFMA and wave
+    at 2.27 GHz with nothing else going on).  `us` is the whole call of the measurement build, for orientation."""
+    import ctypes
+    from bitween_amd.csrc import build as hip_build
+    if not os.path.exists(hip_build.TUNE_LIB):
+        return {"skipped": "libbitween_hip_tune.so is not built (python -m bitween_amd.csrc.build --tune)"}
+    lib = ctypes.CDLL(hip_build.TUNE_LIB)
+    vp, i64, i32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int
+    lib.bw_abi_version.restype = i32
+    if lib.bw_abi_version() != hip.ABI_VERSION:
+        return {"skipped": "libbitween_hip_tune.so is stale (ABI %d): rebuild it" % lib.bw_abi_version()}
+    lib.bw_qgemm_ws.argtypes = [vp, i32, i64, i64, i64, vp, vp, vp, vp, i64, i32, i32, vp, i64, vp, ctypes.c_size_t, vp]
+    lib.bw_qgemm_ws.restype = i32
+    lib.bw_qgemm_workspace_bytes.argtypes, lib.bw_qgemm_workspace_bytes.restype = [i64, i64, i64, i32, i32], ctypes.c_size_t
+    lib.bw_qgemm_tile_rows.argtypes, lib.bw_qgemm_tile_rows.restype = [i64, i64, i64, i32, i32], i32
+    lib.bw_tune_clock_buffer.argtypes = [vp]
+    # the real-time counter's rate: 100 MHz on this part (hipDeviceAttributeWallClockRate); torch does not expose it
+    tick_hz = 100e6
+    clk = torch.zeros(512, device="cuda", dtype=torch.int64)
+    out = {}
+    stream = torch.cuda.current_stream().cuda_stream
+    for bits, g, k, n, mm in ((4, 128, 4096, 8192, 2048), (4, 128, 4096, 14336, 2048), (4, 128, 14336, 4096, 2048), (4, 128, 4096, 14336, 512),
+                              (4, 128, 4096, 14336, 128), (8, 128, 4096, 14336, 2048), (2, 32, 4096, 14336, 2048)):
+        q = make_layer(torch, QuantizedLinear, k, n, bits, g, seed=7)
+        x = torch.randn(mm, k, device="cuda", dtype=torch.float16)
+        y = torch.empty(mm, n, device="cuda", dtype=torch.float16)
+        ws = torch.empty(max(16, lib.bw_qgemm_workspace_bytes(mm, n, k, bits, g)), device="cuda", dtype=torch.uint8)
+        def call():
+            st = lib.bw_qgemm_ws(x.data_ptr(), 0, mm, k, k, q.qweight.data_ptr(), q.scale.data_ptr(), q.zero_point.data_ptr(), None, n, bits, g,
+                                 y.data_ptr(), n, ws.data_ptr(), ws.numel(), stream)
+            assert st == 0, st
+        lib.bw_tune_clock_buffer(None)
+        us = min(time_calls(torch, call, 20, 30) for _ in range(2))    # (the first large GEMMs of a fresh process run slow)
+        clk.zero_()
+        lib.bw_tune_clock_buffer(clk.data_ptr())
+        for _ in range(30):
+            call()
+        torch.cuda.synchronize()
+        lib.bw_tune_clock_buffer(None)
+        d = clk.cpu().view(256, 2).double()
+        d = d[d[:, 1] > 0]
+        rows = lib.bw_qgemm_tile_rows(mm, n, k, bits, g)
+        # MFMAs of one wave in a whole-K loop: (rows / 16) x 4 tiles x K / 32
+        mfmas = rows // 16 * 4 * k // 32
+        cycles = d[:, 0].mean().item()
+        out[f"w{bits}g{g}_{k}x{n}_M{mm}"] = {"us": round(us, 1), "tile_rows": rows, "k_loop_us": round(d[:, 1].mean().item() / tick_hz * 1e6, 1),
+                                           "shader_clock_GHz": round((d[:, 0] / d[:, 1]).mean().item() * tick_hz / 1e9, 3),
+                                           "k_loop_kcycles": round(cycles / 1e3, 1), "cycles_per_mfma": round(cycles / mfmas, 1)}
+        del q, x, y, ws
+    out["note"] = ("workgroups of split tiles run a slice of K: their cycles_per_mfma reads low where the first 256 workgroups "
+                   "include them (M = 128)")
     return out
 
 
@@ -658,6 +755,15 @@ def extras_board_probes(torch, hip, QuantizedLinear, layers):
     out["mfma_16x16x32_f16_ns_per_wave"] = {"mfma_only": round(ns[0], 2), "plus_1_valu": round(ns[1], 2), "plus_2_valu": round(ns[2], 2),
                                             "plus_3_valu": round(ns[3], 2)}
     out["mfma_only_TFLOPs"] = round(cus * 4 * 16384 / ns[0] / 1e3, 1)
+    # the shader clock inside the same kernels (20 launches back to back, about 10 ms of load): what part of "ns per
+    # MFMA" is the clock the part allows under that load
+    lib.probe_mfma_clock.argtypes, lib.probe_mfma_clock.restype = [i32, i32, i32, vp], dbl
+    clk_buf = torch.zeros(8 + 16 * cus, dtype=torch.uint8, device="cuda")
+    ghz = [lib.probe_mfma_clock(v, cus, 20, clk_buf.data_ptr()) for v in range(4)]
+    out["mfma_kernel_shader_clock_GHz"] = {"mfma_only": round(ghz[0], 3), "plus_1_valu": round(ghz[1], 3), "plus_2_valu": round(ghz[2], 3),
+                                           "plus_3_valu": round(ghz[3], 3)}
+    out["mfma_16x16x32_f16_cycles_per_wave"] = {"mfma_only": round(ns[0] * ghz[0], 1), "plus_1_valu": round(ns[1] * ghz[1], 1),
+                                                "plus_2_valu": round(ns[2] * ghz[2], 1), "plus_3_valu": round(ns[3] * ghz[3], 1)}
     return out
 
 
@@ -731,7 +837,7 @@ def extras_opt125m_fc1(torch, hip, QuantizedLinear, layers):
 
 EXTRAS = {"opt125m_fc1": extras_opt125m_fc1, "decode": extras_decode, "decode_infinity_cache_hot": extras_decode_hot,
           "decode_other_formats": extras_decode_other_formats, "hipblaslt_fp16_decode": extras_hipblaslt_decode,
-          "prefill": extras_prefill, "prefill_other_formats": extras_prefill_other_formats, "quantize": extras_quantize, "mixed_precision_model": extras_mixed_precision_model, "eager_call": extras_eager_call,
+          "prefill": extras_prefill, "prefill_clock": extras_prefill_clock, "prefill_other_formats": extras_prefill_other_formats, "quantize": extras_quantize, "mixed_precision_model": extras_mixed_precision_model, "eager_call": extras_eager_call,
           "decode_fused_siblings": extras_decode_fused_siblings, "board_probes": extras_board_probes,
           # the heavy sections last: the GEMMs and the 7B model leave the board warm, which shows in the decode timings
           "backward": extras_backward, "llama7b_decoder_graph": extras_llama7b_decoder_graph,

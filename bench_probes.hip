@@ -6,6 +6,9 @@
 //   probe_mfma_issue     v_mfma_f32_16x16x32_f16 back to back, one wave per SIMD, 32 independent accumulator tiles, with
 //                        0..3 independent VALU instructions after every MFMA: ns per MFMA and wave (how many issue
 //                        slots a single wave has per MFMA)
+//   probe_mfma_clock     the shader clock inside that kernel: core-clock ticks over real-time ticks between the first and
+//                        the last instruction of every workgroup (the part lowers its clock under load, so "ns per
+//                        MFMA" alone does not separate issue limits from clock limits)
 // Every entry point returns a negative value on a HIP error.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -38,8 +41,9 @@ __global__ __launch_bounds__(1024) void read_kernel(const u4v* __restrict__ s, i
 }
 
 template <int VPM>
-__global__ __launch_bounds__(256) void mfma_kernel(float* out, int iters, float seed) {
+__global__ __launch_bounds__(256) void mfma_kernel(float* out, int iters, float seed, unsigned long long* clk) {
     constexpr int NACC = 32;
+    const unsigned long long c0 = clock64(), r0 = wall_clock64();
     f4 acc[NACC];
 #pragma unroll
     for (int i = 0; i < NACC; i++) acc[i] = f4{0.f, 0.f, 0.f, 0.f};
@@ -63,6 +67,17 @@ __global__ __launch_bounds__(256) void mfma_kernel(float* out, int iters, float 
 #pragma unroll
     for (int i = 0; i < NACC; i++) s += acc[i][0] + acc[i][1] + acc[i][2] + acc[i][3];
     if (s == 12345.678f) out[0] = s;
+    if (clk && threadIdx.x == 0) {
+        clk[2 * blockIdx.x] = clock64() - c0;
+        clk[2 * blockIdx.x + 1] = wall_clock64() - r0;
+    }
+}
+
+void launch_mfma(int valu_per_mfma, int workgroups, float* out, int n, unsigned long long* clk) {
+    if (valu_per_mfma == 0) hipLaunchKernelGGL(mfma_kernel<0>, dim3(workgroups), dim3(256), 0, 0, out, n, 1.0f, clk);
+    else if (valu_per_mfma == 1) hipLaunchKernelGGL(mfma_kernel<1>, dim3(workgroups), dim3(256), 0, 0, out, n, 1.0f, clk);
+    else if (valu_per_mfma == 2) hipLaunchKernelGGL(mfma_kernel<2>, dim3(workgroups), dim3(256), 0, 0, out, n, 1.0f, clk);
+    else hipLaunchKernelGGL(mfma_kernel<3>, dim3(workgroups), dim3(256), 0, 0, out, n, 1.0f, clk);
 }
 
 struct Timer {
@@ -137,10 +152,7 @@ extern "C" double probe_mfma_issue(int valu_per_mfma, int workgroups, void* scra
     if (!t.ok) return -2.0;
     auto launch = [&](int n) {
         float* out = (float*)scratch;
-        if (valu_per_mfma == 0) hipLaunchKernelGGL(mfma_kernel<0>, dim3(workgroups), dim3(256), 0, 0, out, n, 1.0f);
-        else if (valu_per_mfma == 1) hipLaunchKernelGGL(mfma_kernel<1>, dim3(workgroups), dim3(256), 0, 0, out, n, 1.0f);
-        else if (valu_per_mfma == 2) hipLaunchKernelGGL(mfma_kernel<2>, dim3(workgroups), dim3(256), 0, 0, out, n, 1.0f);
-        else hipLaunchKernelGGL(mfma_kernel<3>, dim3(workgroups), dim3(256), 0, 0, out, n, 1.0f);
+        launch_mfma(valu_per_mfma, workgroups, out, n, nullptr);
     };
     launch(50);
     if (hipDeviceSynchronize() != hipSuccess || hipEventRecord(t.a, 0) != hipSuccess) return -2.0;
@@ -149,4 +161,20 @@ extern "C" double probe_mfma_issue(int valu_per_mfma, int workgroups, void* scra
     if (hipEventRecord(t.b, 0) != hipSuccess || hipDeviceSynchronize() != hipSuccess || hipEventElapsedTime(&ms, t.a, t.b) != hipSuccess)
         return -2.0;
     return (double)ms * 1e6 / ((double)iters * 32);
+}
+
+// Shader clock in GHz inside the same kernel (mean over the workgroups of the last of `launches` back-to-back
+// launches).  `scratch`: 4 + 16 * workgroups bytes of device memory, 8-byte aligned.
+extern "C" double probe_mfma_clock(int valu_per_mfma, int workgroups, int launches, void* scratch) {
+    if (valu_per_mfma < 0 || valu_per_mfma > 3 || workgroups < 1 || workgroups > 4096 || launches < 1 || !scratch) return -1.0;
+    int dev = 0, khz = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&khz, hipDeviceAttributeWallClockRate, dev) != hipSuccess || khz <= 0)
+        return -2.0;
+    unsigned long long* clk = (unsigned long long*)((char*)scratch + 8);
+    for (int i = 0; i < launches; i++) launch_mfma(valu_per_mfma, workgroups, (float*)scratch, 2000, clk);
+    static unsigned long long host[2 * 4096];
+    if (hipDeviceSynchronize() != hipSuccess || hipMemcpy(host, clk, 16 * (size_t)workgroups, hipMemcpyDeviceToHost) != hipSuccess) return -2.0;
+    double sum = 0.0;
+    for (int w = 0; w < workgroups; w++) sum += (double)host[2 * w] / (double)host[2 * w + 1];
+    return sum / workgroups * khz * 1e-6;
 }

@@ -1,6 +1,7 @@
 """Builds libbitween_hip.so (gfx950) next to its sources.
 
-    python -m bitween_amd.csrc.build
+    python -m bitween_amd.csrc.build            the library
+    python -m bitween_amd.csrc.build --tune     also libbitween_hip_tune.so, the measurement build (see build)
 
 hipcc cross-compiles without a GPU.  The library is loaded by
 bitween_amd.kernels.hip_loader; nothing is built at import time.
@@ -32,8 +33,17 @@ def _run(cmd, verbose):
         print(err, file=sys.stderr)
 
 
-def build(verbose=False):
-    """Compile every source to an object file (in parallel, one hipcc per file), then link the shared library."""
+TUNE_LIB = os.path.join(HERE, "libbitween_hip_tune.so")
+
+
+def build(verbose=False, tune=False):
+    """Compile every source to an object file (in parallel, one hipcc per file), then link the shared library.
+
+    tune=True also makes libbitween_hip_tune.so, the measurement build: the same library with the prefill kernel
+    compiled with -DBW_TUNE, which adds (1) kernel choices from the environment (BW_GEMM_NAT, BW_GEMM_BM,
+    BW_GEMM_PANEL) for same-process A/B runs and (2) bw_tune_clock_buffer(): workgroups 0..255 of a prefill launch leave
+    the core-clock and real-time ticks of their K loop there, from which the shader clock under that kernel follows
+    (bench.py --only prefill_clock).  The package never loads it."""
     from concurrent.futures import ThreadPoolExecutor
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
     objdir = os.path.join(HERE, "build")
@@ -41,11 +51,17 @@ def build(verbose=False):
     compile_flags = [f for f in FLAGS if f != "-shared"] + ["-c"]
     objs = [os.path.join(objdir, s.replace(".hip", ".o")) for s in SOURCES]
     jobs = [[hipcc] + compile_flags + ["-o", o, os.path.join(HERE, s)] for s, o in zip(SOURCES, objs)]
+    tune_obj = os.path.join(objdir, "bw_qgemm_tune.o")
+    if tune:
+        jobs.append([hipcc] + compile_flags + ["-DBW_TUNE", "-o", tune_obj, os.path.join(HERE, "bw_qgemm.hip")])
     with ThreadPoolExecutor(max_workers=min(len(jobs), os.cpu_count() or 1)) as pool:
         list(pool.map(lambda cmd: _run(cmd, verbose), jobs))
     _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs, verbose)
+    if tune:
+        others = [o for s, o in zip(SOURCES, objs) if s != "bw_qgemm.hip"]
+        _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", TUNE_LIB, tune_obj] + others, verbose)
     return LIB
 
 
 if __name__ == "__main__":
-    print(build(verbose=True))
+    print(build(verbose=True, tune="--tune" in sys.argv[1:]))

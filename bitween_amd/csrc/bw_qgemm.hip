@@ -188,6 +188,9 @@ struct GemmArgs {
     // instead of every activation tile (plain row-major ids give an XCD every 8th tile: all m-tiles and few n-tiles
     // whenever tiles_n is a multiple of 8).
     int tiles_m, panel, xcd_tiles;
+#ifdef BW_TUNE   // measurement builds only: where workgroups 0..255 leave (core-clock ticks, real-time ticks) of their K loop
+    unsigned long long* clk;
+#endif
 };
 
 BW_DEV void tile_coords(int tile, const GemmArgs& a, int& tm, int& tn) {
@@ -218,6 +221,9 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
     constexpr bool META4 = WIDE_META && C::CAN_META4, PAIR = WIDE_META && !C::CAN_META4 && C::NG == 2;
     constexpr uint32_t kOob = 0x80000000u;
     extern __shared__ __attribute__((aligned(16))) char smem[];
+#ifdef BW_TUNE
+    const unsigned long long clk_c0 = clock64(), clk_r0 = wall_clock64();
+#endif
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int nl = lane & 15, kq = lane >> 4;
     const int id = (int)blockIdx.x;
@@ -775,6 +781,12 @@ __global__ __launch_bounds__(WAVES * 64) void qgemm_kernel(const GemmArgs a) {
             step(c + 1, buf1, buf0, set1, set0, gc1, gc0, 0);
         }
     }
+#ifdef BW_TUNE
+    if (a.clk && tid == 0 && id < 256) {
+        a.clk[2 * id] = clock64() - clk_c0;
+        a.clk[2 * id + 1] = wall_clock64() - clk_r0;
+    }
+#endif
     // acc[i][j][r] = y[m0 + 16 i + nl][n0 + 16 j + 4 kq + r]
     if (partial) {
         // float32 partial tile to this workgroup's block of the workspace (tile-shaped; rows past M are never
@@ -1087,6 +1099,11 @@ int bw_qgemm_generic(const void* x, int act_dtype, int64_t M, int64_t K, int64_t
     return hipGetLastError() == hipSuccess ? BW_OK : BW_ELAUNCH;
 }
 
+#ifdef BW_TUNE
+static unsigned long long* g_tune_clk = nullptr;
+extern "C" void bw_tune_clock_buffer(void* p) { g_tune_clk = (unsigned long long*)p; }   // 4096 bytes of device memory, or null
+#endif
+
 extern "C" size_t bw_qgemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int bits, int group) {
     if (!bw_shape_ok(N, K, bits, group) || M < 1 || M >= ((int64_t)1 << 31) || !bw_fast_shape(M, N, K, K, bits, group)) return 0;
     // any of the plans may run (the call's own ldx and workspace decide): enough for each of them
@@ -1131,6 +1148,9 @@ extern "C" int bw_qgemm_ws(const void* x, int act_dtype, int64_t M, int64_t K, i
     a.tiles_n = a.full_tiles = 0;
     a.tiles_m = a.panel = 1;
     a.xcd_tiles = 0;
+#ifdef BW_TUNE
+    a.clk = g_tune_clk;
+#endif
     a.splits = 1;
     a.chunks_per_split = a.nchunks;
     hipStream_t st = (hipStream_t)stream;
