@@ -193,3 +193,32 @@ def test_prefill_padded_rows_of_x_and_y(bits, g, m, n, k, ypad):
     w16 = to_gpu(orc.dequantize_f16(qw, s16, z16, g, bits))
     ref = (x @ w16.T).float() + to_gpu(b16).float()
     assert ((y[:, :n].float() - ref).abs().max() <= 2.0 ** -8 * ref.abs().max()).item()
+
+
+@pytest.mark.parametrize("bits,g", [(4, 128), (4, 32), (8, 64), (8, 128), (2, 32), (2, 128)])
+@pytest.mark.parametrize("k", [128, 256, 384])
+def test_prefill_one_to_three_k_steps(bits, g, k):
+    """K of one, two and three steps of the prefill loop (its prologue requests two steps and the loop runs them in
+    pairs, so these are the shapes where most of what is requested lies past the end of a row), at both tile heights:
+    300 rows (128-row tiles) and 53 x 256 - 3 rows against N = 1000 (256-row tiles, the last row tile and the last
+    column tile ragged)."""
+    from bitween_amd.kernels import hip_loader
+    lib = hip_loader.load()
+    for m, n in ((300, 200), (256 * 53 - 3, 1000)):
+        _, qw, s16, z16, b16 = quantized_layer(n, k, bits, g, seed=m + n + k + bits, outliers=True)
+        gen = torch.Generator(device="cuda").manual_seed(m + k + bits)
+        x = torch.randn(m, k, device="cuda", generator=gen).half()
+        d = [to_gpu(a) for a in (qw, s16, z16, b16)]
+        need = lib.bw_qgemm_workspace_bytes(m, n, k, bits, g)
+        ws = torch.empty(max(need, 16), dtype=torch.uint8, device="cuda")
+        y = torch.full((m, n), 7.0, dtype=torch.float16, device="cuda")
+        st = lib.bw_qgemm_ws(x.data_ptr(), 0, m, k, k, d[0].data_ptr(), d[1].data_ptr(), d[2].data_ptr(), d[3].data_ptr(), n, bits, g,
+                             y.data_ptr(), n, ws.data_ptr() if need else None, need, ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+        assert st == 0
+        torch.cuda.synchronize()
+        rows = np.unique(np.concatenate([np.arange(0, m, max(1, m // 30)), np.arange(max(0, m - 6), m)]))
+        idx = torch.from_numpy(rows).cuda()
+        check_matmul(y[idx], x[idx].cpu().numpy(), qw, s16, z16, b16, bits, g)
+        w16 = to_gpu(orc.dequantize_f16(qw, s16, z16, g, bits))
+        ref = (x @ w16.T).float() + to_gpu(b16).float()
+        assert ((y.float() - ref).abs().max() <= 2.0 ** -8 * ref.abs().max()).item()
