@@ -5,18 +5,24 @@
 // 128 x 64 of it (8 x 4 MFMA 16x16 tiles, 128 accumulator registers).  Per K
 // step of one chunk (64 packed bytes per weight row):
 //   * weights go global -> registers with one 128-bit load per lane per 16
-//     rows, already in MFMA B-operand layout, and are unpacked in registers
+//     rows, already in MFMA operand layout, and are unpacked in registers
 //     to the float16 values the reference's dequantize kernel would store
 //     (bitween/modules.py:55-58).  No wave unpacks a weight another wave of
 //     the workgroup also unpacks; each weight is unpacked M/128 times overall.
-//   * activations go global -> LDS once per workgroup (double buffered,
-//     permuted into the k order the unpack emits) and every A fragment read
-//     from LDS feeds 4 MFMAs.
-// Grids that fill the device run the same kernel with 256 x 256 tiles (a wave
-// owns 256 x 64: all 256 accumulation registers): every weight
-// is unpacked once for twice the rows, the activations go memory -> LDS
-// without passing through registers, and the side work of an MFMA step is
-// dealt out one instruction per MFMA (step16 below).
+//   * activations go global -> LDS once per workgroup, double buffered, and
+//     every fragment read from LDS feeds 4 MFMAs.
+// Two schedules of that loop.  Natural order (K a multiple of 128: step16 below):
+// the activations go memory -> LDS without passing through registers (buffer
+// loads with LDS destination), the weights are unpacked to natural k order, and
+// the side work of an MFMA step is dealt out one instruction per MFMA.  Register
+// staged (any other K: step8): the activations pass through registers and are
+// permuted into the k order a cheaper unpack emits.
+// Grids that fill the device run the natural-order schedule with 256 x 256
+// tiles (a wave owns 256 x 64: all 256 accumulation registers): every weight
+// is unpacked once for twice the rows.  Which tile height a call gets is
+// gemm_tile_rows(); a short last round of tiles is cut along K (gemm_plan()),
+// and the tiles are numbered so that the workgroups an XCD runs together share
+// operand tiles in its L2 (GemmArgs::panel).
 // Also holds the shape-generic fallback used when the fast layouts do not
 // apply (odd K or group size): correct for everything the reference accepts.
 #include "bw_common.h"

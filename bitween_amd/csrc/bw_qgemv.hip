@@ -1496,11 +1496,16 @@ int launch_tiles(GemvArgs a, hipStream_t stream) {
         // and group >= 32 give exactly that today; a launch that breaks it must fall back, not hang.)
         if (8 * a.groups > nwaves * 64) return BW_EUNSUPPORTED;
         // every workgroup resident at once (a CU holds 16 waves of this kernel: up to 128 registers each), each
-        // running up to NTMAX tiles
+        // running up to NTMAX tiles - and no more tiles per workgroup than that takes: fewer, longer workgroups would
+        // read x fewer times but leave CUs without a weight stream (4096 x 4096 at 16 rows: 6.05 us with one tile per
+        // workgroup, 7.24 with two, 8.61 with three; 4096 -> 11008: 9.67 with three, 10.63 with four)
         constexpr int NTMAX = BITS == 8 ? (MT == 16 ? 2 : 3) : 4;
         const int slots = bw_device_cus() * (16 / nwaves);
         int nt = (a.ntiles + slots - 1) / slots;
         if (nt > NTMAX) nt = NTMAX;
+#ifdef BW_TUNE
+        if (const char* e = getenv("BW_GEMV_NT")) { const int v = atoi(e); if (v >= nt && v <= NTMAX) nt = v; }
+#endif
         size_t xred;
         while (true) {
             xred = (size_t)nwaves * X_BYTES;                                     // x tiles, later the partial sums
