@@ -137,6 +137,66 @@ BW_DEV void dequant_word2(uint32_t w, const GroupConst<2>& c, h2 out[8]) {
     }
 }
 
+// ---- the same in natural k order ----
+// For kernels whose other operand cannot be permuted on its way (activations that go memory -> LDS without passing
+// through registers; the transposing LDS read of the input-gradient kernel).  A 4-bit word w = bytes B0..B3, nibbles
+// n0..n7: p = [B0 B1 B0 B1] and q = [B2 B3 B2 B3] (one byte permute each) hold n0 in bits 0-3 of their low half and
+// n1 in bits 4-7 of their high half, p >> 8 likewise n2 and n3; masked into the mantissa of 1024.0 that is
+// (1024 + n0, 1024 + 16 n1), and one packed FMA with (1, 1/16) and (-(1024 + z), -(64 + z)) leaves (n0 - z, n1 - z),
+// both exact.  Times the scale: the float16 the reference's dequantize stores (bitween/modules.py:55-58).
+// 2 bits: a 16-bit half-word h = bytes b0 b1 holds fields c0..c7; p = [b0 b1 b0 b1] and p >> 8 = [b1 b0 b1 0] carry c0 / c4
+// in bits 0-1 and c2 / c6 in bits 4-5 of their low half, c1 / c5 in bits 2-3 and c3 / c7 in bits 6-7 of their high half:
+// masks 0x000C0003 and 0x00C00030 give (1024 + c0, 1024 + 4 c1) and (1024 + 16 c2, 1024 + 64 c3); packed FMAs with
+// (1, 1/4), (-(1024+z), -(256+z)) and (1/16, 1/64), (-(64+z), -(16+z)) leave the exact differences.
+// SCALE as above: false leaves the exact q - z.
+template <int BITS> struct GroupConstNat {
+    h2 s, zz, zz2;
+    BW_DEV void set(_Float16 sv, _Float16 zv) {
+        s = splat(sv);
+        if constexpr (BITS == 4) zz = h2{(_Float16)(-1024.0f) - zv, (_Float16)(-64.0f) - zv};
+        else if constexpr (BITS == 2) {
+            zz = h2{(_Float16)(-1024.0f) - zv, (_Float16)(-256.0f) - zv};
+            zz2 = h2{(_Float16)(-64.0f) - zv, (_Float16)(-16.0f) - zv};
+        } else zz = splat((_Float16)(-1024.0f) - zv);
+    }
+};
+
+// half-word `half` (0 or 1) of a 2-bit word -> 4 pairs in natural order
+template <bool SCALE = true>
+BW_DEV void dequant_halfword2_nat(uint32_t w, int half, const GroupConstNat<2>& c, h2 out[4]) {
+    const h2 ka = h2{(_Float16)1.0f, (_Float16)0.25f}, kb = h2{(_Float16)0.0625f, (_Float16)0.015625f};
+    const uint32_t p = half ? __builtin_amdgcn_perm(w, w, 0x03020302u) : __builtin_amdgcn_perm(w, w, 0x01000100u), q = p >> 8;
+    out[0] = __builtin_elementwise_fma(as_h2(and_or(p, 0x000C0003u, kMagic)), ka, c.zz);
+    out[1] = __builtin_elementwise_fma(as_h2(and_or(p, 0x00C00030u, kMagic)), kb, c.zz2);
+    out[2] = __builtin_elementwise_fma(as_h2(and_or(q, 0x000C0003u, kMagic)), ka, c.zz);
+    out[3] = __builtin_elementwise_fma(as_h2(and_or(q, 0x00C00030u, kMagic)), kb, c.zz2);
+    if constexpr (SCALE) {
+#pragma unroll
+        for (int e = 0; e < 4; e++) out[e] = out[e] * c.s;
+    }
+}
+
+// one 4-bit word -> 4 pairs in natural order
+template <bool SCALE = true>
+BW_DEV void dequant_word4_nat(uint32_t w, const GroupConstNat<4>& c, h2 out[4]) {
+    const h2 kk = h2{(_Float16)1.0f, (_Float16)0.0625f};
+    const uint32_t p = __builtin_amdgcn_perm(w, w, 0x01000100u), q = __builtin_amdgcn_perm(w, w, 0x03020302u);
+    const uint32_t src[4] = {p, p >> 8, q, q >> 8};
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+        out[e] = __builtin_elementwise_fma(as_h2(and_or(src[e], 0x00F0000Fu, kMagic)), kk, c.zz);
+        if constexpr (SCALE) out[e] = out[e] * c.s;
+    }
+}
+
+// one 8-bit word -> 2 pairs (natural order as it is)
+template <bool SCALE = true>
+BW_DEV void dequant_word8_nat(uint32_t w, const GroupConstNat<8>& c, h2 out[2]) {
+    out[0] = as_h2(__builtin_amdgcn_perm(0x64646464u, w, 0x04010400u)) + c.zz;
+    out[1] = as_h2(__builtin_amdgcn_perm(0x64646464u, w, 0x04030402u)) + c.zz;
+    if constexpr (SCALE) { out[0] = out[0] * c.s; out[1] = out[1] * c.s; }
+}
+
 // Position p of a block of VPI consecutive k holds original element perm(p):
 // the order in which the routines above emit the values of one word.
 template <int BITS> BW_DEV constexpr int slot_to_k(int p);

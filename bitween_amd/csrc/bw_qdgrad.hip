@@ -10,12 +10,15 @@
 // The reduction runs over N, the dimension the packed words do NOT run along, so a weight tile has to be
 // transposed on its way to the matrix core.  A workgroup owns a 128 or 256 (m) x 128 (k) tile of grad_x and walks
 // N in steps of 32 rows:
-//   * 256 threads each take 16 consecutive k of one row n (one group: groups are >= 32 wide) and dequantise them to
-//     the reference's W16 (magic-number unpack, exact q - z, one multiply by the scale); the lanes of rows n and
-//     n + 1 swap half of their values and write dwords (n, n + 1) into an LDS tile stored k-major (row k holds the
-//     32 n of the step) - that is the transposition;
+//   * 256 threads each take 16 consecutive k of one row n (one group: groups are >= 32 wide), dequantise them to
+//     the reference's W16 in natural k order (magic-number unpack, exact q - z, one multiply by the scale) and write
+//     them as they are - 32 bytes - into an LDS tile stored n-major (row n holds the 128 k of the tile; the 32-byte
+//     pieces of a row XOR-swizzled by the row number);
+//   * the matrix core wants, per lane, 8 consecutive n of one k: ds_read_b64_tr_b16 is that transposition - the 16
+//     lanes of a quarter wave point at 4 rows x 4 pieces of 4 halves and each receives one column of the 4 x 16 block
+//     (element e of lane i = element i % 4 of the piece lane 4 e + i / 4 points at), two reads per operand;
 //   * the 128 / 256 x 32 slice of grad_y goes to a second LDS tile as it is;
-//   * v_mfma_f32_16x16x32_f16 with A = rows of the k-major tile (8 consecutive n per lane) and B = rows of the
+//   * v_mfma_f32_16x16x32_f16 with A = those columns (8 consecutive n per lane) and B = rows of the
 //     grad_y tile: D[k][m], so a lane ends up with 4 consecutive k of one m.
 // LDS is double buffered and filled one step ahead, in the shadow of the current step's MFMAs; global loads run
 // two steps ahead; one barrier per step.  Three (two with the 256-row tile) workgroups share a CU and cover each
@@ -28,8 +31,8 @@
 namespace {
 
 constexpr int DK = 128, DN = 32, DTHREADS = 256;
-constexpr int DPITCH = 80;                           // bytes per LDS row: 32 halves + 16 (rows stay 16-byte aligned)
-constexpr int B_BYTES = DK * DPITCH + (DK / 16) * 16;   // k-major weight tile; every 16-row block shifted 16 bytes
+constexpr int DPITCH = 80;                           // bytes per LDS row of the grad_y tile: 32 halves + 16 (rows stay 16-byte aligned)
+constexpr int B_BYTES = DN * DK * 2;                 // n-major weight tile: 32 rows of 128 halves, unpadded
 // MT = 16-row m tiles per wave (the workgroup's 2 x 2 waves cover 32 MT rows of m).  MT = 4 (161 registers, three
 // workgroups per CU) up to 512 rows of grad_y; MT = 8 (251 registers, two per CU, a quarter fewer LDS reads per MFMA)
 // beyond: 15-20 % faster there, slower below.
@@ -50,29 +53,30 @@ struct DgradArgs {
     int tiles_k, splits, steps_per_split;
 };
 
-BW_DEV uint32_t dpp_xor8(uint32_t v) {               // value of lane ^ 8 (rotate a 16-lane row by 8)
-    return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x128, 0xF, 0xF, true);
-}
+// 32-byte piece p of row n of the weight tile sits at piece p ^ w_swizzle(n): the rows a transposing read touches
+// (n = 8 q + 4 h + 0..3 for the four quarter waves q) then fall into different banks, 8 distinct pieces per half wave
+BW_DEV int w_swizzle(int n) { return (n & 3) | (((n >> 3) & 1) << 2); }
 
-BW_DEV int b_row_offset(int k) { return k * DPITCH + (k >> 4) * 16; }
+typedef short s4 __attribute__((ext_vector_type(4)));
 
 template <int BITS> struct WLoad;
 template <> struct WLoad<4> { typedef u2 type; };
 template <> struct WLoad<8> { typedef u4 type; };
 template <> struct WLoad<2> { typedef uint32_t type; };
 
-// 16 values of one row -> 8 float16 pairs; pair p, half h is element kmap(p, h) of the 16.  SCALE = false: the
-// exact integers q - z (the caller multiplies by the scale in float32).
+// 16 values of one row -> 8 float16 pairs in natural k order.  SCALE = false: the exact integers q - z (the caller
+// multiplies by the scale in float32).
 template <int BITS, bool SCALE>
-BW_DEV void dequant16(const typename WLoad<BITS>::type& w, const GroupConst<BITS>& gc, h2* out) {
+BW_DEV void dequant16(const typename WLoad<BITS>::type& w, const GroupConstNat<BITS>& gc, h2* out) {
     if constexpr (BITS == 4) {
-        dequant_word4<SCALE>(w[0], gc, out);
-        dequant_word4<SCALE>(w[1], gc, out + 4);
+        dequant_word4_nat<SCALE>(w[0], gc, out);
+        dequant_word4_nat<SCALE>(w[1], gc, out + 4);
     } else if constexpr (BITS == 8) {
 #pragma unroll
-        for (int j = 0; j < 4; j++) dequant_word8<SCALE>(w[j], gc, out + 2 * j);
+        for (int j = 0; j < 4; j++) dequant_word8_nat<SCALE>(w[j], gc, out + 2 * j);
     } else {
-        dequant_word2<SCALE>(w, gc, out);
+        dequant_halfword2_nat<SCALE>(w, 0, gc, out);
+        dequant_halfword2_nat<SCALE>(w, 1, gc, out + 4);
     }
 }
 
@@ -92,13 +96,6 @@ BW_DEV f4 mfma16(const h8& a, const h8& b, const f4& c) {
     if constexpr (DT == BW_F16) return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
     else return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf8, a), __builtin_bit_cast(bf8, b), c, 0, 0, 0);
 }
-template <int BITS>
-BW_DEV constexpr int kmap(int p, int h) {
-    if constexpr (BITS == 4) return 8 * (p >> 2) + (p & 3) + 4 * h;
-    else if constexpr (BITS == 8) return 2 * p + h;
-    else return p + 8 * h;
-}
-
 template <int BITS, int GROUP, int MT, int DT>
 __global__ __launch_bounds__(DTHREADS, MT == 4 ? 3 : 2) void qdgrad_kernel(const DgradArgs a) {   // workgroups per CU: 3 (<= 168 registers) or 2
     constexpr int DM = DgradTile<MT>::DM, A_BYTES = DgradTile<MT>::A_BYTES, STAGE = DgradTile<MT>::STAGE;
@@ -125,12 +122,8 @@ __global__ __launch_bounds__(DTHREADS, MT == 4 ? 3 : 2) void qdgrad_kernel(const
     const _Float16* gp[GR];
 #pragma unroll
     for (int r = 0; r < GR; r++) gp[r] = a.go + (int64_t)min(m0 + gm + 128 * r, a.M - 1) * a.ldg + gpart * 16;
-    // Two lanes 8 apart hold the same 16 k of rows n and n + 1.  They swap half of their values so that each
-    // writes whole dwords (n, n + 1) of the k-major tile: the even row's lane takes the first 8 of the 16
-    // values (pairs 0-3), the odd row's lane the rest.
-    const bool odd = wn & 1;
-    const uint32_t sel_lo = odd ? 0x01000504u : 0x05040100u, sel_hi = odd ? 0x03020706u : 0x07060302u;
-    const int b_dst = wks * (16 * DPITCH + 16) + (odd ? kmap<BITS>(4, 0) * DPITCH : 0) + (wn & ~1) * 2;
+    // a thread's 16 values are one 32-byte piece of row wn of the weight tile
+    const int b_dst = wn * (DK * 2) + ((wks ^ w_swizzle(wn)) * 32);
 
     // PD steps of loads are in flight (a step's MFMAs take a fraction of a memory round trip).  Requests are
     // unconditional - past the slice's end they repeat its last step - so the wait counts stay exact.
@@ -157,12 +150,15 @@ __global__ __launch_bounds__(DTHREADS, MT == 4 ? 3 : 2) void qdgrad_kernel(const
 
     const int wk = (wave & 1) * 64, wm = (wave >> 1) * (16 * MT);     // this wave's quarter of the tile
     const int l16 = lane & 15, q = lane >> 4;
+    // rows of the weight tile this lane points the transposing reads at (h = 0, 1) and their swizzle (the same for both)
+    const int tr_row[2] = {(8 * q + (l16 >> 2)) * (DK * 2), (8 * q + 4 + (l16 >> 2)) * (DK * 2)};
+    const int tr_swz = w_swizzle(8 * q + (l16 >> 2));
 
     // slot -> LDS stage: dequantise the 16 weights and scatter them transposed; copy the grad_y rows
     auto fill = [&](int slot, int stage, bool live) {
         char* As = smem + stage * STAGE;
         char* Bs = As + A_BYTES;
-        GroupConst<BITS> gc;
+        GroupConstNat<BITS> gc;
         gc.set(live ? sreg[slot] : (_Float16)0.f, zreg[slot]);        // past the slice's end: weights of zero
         h2 w16[8];
         uint32_t wd[8];                                               // the 8 pairs in the gradient's type
@@ -176,13 +172,8 @@ __global__ __launch_bounds__(DTHREADS, MT == 4 ? 3 : 2) void qdgrad_kernel(const
 #pragma unroll
             for (int i = 0; i < 8; i++) wd[i] = pack2<DT>(__fmul_rn((float)w16[i][0], sf), __fmul_rn((float)w16[i][1], sf));
         }
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const uint32_t lo4 = wd[i], hi4 = wd[4 + i];
-            const uint32_t keep = odd ? hi4 : lo4, recv = dpp_xor8(odd ? lo4 : hi4);
-            *reinterpret_cast<uint32_t*>(Bs + b_dst + kmap<BITS>(i, 0) * DPITCH) = __builtin_amdgcn_perm(recv, keep, sel_lo);
-            *reinterpret_cast<uint32_t*>(Bs + b_dst + kmap<BITS>(i, 1) * DPITCH) = __builtin_amdgcn_perm(recv, keep, sel_hi);
-        }
+        *reinterpret_cast<u4*>(Bs + b_dst) = u4{wd[0], wd[1], wd[2], wd[3]};
+        *reinterpret_cast<u4*>(Bs + b_dst + 16) = u4{wd[4], wd[5], wd[6], wd[7]};
 #pragma unroll
         for (int r = 0; r < GR; r++) {
             u4* dst = reinterpret_cast<u4*>(As + (gm + 128 * r) * DPITCH + gpart * 32);
@@ -211,7 +202,16 @@ __global__ __launch_bounds__(DTHREADS, MT == 4 ? 3 : 2) void qdgrad_kernel(const
             const char* Bs = As + A_BYTES;
             h8 af[4], bf[MT];
 #pragma unroll
-            for (int i = 0; i < 4; i++) af[i] = *reinterpret_cast<const h8*>(Bs + b_row_offset(wk + 16 * i + l16) + q * 16);
+            for (int i = 0; i < 4; i++) {
+                // operand of k-tile i: n = 8 q .. 8 q + 7 of column k = wk + 16 i + l16 - two transposing reads of 4 n each
+                const int piece = (wk >> 4) + i;
+                s4 v[2];
+#pragma unroll
+                for (int h = 0; h < 2; h++)
+                    v[h] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                        (__attribute__((address_space(3))) s4*)(Bs + tr_row[h] + ((piece ^ tr_swz) * 32) + (l16 & 3) * 8));
+                af[i] = __builtin_bit_cast(h8, __builtin_shufflevector(v[0], v[1], 0, 1, 2, 3, 4, 5, 6, 7));
+            }
 #pragma unroll
             for (int j = 0; j < MT; j++) bf[j] = *reinterpret_cast<const h8*>(As + (wm + 16 * j + l16) * DPITCH + q * 16);
             fill((d + 1) % PD, (d + 1) & 1, step + 1 < s_end);

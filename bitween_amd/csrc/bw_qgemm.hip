@@ -95,47 +95,6 @@ BW_DEV void permute_unit(const uint32_t* r, uint32_t* o) {
     }
 }
 
-// Group constants and unpack for fragments in natural k order (256-row tiles, whose activations go from memory to LDS
-// without passing through registers and so cannot be permuted on the way).  A 4-bit word w = bytes B0..B3, nibbles
-// n0..n7: p = [B0 B1 B0 B1] and q = [B2 B3 B2 B3] (one byte permute each) hold n0 in bits 0-3 of their low half and
-// n1 in bits 4-7 of their high half, p >> 8 likewise n2 and n3; masked into the mantissa of 1024.0 that is
-// (1024 + n0, 1024 + 16 n1), and one packed FMA with (1, 1/16) and (-(1024 + z), -(64 + z)) leaves (n0 - z, n1 - z),
-// both exact.  Times the scale: the float16 the reference's dequantize stores (bitween/modules.py:55-58).
-// 2 bits: a 16-bit half-word h = bytes b0 b1 holds fields c0..c7; p = [b0 b1 b0 b1] and p >> 8 = [b1 b0 b1 0] carry c0 / c4
-// in bits 0-1 and c2 / c6 in bits 4-5 of their low half, c1 / c5 in bits 2-3 and c3 / c7 in bits 6-7 of their high half:
-// masks 0x000C0003 and 0x00C00030 give (1024 + c0, 1024 + 4 c1) and (1024 + 16 c2, 1024 + 64 c3); packed FMAs with
-// (1, 1/4), (-(1024+z), -(256+z)) and (1/16, 1/64), (-(64+z), -(16+z)) leave the exact differences.
-template <int BITS> struct GroupConstNat {
-    h2 s, zz, zz2;
-    BW_DEV void set(_Float16 sv, _Float16 zv) {
-        s = splat(sv);
-        if constexpr (BITS == 4) zz = h2{(_Float16)(-1024.0f) - zv, (_Float16)(-64.0f) - zv};
-        else if constexpr (BITS == 2) {
-            zz = h2{(_Float16)(-1024.0f) - zv, (_Float16)(-256.0f) - zv};
-            zz2 = h2{(_Float16)(-64.0f) - zv, (_Float16)(-16.0f) - zv};
-        } else zz = splat((_Float16)(-1024.0f) - zv);
-    }
-};
-
-// half-word `half` (0 or 1) of a 2-bit word -> 4 pairs in natural order
-BW_DEV void dequant_halfword2_nat(uint32_t w, int half, const GroupConstNat<2>& c, h2 out[4]) {
-    const h2 ka = h2{(_Float16)1.0f, (_Float16)0.25f}, kb = h2{(_Float16)0.0625f, (_Float16)0.015625f};
-    const uint32_t p = half ? __builtin_amdgcn_perm(w, w, 0x03020302u) : __builtin_amdgcn_perm(w, w, 0x01000100u), q = p >> 8;
-    out[0] = __builtin_elementwise_fma(as_h2(and_or(p, 0x000C0003u, kMagic)), ka, c.zz) * c.s;
-    out[1] = __builtin_elementwise_fma(as_h2(and_or(p, 0x00C00030u, kMagic)), kb, c.zz2) * c.s;
-    out[2] = __builtin_elementwise_fma(as_h2(and_or(q, 0x000C0003u, kMagic)), ka, c.zz) * c.s;
-    out[3] = __builtin_elementwise_fma(as_h2(and_or(q, 0x00C00030u, kMagic)), kb, c.zz2) * c.s;
-}
-
-BW_DEV void dequant_word4_nat(uint32_t w, const GroupConstNat<4>& c, h2 out[4]) {
-    const h2 kk = h2{(_Float16)1.0f, (_Float16)0.0625f};
-    const uint32_t p = __builtin_amdgcn_perm(w, w, 0x01000100u), q = __builtin_amdgcn_perm(w, w, 0x03020302u);
-    const uint32_t src[4] = {p, p >> 8, q, q >> 8};
-#pragma unroll
-    for (int e = 0; e < 4; e++)
-        out[e] = __builtin_elementwise_fma(as_h2(and_or(src[e], 0x00F0000Fu, kMagic)), kk, c.zz) * c.s;
-}
-
 // Unpack word t of a lane load (8 values for MFMA step t at 4 bits; two steps' worth at 2 bits, half a
 // step at 8 bits is handled by the caller) - thin wrappers so the K loop can unpack just in time.
 template <int BITS>
