@@ -11,7 +11,8 @@ import subprocess
 import sys
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-SOURCES = ["bw_quantize.hip", "bw_qgemv.hip", "bw_qgemm.hip", "bw_qdgrad.hip"]
+SOURCES = ["bw_quantize.hip", "bw_qgemv.hip", "bw_qgemm.hip", "bw_qgemm_rows.hip", "bw_qdgrad.hip"]
+TUNE_SOURCES = ["bw_qgemm.hip", "bw_qgemm_rows.hip"]      # compiled a second time with -DBW_TUNE for the measurement build
 LIB = os.path.join(HERE, "libbitween_hip.so")
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
@@ -51,15 +52,15 @@ def build(verbose=False, tune=False):
     compile_flags = [f for f in FLAGS if f != "-shared"] + ["-c"]
     objs = [os.path.join(objdir, s.replace(".hip", ".o")) for s in SOURCES]
     jobs = [[hipcc] + compile_flags + ["-o", o, os.path.join(HERE, s)] for s, o in zip(SOURCES, objs)]
-    tune_obj = os.path.join(objdir, "bw_qgemm_tune.o")
+    tune_objs = [os.path.join(objdir, s.replace(".hip", "_tune.o")) for s in TUNE_SOURCES]
     if tune:
-        jobs.append([hipcc] + compile_flags + ["-DBW_TUNE", "-o", tune_obj, os.path.join(HERE, "bw_qgemm.hip")])
+        jobs += [[hipcc] + compile_flags + ["-DBW_TUNE", "-o", o, os.path.join(HERE, s)] for s, o in zip(TUNE_SOURCES, tune_objs)]
     with ThreadPoolExecutor(max_workers=min(len(jobs), os.cpu_count() or 1)) as pool:
         list(pool.map(lambda cmd: _run(cmd, verbose), jobs))
     _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs, verbose)
     if tune:
-        others = [o for s, o in zip(SOURCES, objs) if s != "bw_qgemm.hip"]
-        _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", TUNE_LIB, tune_obj] + others, verbose)
+        others = [o for s, o in zip(SOURCES, objs) if s not in TUNE_SOURCES]
+        _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", TUNE_LIB] + tune_objs + others, verbose)
     return LIB
 
 

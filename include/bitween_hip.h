@@ -112,7 +112,7 @@ int bw_dequantize(const int32_t* qweight, const void* scale, int scale_dtype, co
  * bw_qgemv: decode path, 1 <= M <= 16, HBM-bound, no workspace.
  * bw_qgemm: prefill path, any M >= 1, MFMA-bound.
  * bw_qlinear: picks between them by M (what the Python forward calls): the decode kernel, 16 rows per
- *             launch, up to M = bw_qlinear_decode_rows(N, K, bits) (48; 32 for layers of 20 MiB of packed
+ *             launch, up to M = bw_qlinear_decode_rows(N, K, bits) (48; 32 for layers of 10 MiB of packed
  *             weights and more; 16 from 40 MiB on); the prefill kernel (without a workspace) beyond. */
 int bw_qgemv(const void* x, int act_dtype, int64_t M, int64_t K, int64_t ldx,
              const int32_t* qweight, const void* scale16, const void* zp16, const void* bias,

@@ -70,6 +70,10 @@ def test_split_k_workspace_size_is_a_pure_host_function():
     # 256-row tiles need whole K steps of 128 values and a grid that fills the device
     assert rows(4096, 4096, 4096, 2, 128) == 256 and rows(4096, 4096, 4096 + 64, 4, 64) == 128 and rows(512, 14336, 4096, 4, 128) == 128
     assert rows(128, 20, 96, 4, 48) == 0                        # the shape-generic kernel
+    # calls of at most 64 rows take 64-row tiles (natural-order schedule: K a multiple of 128); their split-K blocks fit
+    # the workspace of the 128-row plan
+    assert rows(64, 4096, 4096, 4, 128) == 64 and rows(17, 11008, 4096, 8, 64) == 64 and rows(65, 4096, 4096, 4, 128) == 128
+    assert rows(32, 4096, 4096 + 64, 4, 64) == 128
     assert ws(512, 14336, 4096, 4, 128) == 0                    # 224 tiles: 0.875 of a round
     # few tiles and a long K: every tile split so that one round is filled
     for m, n, k, bits in ((128, 4096, 14336, 4), (512, 4096, 14336, 4), (128, 14336, 4096, 4), (64, 1024, 2048, 8)):
@@ -85,11 +89,11 @@ def test_split_k_workspace_size_is_a_pure_host_function():
 
 
 def test_decode_rows_switch_is_a_pure_host_function():
-    """bw_qlinear keeps up to 48 rows on the decode kernel for small layers, 32 for 20 MiB of packed weights and more
-    (three 16-row launches over a large layer lose to one prefill launch) and 16 from 40 MiB on."""
+    """bw_qlinear keeps up to 48 rows on the decode kernel for layers under 10 MiB of packed weights, 32 under 40 MiB
+    (a third 16-row launch loses to one launch of the prefill kernel's 64-row tiles) and 16 from 40 MiB on."""
     from bitween_amd.kernels import hip_loader
     rows = hip_loader.load().bw_qlinear_decode_rows
-    assert rows(4096, 4096, 4) == 48 and rows(4096, 4096, 8) == 48 and rows(4096, 11008, 2) == 48
+    assert rows(4096, 4096, 4) == 48 and rows(4096, 4096, 8) == 32 and rows(4096, 11008, 2) == 32
     assert rows(11008, 4096, 4) == 32 and rows(14336, 4096, 4) == 32 and rows(4096, 11008, 8) == 16 and rows(12288, 4096, 8) == 16
     assert rows(0, 4096, 4) == 0 and rows(4096, 4096, 3) == 0
 

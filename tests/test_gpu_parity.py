@@ -284,7 +284,10 @@ def test_gemm_split_k_vs_unsplit_and_oracle(bits, g, m, k, n):
     y_small = torch.full((m, n), 7.0, dtype=torch.float16, device="cuda")
     assert run(ws.data_ptr(), need, y_split) == 0
     assert run(None, 0, y_plain) == 0
-    assert run(ws.data_ptr(), need - 4, y_small) == -5          # BW_EWORKSPACE, nothing launched
+    # bw_qgemm_workspace_bytes covers every plan a call of this shape may get (the 128-row plan also where the call
+    # itself runs 64-row tiles, whose blocks are half as large): there only less than two 64-row blocks is surely short
+    short = need - 4 if lib.bw_qgemm_tile_rows(m, n, k, bits, g) != 64 else 2 * 64 * 256 * 4 - 16
+    assert run(ws.data_ptr(), short, y_small) == -5             # BW_EWORKSPACE, nothing launched
     assert run(ws.data_ptr() + 4, need, y_small) == -3          # BW_EALIGN
     torch.cuda.synchronize()
     assert (y_small == 7.0).all()
@@ -777,7 +780,7 @@ def test_forward_under_graph_capture_replays_like_eager(m, dtype):
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("bits,switch,ms", [(4, 32, (32, 33, 40, 48)), (8, 16, (16, 17, 32, 33))])
 def test_rows_33_to_48_on_a_large_layer_take_the_prefill_kernel(dtype, bits, switch, ms):
-    """For a layer of 20 MiB of packed weights and more bw_qlinear hands 33-48 rows to the prefill kernel, from 40 MiB on
+    """For a layer of 10 MiB of packed weights and more bw_qlinear hands 33-48 rows to the prefill kernel, from 40 MiB on
     (4096 -> 11008 at 8 bits) 17-32 rows too; the module forward (validated-buffer path, bfloat16 cast included) must
     follow it and agree with the C entry point."""
     import ctypes
@@ -945,6 +948,39 @@ def test_prefill_256_row_tiles_vs_oracle(bits, g, k):
     ref = x @ to_gpu(w16).T
     assert torch.isfinite(y_plain).all()
     assert ((y_plain.float() - ref.float()).abs().max() <= 2.0 ** -8 * ref.float().abs().max()).item()
+
+
+@pytest.mark.parametrize("bits,g", [(4, 128), (4, 64), (4, 32), (8, 128), (8, 64), (8, 32), (2, 128), (2, 64), (2, 32)])
+def test_prefill_64_row_tiles_vs_oracle(bits, g):
+    """Calls of at most 64 rows run the prefill kernel with 64-row tiles (same arithmetic as bitween/modules.py:85-97):
+    17, 33 and 64 rows, ragged N, K of one / six / seven / 32 steps, split along K through the workspace and un-split,
+    with and without bias - every row against the oracle, one-hot rows bit for bit."""
+    import ctypes
+    hip = _hip()
+    lib = hip.load()
+    n = 1000
+    for k in (128, 768, 896, 4096):
+        _, qw, s16, z16, b16 = quantized_layer(n, k, bits, g, seed=bits * 10 + g + k, outliers=True)
+        w16 = orc.dequantize_f16(qw, s16, z16, g, bits)
+        d = [to_gpu(a) for a in (qw, s16, z16, b16)]
+        for m in (17, 33, 64):
+            assert lib.bw_qgemm_tile_rows(m, n, k, bits, g) == 64
+            gen = torch.Generator(device="cuda").manual_seed(k + bits + m)
+            x = torch.randn(m, k, device="cuda", generator=gen).half()
+            hot = {0: k - 1, m - 1: k // 2}
+            for r, c in hot.items():
+                x[r] = 0
+                x[r, c] = 1.0
+            y_ws = hip.quantized_gemm_hip(x, d[0], d[1], d[2], d[3], bits, g)          # with the split-K workspace
+            y_plain = torch.full((m, n), float("nan"), dtype=torch.float16, device="cuda")
+            assert lib.bw_qgemm(x.data_ptr(), 0, m, k, k, d[0].data_ptr(), d[1].data_ptr(), d[2].data_ptr(), None, n, bits, g,
+                                y_plain.data_ptr(), n, ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)) == 0
+            torch.cuda.synchronize()
+            x_np = x.cpu().numpy()
+            check_matmul(y_ws, x_np, qw, s16, z16, b16, bits, g)
+            check_matmul(y_plain, x_np, qw, s16, z16, None, bits, g)
+            for r, c in hot.items():
+                assert np.array_equal(y_plain[r].cpu().numpy().view(np.uint16), w16[:, c].view(np.uint16))
 
 
 def test_prefill_256_row_tiles_split_the_short_last_round():
