@@ -59,7 +59,11 @@ inline int gemm_tile_rows(int64_t M, int64_t N, int64_t K, int64_t ldx, int bits
 #ifdef BW_TUNE
     if (const char* e = getenv("BW_GEMM_BM")) return atoi(e) == 256 ? 256 : atoi(e) == 64 ? 64 : 128;
 #endif
+    // (up to 128 rows as two 64-row tiles where N is at most 16 tiles wide: 4096 x 4096, 11008 -> 4096 and 14336 -> 4096 at
+    // 80 ... 128 rows 0.88-0.95 of the 128-row time - half the partial-tile traffic of the K split -, but 1.06-1.11 at
+    // N = 11008 and 14336, where every weight would be unpacked twice for nothing)
     if (M <= 64) return 64;
+    if (M <= 128 && (N + BN - 1) / BN <= 16 && !(have_workspace && gemm_plan(M, N, nchunks, true, 64).ws_bytes > workspace_bytes)) return 64;
     const int64_t cus = bw_device_cus();
     auto rounds = [&](int64_t tiles) {
         const int64_t full = tiles / cus, rest = tiles % cus;
@@ -166,9 +170,10 @@ extern "C" size_t bw_qgemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int 
     if (gemm_nat(M, K, K)) {
         const size_t nat128 = gemm_plan(M, N, gemm_chunks(K, bits, true), true, 128).ws_bytes;
         if (nat128 > need) need = nat128;
-        if (gemm_tile_rows(M, N, K, K, bits, true, ~(size_t)0) == 256) {
-            const size_t big = gemm_plan(M, N, gemm_chunks(K, bits, true), true, 256).ws_bytes;
-            if (big > need) need = big;
+        const int rows = gemm_tile_rows(M, N, K, K, bits, true, ~(size_t)0);
+        if (rows != 128) {
+            const size_t other = gemm_plan(M, N, gemm_chunks(K, bits, true), true, rows).ws_bytes;
+            if (other > need) need = other;
         }
     }
     return need;

@@ -72,8 +72,11 @@ def test_split_k_workspace_size_is_a_pure_host_function():
     assert rows(128, 20, 96, 4, 48) == 0                        # the shape-generic kernel
     # calls of at most 64 rows take 64-row tiles (natural-order schedule: K a multiple of 128); their split-K blocks fit
     # the workspace of the 128-row plan
-    assert rows(64, 4096, 4096, 4, 128) == 64 and rows(17, 11008, 4096, 8, 64) == 64 and rows(65, 4096, 4096, 4, 128) == 128
+    assert rows(64, 4096, 4096, 4, 128) == 64 and rows(17, 11008, 4096, 8, 64) == 64 and rows(65, 11008, 4096, 4, 128) == 128
     assert rows(32, 4096, 4096 + 64, 4, 64) == 128
+    # up to 128 rows as two 64-row tiles where N is at most 16 tiles wide (half the partial-tile traffic of the K split)
+    assert rows(128, 4096, 14336, 4, 128) == 64 and rows(96, 4096, 4096, 8, 128) == 64 and rows(129, 4096, 4096, 4, 128) == 128
+    assert rows(128, 4096 + 256, 4096, 4, 128) == 128
     assert ws(512, 14336, 4096, 4, 128) == 0                    # 224 tiles: 0.875 of a round
     # few tiles and a long K: every tile split so that one round is filled
     for m, n, k, bits in ((128, 4096, 14336, 4), (512, 4096, 14336, 4), (128, 14336, 4096, 4), (64, 1024, 2048, 8)):

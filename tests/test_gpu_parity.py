@@ -952,8 +952,8 @@ def test_prefill_256_row_tiles_vs_oracle(bits, g, k):
 
 @pytest.mark.parametrize("bits,g", [(4, 128), (4, 64), (4, 32), (8, 128), (8, 64), (8, 32), (2, 128), (2, 64), (2, 32)])
 def test_prefill_64_row_tiles_vs_oracle(bits, g):
-    """Calls of at most 64 rows run the prefill kernel with 64-row tiles (same arithmetic as bitween/modules.py:85-97):
-    17, 33 and 64 rows, ragged N, K of one / six / seven / 32 steps, split along K through the workspace and un-split,
+    """Calls of at most 64 rows - and up to 128 rows where N is at most 16 tiles wide - run the prefill kernel with 64-row
+    tiles (same arithmetic as bitween/modules.py:85-97): 17, 33, 64, 100 and 128 rows (one and two row tiles), ragged N, K of one / six / seven / 32 steps, split along K through the workspace and un-split,
     with and without bias - every row against the oracle, one-hot rows bit for bit."""
     import ctypes
     hip = _hip()
@@ -963,7 +963,7 @@ def test_prefill_64_row_tiles_vs_oracle(bits, g):
         _, qw, s16, z16, b16 = quantized_layer(n, k, bits, g, seed=bits * 10 + g + k, outliers=True)
         w16 = orc.dequantize_f16(qw, s16, z16, g, bits)
         d = [to_gpu(a) for a in (qw, s16, z16, b16)]
-        for m in (17, 33, 64):
+        for m in (17, 33, 64, 100, 128):
             assert lib.bw_qgemm_tile_rows(m, n, k, bits, g) == 64
             gen = torch.Generator(device="cuda").manual_seed(k + bits + m)
             x = torch.randn(m, k, device="cuda", generator=gen).half()
