@@ -51,6 +51,7 @@ struct DgradArgs {
     float* ws;
     int M, N, K, ldg, ldx, groups, row_bytes;
     int tiles_k, splits, steps_per_split;
+    uint32_t go_bytes, w_bytes, meta_bytes;          // extents for the buffer descriptors of the 256 x 256 kernel
 };
 
 // 32-byte piece p of row n of the weight tile sits at piece p ^ w_swizzle(n): the rows a transposing read touches
@@ -249,25 +250,311 @@ __global__ __launch_bounds__(DTHREADS, MT == 4 ? 3 : 2) void qdgrad_kernel(const
 }
 
 // grad_x tile = sum of its slices' partial tiles, rounded once
-template <int DM, int DT>
+template <int DM, int DT, int DKT = DK>
 __global__ __launch_bounds__(256) void qdgrad_reduce_kernel(const DgradArgs a) {
     const int tile = blockIdx.y;
-    const int quad = (int)(blockIdx.x * blockDim.x + threadIdx.x);    // < DM * DK / 4
-    const int ml = quad / (DK / 4), kl = (quad % (DK / 4)) * 4;
-    const int m = (tile / a.tiles_k) * DM + ml, k = (tile % a.tiles_k) * DK + kl;
+    const int quad = (int)(blockIdx.x * blockDim.x + threadIdx.x);    // < DM * DKT / 4
+    const int ml = quad / (DKT / 4), kl = (quad % (DKT / 4)) * 4;
+    const int m = (tile / a.tiles_k) * DM + ml, k = (tile % a.tiles_k) * DKT + kl;
     if (m >= a.M) return;
-    const float* src = a.ws + (size_t)tile * a.splits * (DM * DK) + ml * DK + kl;
+    const float* src = a.ws + (size_t)tile * a.splits * (DM * DKT) + ml * DKT + kl;
     f4 v = {0.f, 0.f, 0.f, 0.f};
     for (int z = 0; z < a.splits; z++) {
-        const f4 t = *reinterpret_cast<const f4*>(src + (size_t)z * (DM * DK));
+        const f4 t = *reinterpret_cast<const f4*>(src + (size_t)z * (DM * DKT));
 #pragma unroll
         for (int i = 0; i < 4; i++) v[i] += t[i];
     }
     *reinterpret_cast<u2*>(a.gx + (int64_t)m * a.ldx + k) = u2{pack2<DT>(v[0], v[1]), pack2<DT>(v[2], v[3])};
 }
 
+
+// ---- 256 (m) x 256 (k) tiles: one wave per SIMD, the side work dealt out between the wave's own MFMAs ----------------
+//
+// The kernel above keeps 16-32 MFMAs of a wave between two workgroup barriers and lets its four waves dequantise in
+// lockstep; large problems run this one instead.  A wave owns 256 m x 64 k of the tile (all 256 accumulation
+// registers); a step covers 64 rows of n: 128 MFMAs per wave between barriers.
+//   * grad_y tile (256 rows x 128 bytes) memory -> LDS by buffer loads with LDS destination, 8 rows per instruction, the
+//     16-byte pieces of a row XOR-swizzled by (row >> 1) & 7 (through the lane's source address) so that the fragment
+//     reads of 16 rows spread over the banks; read through a ring of 8 fragments, one read per four MFMAs;
+//   * weights: a thread owns two units of a step - 32 consecutive k of one row n each - requested two steps ahead,
+//     dequantised to natural k order during the step before they are needed (48 pieces of one to three instructions per
+//     unit, one piece per MFMA gap) and written n-major into the weight tile (64 rows x 512 bytes, 32-byte pieces
+//     swizzled as above); every wave reads its 4 k-tiles back transposed (ds_read_b64_tr_b16, 16 reads per step);
+//   * the step's barrier waits for LDS only and for the grad_y loads (explicit count: the weight requests made after them
+//     stay in flight).
+// Slices of N for small grids as above (float32 partial tiles + qdgrad_reduce_kernel).  Needs K % 256 == 0, N % 64 == 0.
+constexpr int QM = 256, QK = 256, QN = 64;
+
+template <int OFF>
+BW_DEV void lds_read_b128_asm(h8& dst, uint32_t addr) {       // (assembly: an LDS read the compiler would order behind the loads to LDS in flight)
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(OFF));
+}
+template <int OFF>
+BW_DEV void lds_read_tr_asm(u2& dst, uint32_t addr) {
+    asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(OFF));
+}
+template <int DT>
+BW_DEV void mfma_acc_agpr(f4& acc, const h8& a, const h8& b) {  // accumulators in the AGPR file: all 256 VGPRs stay free for operands
+    if constexpr (DT == BW_F16) asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
+    else asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
+}
+BW_DEV __amdgpu_buffer_rsrc_t dgrad_rsrc(const void* p, uint32_t bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), (short)0, (int)bytes, 0x00020000);
+}
+
+template <int BITS, int GROUP, int DT>
+__global__ __launch_bounds__(256) void qdgrad256_kernel(const DgradArgs a) {
+    constexpr int MT = QM / 16, NT = 4, XRING = 8, MF = QN / 32;
+    constexpr int WL = BITS == 8 ? 2 : 1;                  // 16-byte (8-byte at 2 bits) loads per unit
+    constexpr int REQ = 2 * (WL + 2);                      // requests of one step per thread: two units' words, scale, zero point
+    constexpr int G_BYTES = QM * QN * 2, W_BYTES = QN * QK * 2;
+    constexpr uint32_t kOob = 0x80000000u;
+    static_assert(MF == 2 && XRING <= MT, "schedule below: two MFMA steps of 64 gaps");
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    char* gbuf[2] = {smem, smem + G_BYTES};
+    char* wbuf[2] = {smem + 2 * G_BYTES, smem + 2 * G_BYTES + W_BYTES};
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int nl = lane & 15, kq = lane >> 4;
+    const int tile = (int)blockIdx.x / a.splits, split = (int)blockIdx.x % a.splits;
+    const int m0 = (tile / a.tiles_k) * QM, k0 = (tile % a.tiles_k) * QK;
+    const int s_begin = split * a.steps_per_split, s_end = min(s_begin + a.steps_per_split, a.N / QN);
+    const __amdgpu_buffer_rsrc_t rw = dgrad_rsrc(a.qweight, a.w_bytes), rg = dgrad_rsrc(a.go, a.go_bytes);
+    const __amdgpu_buffer_rsrc_t rs = dgrad_rsrc(a.scale, a.meta_bytes), rz = dgrad_rsrc(a.zp, a.meta_bytes);
+    const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+
+    // weight units of a thread: unit e: row n = tid / 8 + 32 e of the step, the 32 k at block tid % 8 of the tile's 256
+    const int un = tid >> 3, ub = tid & 7;
+    uint32_t w_off[2], m_off[2], w_dst[2];
+#pragma unroll
+    for (int e = 0; e < 2; e++) {
+        const int n = un + 32 * e;
+        w_off[e] = (uint32_t)n * a.row_bytes + (uint32_t)(k0 + 32 * ub) * BITS / 8;
+        m_off[e] = ((uint32_t)n * a.groups + (uint32_t)(k0 + 32 * ub) / GROUP) * 2;
+        // 32-byte pieces 2 ub and 2 ub + 1 of row n; the swizzle touches the low 3 bits of the piece index, so the second
+        // piece sits at the first one's address ^ 32
+        w_dst[e] = n * (QK * 2) + (((2 * ub) ^ w_swizzle(n)) * 32);
+    }
+    struct WSet { u4 w[2][WL]; uint32_t s[2], z[2]; };
+    WSet set0, set1;
+    auto w_req = [&](int step, WSet& ws) {                 // past the slice's end: offsets beyond every buffer read as zero
+        const uint32_t so = step < s_end ? (uint32_t)step * QN * a.row_bytes : kOob;
+        const uint32_t mo = step < s_end ? (uint32_t)step * QN * a.groups * 2 : kOob;
+#pragma unroll
+        for (int e = 0; e < 2; e++) {
+            if constexpr (BITS == 2) {
+                const u2 v = __builtin_amdgcn_raw_buffer_load_b64(rw, w_off[e] + so, 0, 0);
+                ws.w[e][0][0] = v[0];
+                ws.w[e][0][1] = v[1];
+            } else {
+#pragma unroll
+                for (int l = 0; l < WL; l++) ws.w[e][l] = __builtin_amdgcn_raw_buffer_load_b128(rw, w_off[e] + so + 16 * l, 0, 0);
+            }
+            ws.s[e] = __builtin_amdgcn_raw_buffer_load_b16(rs, m_off[e] + mo, 0, 0);
+            ws.z[e] = __builtin_amdgcn_raw_buffer_load_b16(rz, m_off[e] + mo, 0, 0);
+        }
+    };
+    // grad_y tile: a wave brings in rows 64 wave .. + 63, unit u = 8 rows; lane L: row L / 8, LDS piece L % 8 holds source
+    // piece (L % 8) ^ s, s = (row >> 1) & 7 = (4 (u & 1) + (L >> 4)) & 7
+    uint32_t gd_base[2];
+#pragma unroll
+    for (int par = 0; par < 2; par++) {
+        const int sw = (4 * par + (lane >> 4)) & 7;
+        gd_base[par] = (uint32_t)((m0 + 64 * wave + (lane >> 3)) * a.ldg) * 2 + (((lane & 7) ^ sw) * 16);
+    }
+    auto g_dma = [&](int u, int step, char* buf) {
+        uint32_t so = step < s_end ? (uint32_t)(u * 8 * a.ldg) * 2 + (uint32_t)step * QN * 2 : kOob;
+        asm("" : "+s"(so));                                   // one scalar sum, one VALU add
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rg, (__attribute__((address_space(3))) void*)(buf + (64 * wave_u + 8 * u) * 128), 16,
+                                                 gd_base[u & 1] + so, 0, 0, 0);
+    };
+    // grad_y fragment (m-tile i, MFMA step t) of the lane: row 16 i + nl, source piece 4 t + kq
+    uint32_t fa[MF];
+#pragma unroll
+    for (int t = 0; t < MF; t++) fa[t] = (uint32_t)(nl * 128 + (((4 * t + kq) ^ (nl >> 1)) * 16));
+    // weight fragment (k-tile j of the wave, step t, half h): the lane points at row 32 t + 8 kq + 4 h + (nl >> 2), piece
+    // 4 wave + j, 8 (nl & 3) bytes in; the swizzle of those rows is the same for both h and both t
+    const int tsw = w_swizzle(8 * kq + (nl >> 2));
+    uint32_t ta[2], tp[NT];
+#pragma unroll
+    for (int h = 0; h < 2; h++) ta[h] = (uint32_t)((8 * kq + 4 * h + (nl >> 2)) * (QK * 2) + (nl & 3) * 8);
+#pragma unroll
+    for (int j = 0; j < NT; j++) tp[j] = (uint32_t)(((4 * wave + j) ^ tsw) * 32);
+
+    f4 acc[MT][NT];
+#pragma unroll
+    for (int i = 0; i < MT; i++)
+#pragma unroll
+        for (int j = 0; j < NT; j++) acc[i][j] = f4{0.f, 0.f, 0.f, 0.f};
+    h8 xf[XRING];
+    u2 wfr[MF][NT][2];                                     // [t][j][h]
+    uint32_t od[2][16];                                    // a unit's 16 pairs in the gradient's type, natural k order
+    h2 ot[2][16];
+    GroupConstNat<BITS> gcn[2];
+
+    // Piece P (0 .. 47) of the dequantisation of unit e of `ws`: extract (1-3 instructions), exact q - z, times the scale.
+    auto piece = [&](auto ec, auto pc, const WSet& ws) {
+        constexpr int e = decltype(ec)::value, P = decltype(pc)::value;
+        if constexpr (P == 0) gcn[e].set(__builtin_bit_cast(_Float16, (uint16_t)ws.s[e]), __builtin_bit_cast(_Float16, (uint16_t)ws.z[e]));
+        auto finish = [&](int idx) {                          // ot[e][idx] = exact q - z  ->  od[e][idx]
+            if constexpr (DT == BW_F16) od[e][idx] = as_u32(ot[e][idx] * gcn[e].s);
+            else {
+                const float sf = (float)gcn[e].s[0];
+                od[e][idx] = pack2<DT>(__fmul_rn((float)ot[e][idx][0], sf), __fmul_rn((float)ot[e][idx][1], sf));
+            }
+        };
+        if constexpr (BITS == 4) {
+            constexpr int wd = P / 12, v = P % 12;
+            const uint32_t word = ws.w[e][0][wd];
+            const h2 kk = h2{(_Float16)1.0f, (_Float16)0.0625f};
+            if constexpr (v < 4) {
+                const uint32_t pq = v < 2 ? __builtin_amdgcn_perm(word, word, 0x01000100u) : __builtin_amdgcn_perm(word, word, 0x03020302u);
+                ot[e][4 * wd + v] = as_h2(and_or((v & 1) ? pq >> 8 : pq, 0x00F0000Fu, kMagic));
+            } else if constexpr (v < 8) {
+                ot[e][4 * wd + v - 4] = __builtin_elementwise_fma(ot[e][4 * wd + v - 4], kk, gcn[e].zz);
+            } else {
+                finish(4 * wd + v - 8);
+            }
+        } else if constexpr (BITS == 2) {
+            constexpr int hw = P / 12, v = P % 12;             // half-word hw of the unit's two words
+            const uint32_t word = ws.w[e][0][hw / 2];
+            const h2 ka = h2{(_Float16)1.0f, (_Float16)0.25f}, kb = h2{(_Float16)0.0625f, (_Float16)0.015625f};
+            if constexpr (v < 4) {
+                const uint32_t p = (hw & 1) ? __builtin_amdgcn_perm(word, word, 0x03020302u) : __builtin_amdgcn_perm(word, word, 0x01000100u);
+                ot[e][4 * hw + v] = as_h2(and_or(v < 2 ? p : p >> 8, (v & 1) ? 0x00C00030u : 0x000C0003u, kMagic));
+            } else if constexpr (v < 8) {
+                ot[e][4 * hw + v - 4] = __builtin_elementwise_fma(ot[e][4 * hw + v - 4], (v & 1) ? kb : ka, (v & 1) ? gcn[e].zz2 : gcn[e].zz);
+            } else {
+                finish(4 * hw + v - 8);
+            }
+        } else {
+            constexpr int pr = P / 3, op = P % 3;              // pair pr: bytes 2 (pr % 2), + 1 of word pr / 2
+            const uint32_t word = ws.w[e][pr / 8][(pr / 2) % 4];
+            if constexpr (op == 0) ot[e][pr] = as_h2(__builtin_amdgcn_perm(0x64646464u, word, (pr & 1) ? 0x04030402u : 0x04010400u));
+            else if constexpr (op == 1) ot[e][pr] = ot[e][pr] + gcn[e].zz;
+            else finish(pr);
+        }
+    };
+    auto w_store = [&](auto ec, auto qc, char* wt) {          // 16-byte quarter q (pairs 4 q .. 4 q + 3) of unit e
+        constexpr int e = decltype(ec)::value, q = decltype(qc)::value;
+        char* d = wt + ((q & 2) ? (w_dst[e] ^ 32) : w_dst[e]) + (q & 1) * 16;
+        *reinterpret_cast<u4*>(d) = u4{od[e][4 * q], od[e][4 * q + 1], od[e][4 * q + 2], od[e][4 * q + 3]};
+    };
+
+    auto step = [&](int s, const char* gcur, char* gnxt, const char* wcur, char* wnxt, WSet& ws, const WSet& wsn) {
+        // ws: the words that became wcur a step ago - free, so the requests of step s + 2 land there; wsn: the words of
+        // step s + 1, dequantised into wnxt during this step
+        __builtin_amdgcn_sched_barrier(0);
+        const uint32_t g_a = (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) char*)gcur;
+        const uint32_t w_a = (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) char*)wcur;
+        static_for<0, MF>([&](auto tc) {                       // the step's weight fragments, t = 0 first
+            constexpr int t = decltype(tc)::value;
+            static_for<0, NT>([&](auto jc) {
+                constexpr int j = decltype(jc)::value;
+                lds_read_tr_asm<t * 32 * QK * 2>(wfr[t][j][0], w_a + ta[0] + tp[j]);
+                lds_read_tr_asm<t * 32 * QK * 2>(wfr[t][j][1], w_a + ta[1] + tp[j]);
+            });
+        });
+        auto frag_read = [&](auto tc, auto ic) {
+            constexpr int t = decltype(tc)::value, i = decltype(ic)::value;
+            lds_read_b128_asm<i * 16 * 128>(xf[(MT * t + i) % XRING], g_a + fa[t]);
+        };
+        static_for<0, XRING>([&](auto Sc) {
+            constexpr int S0 = decltype(Sc)::value;
+            frag_read(std::integral_constant<int, S0 / MT>{}, std::integral_constant<int, S0 % MT>{});
+        });
+        static_for<0, MF>([&](auto tc) {
+            constexpr int t = decltype(tc)::value;
+            static_for<0, NT * MT>([&](auto gcnt) {
+                constexpr int g = decltype(gcnt)::value, i = g / NT, j = g % NT;
+                constexpr int S = MT * t + i, SLAST = MT * MF - 1 - XRING;
+                __builtin_amdgcn_sched_barrier(0);
+                // (the 16 weight-fragment reads were issued before the ring reads and return first)
+                if constexpr (j == 0) __builtin_amdgcn_s_waitcnt(0xC07F | ((XRING - 1 - (S > SLAST + 1 ? S - SLAST - 1 : 0)) << 8));
+                mfma_acc_agpr<DT>(acc[i][j], __builtin_bit_cast(h8, u4{wfr[t][j][0][0], wfr[t][j][0][1], wfr[t][j][1][0], wfr[t][j][1][1]}), xf[S % XRING]);
+                __builtin_amdgcn_sched_barrier(0);
+                // ---- side work of gap G = 64 t + g: the first three gaps of a slot take one dequantisation piece each
+                // (unit t: 16 slots x 3 = its 48 pieces), the fourth belongs to the slot's ring read
+                constexpr int G = 64 * t + g;
+                if constexpr (j < 3) piece(std::integral_constant<int, t>{}, std::integral_constant<int, 3 * i + j>{}, wsn);
+                if constexpr (j == 3 && i >= 12) w_store(std::integral_constant<int, t>{}, std::integral_constant<int, i - 12>{}, wnxt);
+                if constexpr (t == 0 && j == 1 && i < 8) g_dma(i, s + 1, gnxt);
+                if constexpr (j == NT - 1) {
+                    constexpr int S2 = S + XRING;
+                    if constexpr (S2 < MT * MF) frag_read(std::integral_constant<int, S2 / MT>{}, std::integral_constant<int, S2 % MT>{});
+                }
+                (void)G;
+                asm volatile("" ::: "memory");
+            });
+        });
+        __builtin_amdgcn_sched_barrier(0);
+        w_req(s + 2, ws);
+        asm volatile("" ::: "memory");
+        wait_loads<REQ>();                                    // the next grad_y tile has landed: only the requests just made are out
+        lds_barrier();
+    };
+
+    // prologue: grad_y tile of the first step, the words of the first two steps, the first weight tile
+#pragma unroll
+    for (int u = 0; u < 8; u++) g_dma(u, s_begin, gbuf[0]);
+    w_req(s_begin, set0);
+    w_req(s_begin + 1, set1);
+    asm volatile("" ::: "memory");
+    static_for<0, 2>([&](auto ec) {
+        static_for<0, 48>([&](auto pc) { piece(ec, pc, set0); });
+        static_for<0, 4>([&](auto qc) { w_store(ec, qc, wbuf[0]); });
+    });
+    asm volatile("" ::: "memory");
+    wait_loads<REQ>();
+    lds_barrier();
+    // whole passes of two steps (a step past the slice's end multiplies zeros)
+    for (int s = s_begin; s < s_end; s += 2) {
+        step(s, gbuf[0], gbuf[1], wbuf[0], wbuf[1], set0, set1);
+        step(s + 1, gbuf[1], gbuf[0], wbuf[1], wbuf[0], set1, set0);
+    }
+    // acc[i][j][r] = grad_x[m0 + 16 i + nl][k0 + 64 wave + 16 j + 4 kq + r]
+    if (a.splits > 1) {
+        float* dst = a.ws + (size_t)blockIdx.x * (QM * QK) + 64 * wave + 4 * kq;
+#pragma unroll
+        for (int i = 0; i < MT; i++) {
+            if (m0 + 16 * i + nl >= a.M) continue;
+#pragma unroll
+            for (int j = 0; j < NT; j++) *reinterpret_cast<f4*>(dst + (16 * i + nl) * QK + 16 * j) = acc[i][j];
+        }
+        return;
+    }
+    // the wave's 256 x 64 block leaves through its quarter of LDS as whole 128-byte rows
+    __builtin_amdgcn_s_waitcnt(0xC07F);
+    char* ob = smem + wave * (QM * 128);
+#pragma unroll
+    for (int j = 0; j < NT; j++) {
+        const int ch = 4 * j + kq;
+#pragma unroll
+        for (int i = 0; i < MT; i++) {
+            const int row = 16 * i + nl;
+            const f4 v = acc[i][j];
+            *reinterpret_cast<u2*>(ob + row * 128 + (((ch >> 1) ^ (row & 7)) * 16) + (ch & 1) * 8) = u2{pack2<DT>(v[0], v[1]), pack2<DT>(v[2], v[3])};
+        }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    const bool wide = a.ldx % 8 == 0 && (((uintptr_t)a.gx) & 15) == 0;
+#pragma unroll
+    for (int q = 0; q < QM / 8; q++) {
+        const int row = 8 * q + (lane >> 3), unit = lane & 7;
+        const u4 v = *reinterpret_cast<const u4*>(ob + row * 128 + ((unit ^ (row & 7)) * 16));
+        if (m0 + row >= a.M) continue;
+        _Float16* dst = a.gx + (int64_t)(m0 + row) * a.ldx + k0 + 64 * wave + unit * 8;
+        if (wide) *reinterpret_cast<u4*>(dst) = v;
+        else {
+            *reinterpret_cast<u2*>(dst) = u2{v[0], v[1]};
+            *reinterpret_cast<u2*>(dst + 4) = u2{v[2], v[3]};
+        }
+    }
+}
+
 struct DgradPlan {
-    int mt, tiles_k, tiles, splits, steps_per_split;
+    int mt, tiles_k, tiles, splits, steps_per_split;   // mt = 16: the 256 x 256 kernel
     size_t ws_bytes;
 };
 
@@ -284,6 +571,42 @@ inline int dgrad_cus() {
 // Three workgroups fit a CU and hide each other's barriers.  With fewer tiles than two per CU N is cut into slices:
 // to two workgroups per CU (three measured slower: more partial-tile traffic) when a slice keeps at least 24 steps,
 // else to one per CU with at least 8 (short slices pay their prologue and the partial tiles' traffic).
+// The 256 x 256 kernel takes a problem when it is large enough: at least 3072 tile-steps (tiles x steps of 64 rows of n;
+// measured against the kernel above on 4096 x 4096, 4096 -> 14336 and 14336 -> 4096 at 256 / 512 / 2048 rows: 0.69-0.84
+// of its time from 3584 tile-steps up, one tie; 1.16-1.33 at 1024 and 2048), more than 128 rows, K in whole tiles, N in
+// whole steps, extents that fit the 32-bit offsets of buffer addressing - and, below one workgroup per CU, a workspace:
+// N is then cut into slices of at least 8 steps so that every CU has one.
+inline bool dgrad256_shape(int64_t M, int64_t N, int64_t K, int64_t ldg, int bits, int group) {
+    const int64_t lim = (int64_t)1 << 31;
+    return M > 128 && K % QK == 0 && N % QN == 0 && ((M + QM - 1) / QM) * (K / QK) * (N / QN) >= 3072 &&
+           N * (K * bits / 8) < lim && (M + QM) * ldg * 2 < lim && N * (K / group) * 2 < lim;
+}
+
+inline DgradPlan dgrad256_plan(int64_t M, int64_t N, int64_t K, bool have_workspace) {
+    DgradPlan p;
+    p.mt = 16;
+    p.tiles_k = (int)(K / QK);
+    p.tiles = p.tiles_k * (int)((M + QM - 1) / QM);
+    const int nsteps = (int)(N / QN);
+    p.splits = 1;
+    p.steps_per_split = nsteps;
+    p.ws_bytes = 0;
+    const int cus = dgrad_cus();
+    if (!have_workspace || p.tiles > cus / 2) return p;
+    int s = cus / p.tiles;
+    if (s > nsteps / 8) s = nsteps / 8;
+    if (s > 16) s = 16;
+    if (s < 2) return p;
+    int sps = (nsteps + s - 1) / s;
+    sps += sps & 1;                                          // the loop runs two steps per pass
+    s = (nsteps + sps - 1) / sps;
+    if (s < 2) return p;
+    p.splits = s;
+    p.steps_per_split = sps;
+    p.ws_bytes = (size_t)p.tiles * s * QM * QK * sizeof(float);
+    return p;
+}
+
 inline DgradPlan dgrad_plan(int64_t M, int64_t N, int64_t K, bool have_workspace) {
     DgradPlan p;
     p.mt = M > 512 ? 8 : 4;
@@ -333,7 +656,41 @@ int launch_dgrad_mt(const DgradArgs& a, const DgradPlan& p, hipStream_t stream) 
 }
 
 template <int BITS, int GROUP, int DT>
+int launch_dgrad256(DgradArgs a, void* workspace, size_t workspace_bytes, hipStream_t stream) {
+    const DgradPlan p = dgrad256_plan(a.M, a.N, a.K, workspace != nullptr);
+    if (p.ws_bytes > workspace_bytes) return BW_EWORKSPACE;
+    a.ws = (float*)workspace;
+    a.tiles_k = p.tiles_k;
+    a.splits = p.splits;
+    a.steps_per_split = p.steps_per_split;
+    a.go_bytes = (uint32_t)((((int64_t)a.M - 1) * a.ldg + a.N) * 2);
+    a.w_bytes = (uint32_t)((int64_t)a.N * a.row_bytes);
+    a.meta_bytes = (uint32_t)((int64_t)a.N * a.groups * 2);
+    auto kern = qdgrad256_kernel<BITS, GROUP, DT>;
+    constexpr int lds = 2 * (QM * QN * 2) + 2 * (QN * QK * 2);
+    static uint64_t big_lds_devices = 0;                   // per instantiation
+    if (!bw_allow_big_lds(reinterpret_cast<const void*>(kern), big_lds_devices)) return BW_ELAUNCH;
+    hipLaunchKernelGGL(kern, dim3((unsigned)(p.tiles * p.splits)), dim3(256), lds, stream, a);
+    if (hipGetLastError() != hipSuccess) return BW_ELAUNCH;
+    if (p.splits > 1) {
+        hipLaunchKernelGGL((qdgrad_reduce_kernel<QM, DT, QK>), dim3(QM * QK / 4 / 256, (unsigned)p.tiles), dim3(256), 0, stream, a);
+        if (hipGetLastError() != hipSuccess) return BW_ELAUNCH;
+    }
+    return BW_OK;
+}
+
+// which kernel a call gets: the 256 x 256 one when the problem is large enough and, where its grid would leave CUs
+// idle, a workspace is on offer
+inline bool dgrad_use256(int64_t M, int64_t N, int64_t K, int64_t ldg, int bits, int group, bool have_workspace) {
+    if (!dgrad256_shape(M, N, K, ldg, bits, group)) return false;
+    const int64_t tiles = ((M + QM - 1) / QM) * (K / QK);
+    return have_workspace || tiles > dgrad_cus() / 2;
+}
+
+template <int BITS, int GROUP, int DT>
 int launch_dgrad(DgradArgs a, void* workspace, size_t workspace_bytes, hipStream_t stream) {
+    if (dgrad_use256(a.M, a.N, a.K, a.ldg, BITS, GROUP, workspace != nullptr))
+        return launch_dgrad256<BITS, GROUP, DT>(a, workspace, workspace_bytes, stream);
     const DgradPlan p = dgrad_plan(a.M, a.N, a.K, workspace != nullptr);
     if (p.ws_bytes > workspace_bytes) return BW_EWORKSPACE;
     a.ws = (float*)workspace;
@@ -347,7 +704,19 @@ int launch_dgrad(DgradArgs a, void* workspace, size_t workspace_bytes, hipStream
 
 extern "C" size_t bw_qdgrad_workspace_bytes(int64_t M, int64_t N, int64_t K, int bits, int group) {
     if (!bw_shape_ok(N, K, bits, group) || !dgrad_fast_shape(M, N, K, N, K, bits, group)) return 0;
-    return dgrad_plan(M, N, K, true).ws_bytes;
+    // enough for either kernel (the call's own leading dimensions decide between them)
+    const size_t a = dgrad_plan(M, N, K, true).ws_bytes;
+    const size_t b = dgrad256_shape(M, N, K, N, bits, group) ? dgrad256_plan(M, N, K, true).ws_bytes : 0;
+    return a > b ? a : b;
+}
+
+// Rows of grad_x a workgroup owns for this shape (with a workspace on offer): 128 or 256 for the kernel that walks N in
+// steps of 32 rows, 257 for the 256 x 256 kernel, 0 where the fused path does not apply.  A diagnostic, and what the
+// Python backward asks before it chooses between this kernel and dequantise + library GEMM.
+extern "C" int bw_qdgrad_tile_rows(int64_t M, int64_t N, int64_t K, int bits, int group) {
+    if (!bw_shape_ok(N, K, bits, group) || !dgrad_fast_shape(M, N, K, N, K, bits, group)) return 0;
+    if (dgrad_use256(M, N, K, N, bits, group, true)) return 257;
+    return M > 512 ? 256 : 128;
 }
 
 extern "C" int bw_qdgrad(const void* grad_y, int act_dtype, int64_t M, int64_t N, int64_t ldg, const int32_t* qweight,

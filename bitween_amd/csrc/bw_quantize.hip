@@ -568,7 +568,7 @@ extern "C" int bw_dequantize(const int32_t* qweight, const void* scale, int scal
     return BW_EINVAL;
 }
 
-extern "C" int bw_abi_version(void) { return 9; }
+extern "C" int bw_abi_version(void) { return 10; }
 
 extern "C" const char* bw_strerror(int status) {
     switch (status) {

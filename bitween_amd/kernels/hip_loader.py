@@ -20,9 +20,9 @@ BW_F16, BW_BF16, BW_F32, BW_I32, BW_F64 = 0, 1, 2, 3, 4
 BW_SCALE_RECIPROCAL = 0x100   # flag for math_dtype: scale = (max - min) * fl32(1 / Qmax), as eager torch computes it on a GPU
 _DTYPE_CODE = {torch.float16: BW_F16, torch.bfloat16: BW_BF16, torch.float32: BW_F32, torch.int32: BW_I32, torch.float64: BW_F64}
 
-ABI_VERSION = 9            # what bw_abi_version() of a matching library returns
+ABI_VERSION = 10           # what bw_abi_version() of a matching library returns
 ENTRY_POINTS = ("bw_abi_version", "bw_strerror", "bw_quantize_pack", "bw_quantize_pack_add", "bw_dequantize", "bw_qgemv", "bw_qgemm",
-                "bw_qgemm_ws", "bw_qgemm_static", "bw_qgemm_workspace_bytes", "bw_qgemm_tile_rows", "bw_qlinear", "bw_qdgrad", "bw_qdgrad_workspace_bytes", "bw_cast_bf16_f16", "bw_qlinear_decode_rows", "bw_qgemv_last_kernel")
+                "bw_qgemm_ws", "bw_qgemm_static", "bw_qgemm_workspace_bytes", "bw_qgemm_tile_rows", "bw_qlinear", "bw_qdgrad", "bw_qdgrad_workspace_bytes", "bw_qdgrad_tile_rows", "bw_cast_bf16_f16", "bw_qlinear_decode_rows", "bw_qgemv_last_kernel")
 
 
 class BitweenHipError(RuntimeError):
@@ -63,6 +63,8 @@ def load():
     lib.bw_qgemm_tile_rows.restype = i32
     lib.bw_qdgrad_workspace_bytes.argtypes = [i64, i64, i64, i32, i32]
     lib.bw_qdgrad_workspace_bytes.restype = ctypes.c_size_t
+    lib.bw_qdgrad_tile_rows.argtypes = [i64, i64, i64, i32, i32]
+    lib.bw_qdgrad_tile_rows.restype = i32
     lib.bw_qdgrad.argtypes = [vp, i32, i64, i64, i64, vp, vp, vp, i64, i32, i32, vp, i64, vp, ctypes.c_size_t, vp]
     lib.bw_qdgrad.restype = i32
     lib.bw_cast_bf16_f16.argtypes = [vp, i64, i64, i64, vp, i64, vp]
@@ -308,6 +310,14 @@ def decode_with_plan(plan, x, m):
             return None
         _check(st, "bw_qlinear")
     return y
+
+
+def input_grad_prefers_fused(m, n, k, bits, group_size, max_rows, large_max_rows):
+    """Whether the backward should take the fused kernel for an m-row gradient: up to `max_rows` rows always (the
+    kernel that walks N in steps of 32 rows); up to `large_max_rows` where the library's plan is its 256 x 256 kernel,
+    which beats dequantise + library GEMM there (measured on Llama-shaped layers: 0.45-1.0 of its time up to 2048
+    rows, 1.0-1.13 at 4096)."""
+    return m <= max_rows or (m <= large_max_rows and load().bw_qdgrad_tile_rows(m, n, k, bits, group_size) == 257)
 
 
 def quantized_input_grad(grad_y, qweight, scale, zero_point, bits, group_size):

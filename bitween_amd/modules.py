@@ -13,7 +13,8 @@ from . import functional as _functional
 from .kernels import hip_loader as _hip
 
 
-FUSED_DGRAD_MAX_ROWS = 512       # measured on MI355X, Llama-shaped layers: fused wins up to here (3x at 128 rows)
+FUSED_DGRAD_MAX_ROWS = 512       # measured on MI355X, Llama-shaped layers: the 128-row fused kernel wins up to here (3x at 128 rows)
+FUSED_DGRAD_LARGE_MAX_ROWS = 2048  # ... and the 256 x 256 kernel, where the library plans it (large layers), up to here
 
 
 class QuantizedLinearFunction(torch.autograd.Function):
@@ -37,11 +38,12 @@ class QuantizedLinearFunction(torch.autograd.Function):
         x, qweight, scale, zero_point, bias = ctx.saved_tensors
         grad_input = None
         if ctx.needs_input_grad[0]:
-            # float16 / bfloat16 gradients, up to FUSED_DGRAD_MAX_ROWS rows: one fused kernel, the weights are never
-            # materialised.  Beyond that the library GEMM on dequantised weights is faster (the fused kernel
-            # re-dequantises the weights for every 128 rows of grad_output).
+            # float16 / bfloat16 gradients: one fused kernel, the weights are never materialised - up to
+            # FUSED_DGRAD_MAX_ROWS rows always, up to FUSED_DGRAD_LARGE_MAX_ROWS where the library runs its 256 x 256
+            # kernel (large layers); otherwise the library GEMM on dequantised weights is faster.
             go2 = grad_output.reshape(-1, grad_output.shape[-1])
-            if grad_output.dtype in (torch.float16, torch.bfloat16) and grad_output.is_cuda and go2.shape[0] <= FUSED_DGRAD_MAX_ROWS:
+            if grad_output.dtype in (torch.float16, torch.bfloat16) and grad_output.is_cuda and _hip.input_grad_prefers_fused(
+                    go2.shape[0], qweight.shape[0], x.shape[-1], ctx.bits, ctx.group_size, FUSED_DGRAD_MAX_ROWS, FUSED_DGRAD_LARGE_MAX_ROWS):
                 gx = _hip.quantized_input_grad(go2, qweight, scale, zero_point, ctx.bits, ctx.group_size)
                 if gx is not None:
                     return gx.view(*grad_output.shape[:-1], gx.shape[-1]), None, None, None, None, None, None

@@ -182,8 +182,14 @@ int bw_cast_bf16_f16(const void* x, int64_t rows, int64_t cols, int64_t ldx, voi
  * return BW_EUNSUPPORTED (the Python backward then dequantises with bw_dequantize and calls the library GEMM).
  * When M * K is small the reduction over N is cut into slices whose float32 partial sums go through a
  * caller-provided workspace of bw_qdgrad_workspace_bytes(...) bytes (16-byte aligned; 0 = none needed);
- * workspace == NULL runs unsliced. */
+ * workspace == NULL runs unsliced.
+ * Two kernels: one that owns 128 (256 beyond 512 rows) x 128 tiles of grad_x and walks N in steps of 32 rows, and - for
+ * large problems with K % 256 == 0 and N % 64 == 0 - one with 256 x 256 tiles and steps of 64 rows;
+ * bw_qdgrad_tile_rows tells which a shape gets (128, 256, 257 = the 256 x 256 kernel, 0 = no fused path): a diagnostic,
+ * and what the Python backward asks before it prefers this entry point over dequantise + GEMM beyond 512 rows. */
 size_t bw_qdgrad_workspace_bytes(int64_t M, int64_t N, int64_t K, int bits, int group);
+
+int bw_qdgrad_tile_rows(int64_t M, int64_t N, int64_t K, int bits, int group);
 
 int bw_qdgrad(const void* grad_y, int act_dtype, int64_t M, int64_t N, int64_t ldg,
               const int32_t* qweight, const void* scale16, const void* zp16,

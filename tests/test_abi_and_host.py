@@ -28,7 +28,7 @@ def test_library_exports_every_declared_symbol():
     for name in declared:
         assert hasattr(lib, name), name
     lib.bw_abi_version.restype = ctypes.c_int
-    assert lib.bw_abi_version() == hip_loader.ABI_VERSION == 9
+    assert lib.bw_abi_version() == hip_loader.ABI_VERSION == 10
     lib.bw_strerror.restype = ctypes.c_char_p
     assert lib.bw_strerror(0) == b"ok" and b"invalid" in lib.bw_strerror(-1)
 

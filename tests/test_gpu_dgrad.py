@@ -231,3 +231,56 @@ def test_module_backward_takes_the_fused_kernel_for_bfloat16_gradients():
     w = bitween_amd.dequantize_rtn(q.qweight, q.scale, q.zero_point, 128, 4).to(torch.bfloat16)
     want = go.float() @ w.float()
     assert (got.float() - want).abs().max().item() <= 2.0 ** -7 * want.abs().max().item()
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("bits,g", COMBOS)
+def test_dgrad_256_tiles_vs_oracle(bits, g, dtype):
+    """Large problems run the 256 x 256 kernel (bw_qdgrad_tile_rows == 257): grad_y tile memory -> LDS by buffer loads,
+    the dequantised weight tile read transposed from LDS, steps of 64 rows of n.  Ragged M (1100 rows: five row tiles, the
+    last 76 rows high), rows of grad_y and grad_x padded, N sliced through the workspace (20 tiles on 256 CUs) and, where
+    the grid is large enough without one, unsliced; sampled rows against the oracle, one-hot rows return rows of the
+    weight in the gradient's type bit for bit, the whole result against the library GEMM on the dequantised weight."""
+    from bitween_amd.kernels import hip_loader
+    lib = hip_loader.load()
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    tdt, code = (torch.float16, 0) if dtype == "f16" else (torch.bfloat16, 1)
+    for (m, n, k) in ((1100, 64 * 154, 1024), (300, 64 * 800, 512), (256 * 160 + 9, 64 * 6, 1024)):
+        assert lib.bw_qdgrad_tile_rows(m, n, k, bits, g) == 257
+        _, qw, s16, z16, _ = quantized_layer(n, k, bits, g, seed=n + k + bits + g + 5, outliers=True, bias=False)
+        d = [to_gpu(a) for a in (qw, s16, z16)]
+        wt = orc.dequantize_f16(qw, s16, z16, g, bits).astype(np.float32) if dtype == "f16" else orc.dequantize_bf16(qw, s16, z16, g, bits)
+        gen = torch.Generator(device="cuda").manual_seed(m + n + bits)
+        ldg, ldx = n + 8, k + 4
+        gobuf = torch.full((m, ldg), float("nan"), dtype=tdt, device="cuda")
+        go = torch.randn(m, n, device="cuda", generator=gen).to(tdt)
+        hot = {0: 0, 1: n - 1, m // 2: n // 2 + 1, m - 1: 63}
+        for r, c in hot.items():
+            go[r] = 0
+            go[r, c] = 1.0
+        gobuf[:, :n] = go
+        need = lib.bw_qdgrad_workspace_bytes(m, n, k, bits, g)
+        ws = torch.empty(max(need, 16), dtype=torch.uint8, device="cuda")
+        wg = torch.from_numpy(np.ascontiguousarray(wt)).cuda().to(tdt)
+        ref_all = (go @ wg).float()
+        tiles = -(-m // 256) * (k // 256)
+        for use_ws in ((True, False) if tiles > 128 else (True,)):     # without a workspace small grids stay on the other kernel
+            gx = torch.full((m, ldx), 7.0, dtype=tdt, device="cuda")
+            st = lib.bw_qdgrad(gobuf.data_ptr(), code, m, n, ldg, d[0].data_ptr(), d[1].data_ptr(), d[2].data_ptr(), k, bits, g,
+                               gx.data_ptr(), ldx, ws.data_ptr() if (use_ws and need) else None, need if use_ws else 0, stream)
+            torch.cuda.synchronize()
+            assert st == 0
+            assert (gx[:, k:] == 7.0).all()                          # nothing written past a row's K outputs
+            got_all = gx[:, :k].float()
+            assert torch.isfinite(got_all).all()
+            assert ((got_all - ref_all).abs().max() <= 2.0 ** -7 * ref_all.abs().max()).item()
+            rows = np.unique(np.concatenate([np.arange(0, m, max(1, m // 24)), np.arange(max(0, m - 5), m), np.array(list(hot))]))
+            go_np = go[torch.from_numpy(rows).cuda()].float().cpu().numpy()
+            ref = orc.qlinear_backward(go_np if dtype == "bf16" else go_np.astype(np.float16), qw, s16, z16, bits, g,
+                                       **({"dtype": "bf16"} if dtype == "bf16" else {}))
+            got = gx[torch.from_numpy(rows).cuda()][:, :k].double().cpu().numpy()
+            mag = np.abs(go_np.astype(np.float64)) @ np.abs(wt.astype(np.float64))
+            bound = (2.0 ** -10 if dtype == "f16" else 2.0 ** -8) * np.abs(ref) + 2e-6 * mag + 1e-7
+            assert (np.abs(got - ref) <= bound).all(), float((np.abs(got - ref) / bound).max())
+            for r, c in hot.items():
+                assert np.array_equal(gx[r, :k].float().cpu().numpy(), wt[c].astype(np.float32))
