@@ -302,21 +302,23 @@ BW_DEV __amdgpu_buffer_rsrc_t dgrad_rsrc(const void* p, uint32_t bytes) {
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), (short)0, (int)bytes, 0x00020000);
 }
 
-template <int BITS, int GROUP, int DT>
+template <int BITS, int GROUP, int DT, int MT>     // MT = 16: 256 rows of m per tile; MT = 8: 128 rows (twice the dequantisation per MFMA)
 __global__ __launch_bounds__(256) void qdgrad256_kernel(const DgradArgs a) {
-    constexpr int MT = QM / 16, NT = 4, XRING = 8, MF = QN / 32;
+    constexpr int QMv = MT * 16, NT = 4, XRING = 8, MF = QN / 32;
+    constexpr int WR = QMv / 4, UNITS = WR / 8;            // rows of grad_y a wave brings in, 8 per instruction
+    constexpr int PPG = 48 / (3 * MT);                     // dequantisation pieces per gap: a unit's 48 over the first three gaps of MT slots
     constexpr int WL = BITS == 8 ? 2 : 1;                  // 16-byte (8-byte at 2 bits) loads per unit
     constexpr int REQ = 2 * (WL + 2);                      // requests of one step per thread: two units' words, scale, zero point
-    constexpr int G_BYTES = QM * QN * 2, W_BYTES = QN * QK * 2;
+    constexpr int G_BYTES = QMv * QN * 2, W_BYTES = QN * QK * 2;
     constexpr uint32_t kOob = 0x80000000u;
-    static_assert(MF == 2 && XRING <= MT, "schedule below: two MFMA steps of 64 gaps");
+    static_assert(MF == 2 && XRING <= MT && (MT == 16 || MT == 8), "schedule below: two MFMA steps, a ring no longer than a step");
     extern __shared__ __attribute__((aligned(16))) char smem[];
     char* gbuf[2] = {smem, smem + G_BYTES};
     char* wbuf[2] = {smem + 2 * G_BYTES, smem + 2 * G_BYTES + W_BYTES};
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int nl = lane & 15, kq = lane >> 4;
     const int tile = (int)blockIdx.x / a.splits, split = (int)blockIdx.x % a.splits;
-    const int m0 = (tile / a.tiles_k) * QM, k0 = (tile % a.tiles_k) * QK;
+    const int m0 = (tile / a.tiles_k) * QMv, k0 = (tile % a.tiles_k) * QK;
     const int s_begin = split * a.steps_per_split, s_end = min(s_begin + a.steps_per_split, a.N / QN);
     const __amdgpu_buffer_rsrc_t rw = dgrad_rsrc(a.qweight, a.w_bytes), rg = dgrad_rsrc(a.go, a.go_bytes);
     const __amdgpu_buffer_rsrc_t rs = dgrad_rsrc(a.scale, a.meta_bytes), rz = dgrad_rsrc(a.zp, a.meta_bytes);
@@ -353,18 +355,18 @@ __global__ __launch_bounds__(256) void qdgrad256_kernel(const DgradArgs a) {
             ws.z[e] = __builtin_amdgcn_raw_buffer_load_b16(rz, m_off[e] + mo, 0, 0);
         }
     };
-    // grad_y tile: a wave brings in rows 64 wave .. + 63, unit u = 8 rows; lane L: row L / 8, LDS piece L % 8 holds source
+    // grad_y tile: a wave brings in rows WR wave .. + WR - 1, unit u = 8 rows; lane L: row L / 8, LDS piece L % 8 holds source
     // piece (L % 8) ^ s, s = (row >> 1) & 7 = (4 (u & 1) + (L >> 4)) & 7
     uint32_t gd_base[2];
 #pragma unroll
     for (int par = 0; par < 2; par++) {
         const int sw = (4 * par + (lane >> 4)) & 7;
-        gd_base[par] = (uint32_t)((m0 + 64 * wave + (lane >> 3)) * a.ldg) * 2 + (((lane & 7) ^ sw) * 16);
+        gd_base[par] = (uint32_t)((m0 + WR * wave + (lane >> 3)) * a.ldg) * 2 + (((lane & 7) ^ sw) * 16);
     }
     auto g_dma = [&](int u, int step, char* buf) {
         uint32_t so = step < s_end ? (uint32_t)(u * 8 * a.ldg) * 2 + (uint32_t)step * QN * 2 : kOob;
         asm("" : "+s"(so));                                   // one scalar sum, one VALU add
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(rg, (__attribute__((address_space(3))) void*)(buf + (64 * wave_u + 8 * u) * 128), 16,
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rg, (__attribute__((address_space(3))) void*)(buf + (WR * wave_u + 8 * u) * 128), 16,
                                                  gd_base[u & 1] + so, 0, 0, 0);
     };
     // grad_y fragment (m-tile i, MFMA step t) of the lane: row 16 i + nl, source piece 4 t + kq
@@ -472,17 +474,16 @@ __global__ __launch_bounds__(256) void qdgrad256_kernel(const DgradArgs a) {
                 if constexpr (j == 0) __builtin_amdgcn_s_waitcnt(0xC07F | ((XRING - 1 - (S > SLAST + 1 ? S - SLAST - 1 : 0)) << 8));
                 mfma_acc_agpr<DT>(acc[i][j], __builtin_bit_cast(h8, u4{wfr[t][j][0][0], wfr[t][j][0][1], wfr[t][j][1][0], wfr[t][j][1][1]}), xf[S % XRING]);
                 __builtin_amdgcn_sched_barrier(0);
-                // ---- side work of gap G = 64 t + g: the first three gaps of a slot take one dequantisation piece each
-                // (unit t: 16 slots x 3 = its 48 pieces), the fourth belongs to the slot's ring read
-                constexpr int G = 64 * t + g;
-                if constexpr (j < 3) piece(std::integral_constant<int, t>{}, std::integral_constant<int, 3 * i + j>{}, wsn);
-                if constexpr (j == 3 && i >= 12) w_store(std::integral_constant<int, t>{}, std::integral_constant<int, i - 12>{}, wnxt);
-                if constexpr (t == 0 && j == 1 && i < 8) g_dma(i, s + 1, gnxt);
+                // ---- side work: the first three gaps of a slot take PPG dequantisation pieces each (unit t: MT slots x 3
+                // gaps = its 48 pieces), the fourth belongs to the slot's ring read
+                if constexpr (j < 3)
+                    static_for<0, PPG>([&](auto pp) { piece(std::integral_constant<int, t>{}, std::integral_constant<int, PPG * (3 * i + j) + decltype(pp)::value>{}, wsn); });
+                if constexpr (j == 3 && i >= MT - 4) w_store(std::integral_constant<int, t>{}, std::integral_constant<int, i - (MT - 4)>{}, wnxt);
+                if constexpr (t == 0 && j == 1 && i < UNITS) g_dma(i, s + 1, gnxt);
                 if constexpr (j == NT - 1) {
                     constexpr int S2 = S + XRING;
                     if constexpr (S2 < MT * MF) frag_read(std::integral_constant<int, S2 / MT>{}, std::integral_constant<int, S2 % MT>{});
                 }
-                (void)G;
                 asm volatile("" ::: "memory");
             });
         });
@@ -495,7 +496,7 @@ __global__ __launch_bounds__(256) void qdgrad256_kernel(const DgradArgs a) {
 
     // prologue: grad_y tile of the first step, the words of the first two steps, the first weight tile
 #pragma unroll
-    for (int u = 0; u < 8; u++) g_dma(u, s_begin, gbuf[0]);
+    for (int u = 0; u < UNITS; u++) g_dma(u, s_begin, gbuf[0]);
     w_req(s_begin, set0);
     w_req(s_begin + 1, set1);
     asm volatile("" ::: "memory");
@@ -513,7 +514,7 @@ __global__ __launch_bounds__(256) void qdgrad256_kernel(const DgradArgs a) {
     }
     // acc[i][j][r] = grad_x[m0 + 16 i + nl][k0 + 64 wave + 16 j + 4 kq + r]
     if (a.splits > 1) {
-        float* dst = a.ws + (size_t)blockIdx.x * (QM * QK) + 64 * wave + 4 * kq;
+        float* dst = a.ws + (size_t)blockIdx.x * (QMv * QK) + 64 * wave + 4 * kq;
 #pragma unroll
         for (int i = 0; i < MT; i++) {
             if (m0 + 16 * i + nl >= a.M) continue;
@@ -522,9 +523,9 @@ __global__ __launch_bounds__(256) void qdgrad256_kernel(const DgradArgs a) {
         }
         return;
     }
-    // the wave's 256 x 64 block leaves through its quarter of LDS as whole 128-byte rows
+    // the wave's QMv x 64 block leaves through its quarter of LDS as whole 128-byte rows
     __builtin_amdgcn_s_waitcnt(0xC07F);
-    char* ob = smem + wave * (QM * 128);
+    char* ob = smem + wave * (QMv * 128);
 #pragma unroll
     for (int j = 0; j < NT; j++) {
         const int ch = 4 * j + kq;
@@ -540,7 +541,7 @@ __global__ __launch_bounds__(256) void qdgrad256_kernel(const DgradArgs a) {
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     const bool wide = a.ldx % 8 == 0 && (((uintptr_t)a.gx) & 15) == 0;
 #pragma unroll
-    for (int q = 0; q < QM / 8; q++) {
+    for (int q = 0; q < QMv / 8; q++) {
         const int row = 8 * q + (lane >> 3), unit = lane & 7;
         const u4 v = *reinterpret_cast<const u4*>(ob + row * 128 + ((unit ^ (row & 7)) * 16));
         if (m0 + row >= a.M) continue;
@@ -571,22 +572,29 @@ inline int dgrad_cus() {
 // Three workgroups fit a CU and hide each other's barriers.  With fewer tiles than two per CU N is cut into slices:
 // to two workgroups per CU (three measured slower: more partial-tile traffic) when a slice keeps at least 24 steps,
 // else to one per CU with at least 8 (short slices pay their prologue and the partial tiles' traffic).
-// The 256 x 256 kernel takes a problem when it is large enough: at least 3072 tile-steps (tiles x steps of 64 rows of n;
-// measured against the kernel above on 4096 x 4096, 4096 -> 14336 and 14336 -> 4096 at 256 / 512 / 2048 rows: 0.69-0.84
-// of its time from 3584 tile-steps up, one tie; 1.16-1.33 at 1024 and 2048), more than 128 rows, K in whole tiles, N in
-// whole steps, extents that fit the 32-bit offsets of buffer addressing - and, below one workgroup per CU, a workspace:
-// N is then cut into slices of at least 8 steps so that every CU has one.
-inline bool dgrad256_shape(int64_t M, int64_t N, int64_t K, int64_t ldg, int bits, int group) {
+// The 256 x 256 kernel takes a problem when it is large enough, counted in tile-steps (tiles x steps of 64 rows of n),
+// K in whole tiles, N in whole steps, extents that fit the 32-bit offsets of buffer addressing - and, below one
+// workgroup per CU, a workspace: N is then cut into slices of at least 8 steps so that every CU has one.  Measured
+// against the stepping kernel on 4096 x 4096, 4096 -> 11008 / 14336 and 14336 -> 4096 at 64 ... 4096 rows:
+//   256 rows of m per tile: beyond 384 rows from 3072 tile-steps (0.63-0.88 of the stepping kernel's time; at 512 rows
+//   level with the 128-row variant for float16 and ahead for bfloat16, whose dequantisation is twice as long);
+//   128 rows of m per tile (twice the dequantisation per MFMA, half the padding): up to 512 rows from 2560 tile-steps
+//   (0.66-0.96; 4096 x 4096 up to 256 rows - 1024 and 2048 tile-steps - is 1.07-1.11 and stays on the stepping kernel).
+// Returns the rows of m per tile (256 or 128), 0 = the stepping kernel.
+inline int dgrad256_rows(int64_t M, int64_t N, int64_t K, int64_t ldg, int bits, int group) {
     const int64_t lim = (int64_t)1 << 31;
-    return M > 128 && K % QK == 0 && N % QN == 0 && ((M + QM - 1) / QM) * (K / QK) * (N / QN) >= 3072 &&
-           N * (K * bits / 8) < lim && (M + QM) * ldg * 2 < lim && N * (K / group) * 2 < lim;
+    if (K % QK || N % QN || N * (K * bits / 8) >= lim || (M + QM) * ldg * 2 >= lim || N * (K / group) * 2 >= lim) return 0;
+    const int64_t col_steps = (K / QK) * (N / QN);
+    if (M > 384 && ((M + QM - 1) / QM) * col_steps >= 3072) return QM;
+    if (M <= 512 && ((M + 127) / 128) * col_steps >= 2560) return 128;
+    return 0;
 }
 
-inline DgradPlan dgrad256_plan(int64_t M, int64_t N, int64_t K, bool have_workspace) {
+inline DgradPlan dgrad256_plan(int64_t M, int64_t N, int64_t K, bool have_workspace, int qm = QM) {
     DgradPlan p;
-    p.mt = 16;
+    p.mt = qm / 16;
     p.tiles_k = (int)(K / QK);
-    p.tiles = p.tiles_k * (int)((M + QM - 1) / QM);
+    p.tiles = p.tiles_k * (int)((M + qm - 1) / qm);
     const int nsteps = (int)(N / QN);
     p.splits = 1;
     p.steps_per_split = nsteps;
@@ -603,7 +611,7 @@ inline DgradPlan dgrad256_plan(int64_t M, int64_t N, int64_t K, bool have_worksp
     if (s < 2) return p;
     p.splits = s;
     p.steps_per_split = sps;
-    p.ws_bytes = (size_t)p.tiles * s * QM * QK * sizeof(float);
+    p.ws_bytes = (size_t)p.tiles * s * qm * QK * sizeof(float);
     return p;
 }
 
@@ -655,9 +663,10 @@ int launch_dgrad_mt(const DgradArgs& a, const DgradPlan& p, hipStream_t stream) 
     return BW_OK;
 }
 
-template <int BITS, int GROUP, int DT>
+template <int BITS, int GROUP, int DT, int MT = 16>
 int launch_dgrad256(DgradArgs a, void* workspace, size_t workspace_bytes, hipStream_t stream) {
-    const DgradPlan p = dgrad256_plan(a.M, a.N, a.K, workspace != nullptr);
+    constexpr int QMv = MT * 16;
+    const DgradPlan p = dgrad256_plan(a.M, a.N, a.K, workspace != nullptr, QMv);
     if (p.ws_bytes > workspace_bytes) return BW_EWORKSPACE;
     a.ws = (float*)workspace;
     a.tiles_k = p.tiles_k;
@@ -666,31 +675,43 @@ int launch_dgrad256(DgradArgs a, void* workspace, size_t workspace_bytes, hipStr
     a.go_bytes = (uint32_t)((((int64_t)a.M - 1) * a.ldg + a.N) * 2);
     a.w_bytes = (uint32_t)((int64_t)a.N * a.row_bytes);
     a.meta_bytes = (uint32_t)((int64_t)a.N * a.groups * 2);
-    auto kern = qdgrad256_kernel<BITS, GROUP, DT>;
-    constexpr int lds = 2 * (QM * QN * 2) + 2 * (QN * QK * 2);
+    auto kern = qdgrad256_kernel<BITS, GROUP, DT, MT>;
+    constexpr int lds = 2 * (QMv * QN * 2) + 2 * (QN * QK * 2);
     static uint64_t big_lds_devices = 0;                   // per instantiation
     if (!bw_allow_big_lds(reinterpret_cast<const void*>(kern), big_lds_devices)) return BW_ELAUNCH;
     hipLaunchKernelGGL(kern, dim3((unsigned)(p.tiles * p.splits)), dim3(256), lds, stream, a);
     if (hipGetLastError() != hipSuccess) return BW_ELAUNCH;
     if (p.splits > 1) {
-        hipLaunchKernelGGL((qdgrad_reduce_kernel<QM, DT, QK>), dim3(QM * QK / 4 / 256, (unsigned)p.tiles), dim3(256), 0, stream, a);
+        hipLaunchKernelGGL((qdgrad_reduce_kernel<QMv, DT, QK>), dim3(QMv * QK / 4 / 256, (unsigned)p.tiles), dim3(256), 0, stream, a);
         if (hipGetLastError() != hipSuccess) return BW_ELAUNCH;
     }
     return BW_OK;
 }
 
-// which kernel a call gets: the 256 x 256 one when the problem is large enough and, where its grid would leave CUs
-// idle, a workspace is on offer
-inline bool dgrad_use256(int64_t M, int64_t N, int64_t K, int64_t ldg, int bits, int group, bool have_workspace) {
-    if (!dgrad256_shape(M, N, K, ldg, bits, group)) return false;
-    const int64_t tiles = ((M + QM - 1) / QM) * (K / QK);
-    return have_workspace || tiles > dgrad_cus() / 2;
+// which kernel a call gets: the 256 x 256 one (with 256 or 128 rows of m) when the problem is large enough and, where its
+// grid would leave CUs idle, a workspace is on offer; 0 = the stepping kernel
+inline int dgrad_use256(int64_t M, int64_t N, int64_t K, int64_t ldg, int bits, int group, bool have_workspace) {
+    const int rows = dgrad256_rows(M, N, K, ldg, bits, group);
+    if (!rows) return 0;
+    const int64_t tiles = ((M + rows - 1) / rows) * (K / QK);
+    return (have_workspace || tiles > dgrad_cus() / 2) ? rows : 0;
 }
+
+#ifdef BW_TUNE
+static int g_dgrad_force = 0;                              // measurement builds: 1 = stepping kernel, 16 / 8 = the 256 x 256 kernel with 256 / 128 rows
+extern "C" void bw_tune_dgrad_kernel(int kind) { g_dgrad_force = kind; }
+#endif
 
 template <int BITS, int GROUP, int DT>
 int launch_dgrad(DgradArgs a, void* workspace, size_t workspace_bytes, hipStream_t stream) {
-    if (dgrad_use256(a.M, a.N, a.K, a.ldg, BITS, GROUP, workspace != nullptr))
-        return launch_dgrad256<BITS, GROUP, DT>(a, workspace, workspace_bytes, stream);
+#ifdef BW_TUNE
+    if (g_dgrad_force == 16) return launch_dgrad256<BITS, GROUP, DT, 16>(a, workspace, workspace_bytes, stream);
+    if (g_dgrad_force == 8) return launch_dgrad256<BITS, GROUP, DT, 8>(a, workspace, workspace_bytes, stream);
+    if (g_dgrad_force != 1)
+#endif
+    if (const int rows = dgrad_use256(a.M, a.N, a.K, a.ldg, BITS, GROUP, workspace != nullptr))
+        return rows == QM ? launch_dgrad256<BITS, GROUP, DT, 16>(a, workspace, workspace_bytes, stream)
+                          : launch_dgrad256<BITS, GROUP, DT, 8>(a, workspace, workspace_bytes, stream);
     const DgradPlan p = dgrad_plan(a.M, a.N, a.K, workspace != nullptr);
     if (p.ws_bytes > workspace_bytes) return BW_EWORKSPACE;
     a.ws = (float*)workspace;
@@ -706,16 +727,17 @@ extern "C" size_t bw_qdgrad_workspace_bytes(int64_t M, int64_t N, int64_t K, int
     if (!bw_shape_ok(N, K, bits, group) || !dgrad_fast_shape(M, N, K, N, K, bits, group)) return 0;
     // enough for either kernel (the call's own leading dimensions decide between them)
     const size_t a = dgrad_plan(M, N, K, true).ws_bytes;
-    const size_t b = dgrad256_shape(M, N, K, N, bits, group) ? dgrad256_plan(M, N, K, true).ws_bytes : 0;
+    const int rows = dgrad256_rows(M, N, K, N, bits, group);
+    const size_t b = rows ? dgrad256_plan(M, N, K, true, rows).ws_bytes : 0;
     return a > b ? a : b;
 }
 
 // Rows of grad_x a workgroup owns for this shape (with a workspace on offer): 128 or 256 for the kernel that walks N in
-// steps of 32 rows, 257 for the 256 x 256 kernel, 0 where the fused path does not apply.  A diagnostic, and what the
+// steps of 32 rows, 129 or 257 for the 256 x 256 kernel with 128 or 256 rows of m, 0 where the fused path does not apply.  A diagnostic, and what the
 // Python backward asks before it chooses between this kernel and dequantise + library GEMM.
 extern "C" int bw_qdgrad_tile_rows(int64_t M, int64_t N, int64_t K, int bits, int group) {
     if (!bw_shape_ok(N, K, bits, group) || !dgrad_fast_shape(M, N, K, N, K, bits, group)) return 0;
-    if (dgrad_use256(M, N, K, N, bits, group, true)) return 257;
+    if (const int rows = dgrad_use256(M, N, K, N, bits, group, true)) return rows + 1;
     return M > 512 ? 256 : 128;
 }
 

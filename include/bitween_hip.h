@@ -185,7 +185,8 @@ int bw_cast_bf16_f16(const void* x, int64_t rows, int64_t cols, int64_t ldx, voi
  * workspace == NULL runs unsliced.
  * Two kernels: one that owns 128 (256 beyond 512 rows) x 128 tiles of grad_x and walks N in steps of 32 rows, and - for
  * large problems with K % 256 == 0 and N % 64 == 0 - one with 256 x 256 tiles and steps of 64 rows;
- * bw_qdgrad_tile_rows tells which a shape gets (128, 256, 257 = the 256 x 256 kernel, 0 = no fused path): a diagnostic,
+ * bw_qdgrad_tile_rows tells which a shape gets (128, 256; 129, 257 = the 256 x 256 kernel with 128 (up to 512 rows of
+ * grad_y) or 256 rows of m per tile; 0 = no fused path): a diagnostic,
  * and what the Python backward asks before it prefers this entry point over dequantise + GEMM beyond 512 rows. */
 size_t bw_qdgrad_workspace_bytes(int64_t M, int64_t N, int64_t K, int bits, int group);
 

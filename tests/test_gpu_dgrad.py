@@ -236,17 +236,18 @@ def test_module_backward_takes_the_fused_kernel_for_bfloat16_gradients():
 @pytest.mark.parametrize("dtype", ["f16", "bf16"])
 @pytest.mark.parametrize("bits,g", COMBOS)
 def test_dgrad_256_tiles_vs_oracle(bits, g, dtype):
-    """Large problems run the 256 x 256 kernel (bw_qdgrad_tile_rows == 257): grad_y tile memory -> LDS by buffer loads,
-    the dequantised weight tile read transposed from LDS, steps of 64 rows of n.  Ragged M (1100 rows: five row tiles, the
-    last 76 rows high), rows of grad_y and grad_x padded, N sliced through the workspace (20 tiles on 256 CUs) and, where
+    """Large problems run the 256 x 256 kernel (bw_qdgrad_tile_rows == 257; 129 = its variant with 128 rows of m per tile,
+    up to 512 rows of grad_y): grad_y tile memory -> LDS by buffer loads, the dequantised weight tile read transposed from
+    LDS, steps of 64 rows of n.  Ragged M (1100 rows: five row tiles, the last 76 rows high; 300 rows: three 128-row tiles;
+    64 rows: half a tile), rows of grad_y and grad_x padded, N sliced through the workspace (20 tiles on 256 CUs) and, where
     the grid is large enough without one, unsliced; sampled rows against the oracle, one-hot rows return rows of the
     weight in the gradient's type bit for bit, the whole result against the library GEMM on the dequantised weight."""
     from bitween_amd.kernels import hip_loader
     lib = hip_loader.load()
     stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
     tdt, code = (torch.float16, 0) if dtype == "f16" else (torch.bfloat16, 1)
-    for (m, n, k) in ((1100, 64 * 154, 1024), (300, 64 * 800, 512), (256 * 160 + 9, 64 * 6, 1024)):
-        assert lib.bw_qdgrad_tile_rows(m, n, k, bits, g) == 257
+    for (m, n, k, plan) in ((1100, 64 * 154, 1024, 257), (300, 64 * 800, 512, 129), (256 * 160 + 9, 64 * 6, 1024, 257), (64, 64 * 640, 1024, 129)):
+        assert lib.bw_qdgrad_tile_rows(m, n, k, bits, g) == plan
         _, qw, s16, z16, _ = quantized_layer(n, k, bits, g, seed=n + k + bits + g + 5, outliers=True, bias=False)
         d = [to_gpu(a) for a in (qw, s16, z16)]
         wt = orc.dequantize_f16(qw, s16, z16, g, bits).astype(np.float32) if dtype == "f16" else orc.dequantize_bf16(qw, s16, z16, g, bits)
