@@ -24,6 +24,11 @@
 // two steps ahead; one barrier per step.  Three (two with the 256-row tile) workgroups share a CU and cover each
 // other's barriers.
 // Small M * K leaves the chip idle, so N is cut into slices whose float32 partial tiles a second kernel adds up.
+//
+// Two kernels share that scheme.  qdgrad_kernel (the "stepping" kernel, described above) serves small layers.  Large
+// problems run qdgrad256_kernel further down: 256 columns of k per tile and 256 or 128 rows of m, one wave per SIMD,
+// steps of 64 rows of n with the side work dealt out between the wave's own MFMAs - the forward kernel's natural-order
+// schedule turned around.  dgrad256_rows() holds the measured rule that picks between them.
 #include <hip/hip_runtime.h>
 
 #include "bw_common.h"
