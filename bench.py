@@ -768,8 +768,9 @@ def extras_board_probes(torch, hip, QuantizedLinear, layers):
 
 
 def extras_backward(torch, hip, QuantizedLinear, layers):
-    """grad_input of QuantizedLinearFunction.backward, 4096 -> 14336 W4 g128: the fused kernel (bw_qdgrad), the
-    path it replaces (HIP dequantise to float16 + library GEMM) and that GEMM alone on resident fp16 weights."""
+    """grad_input of QuantizedLinearFunction.backward, 4096 -> 14336 W4 g128: the fused kernel (bw_qdgrad; which of
+    its kernels a row count gets is `kernel_tile_rows`), the path it replaces (HIP dequantise to float16 + library GEMM)
+    and that GEMM alone on resident fp16 weights."""
     k, n = 4096, 14336
     q = make_layer(torch, QuantizedLinear, k, n, 4, 128, seed=11)
     w16 = hip.dequantize(q.qweight, q.scale, q.zero_point, 128, 4, torch.float16)
@@ -789,6 +790,8 @@ def extras_backward(torch, hip, QuantizedLinear, layers):
         t_deq = time_calls(torch, lambda: hip.dequantize(q.qweight, q.scale, q.zero_point, 128, 4, torch.float16), 30, 5)
         t_gemm = time_calls(torch, lambda: go @ w16, 30, 5)
         out["4096x14336_M%d" % m] = {"fused_dgrad_us": round(t_fused, 1), "fused_TFLOPs": round(2.0 * m * n * k / t_fused / 1e6, 1),
+                                     # 128 / 256: the kernel that walks N in steps of 32 rows; 129 / 257: the 256 x 256 kernel
+                                     "kernel_tile_rows": hip.load().bw_qdgrad_tile_rows(m, n, k, 4, 128),
                                      "dequantize_plus_gemm_us": round(t_ours, 1), "dequantize_us": round(t_deq, 1),
                                      "fp16_gemm_us": round(t_gemm, 1)}
         # bfloat16 gradients: the same kernel with the weight rounded to bfloat16 in registers, against the
